@@ -1,0 +1,279 @@
+"""Benchmark of the hot path on one MI355X.
+
+A step is one pass of the local multi-source reduction over one batch of staged chunks:
+reduce_scatter_tensor SUM, fp32, world size 8 seen from rank 0 -- eight staged 16 MiB chunks
+folded in rank order into one 16 MiB output (4,194,304 elements).  Inputs are resident in HBM
+before the timed region.  Prints one JSON line.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+INFINITY_CACHE_BYTES = 256 << 20
+
+
+def build_workload(name, torch, abi, dev):
+    """Returns (describe, algorithmic_bytes, nsets, launch(i), check()) for a named workload.
+    Every workload rotates over enough distinct buffer sets that their footprint exceeds twice
+    the 256 MB Infinity Cache, so no launch finds its operands cached by an earlier one."""
+    st = torch.cuda.current_stream().cuda_stream
+    L = abi.lib()
+
+    def nsets_for(set_bytes):
+        return max(2, -(-2 * INFINITY_CACHE_BYTES // set_bytes) + 1)
+
+    if name.startswith("reduce"):
+        # reduce_fp32_p8 (headline), reduce_bf16_p16, reduce_fp32_p64_{sum,avg,max}
+        spec = {
+            "reduce_fp32_p8": (8, 4194304, torch.float32, abi.DTYPE_FLOAT32, abi.OP_SUM, "randn", 1.0),
+            "reduce_bf16_p16": (16, 33554432, torch.bfloat16, abi.DTYPE_BFLOAT16, abi.OP_SUM, "randn1e-3", 1.0),
+            "reduce_fp32_p64_sum": (64, 1048576, torch.float32, abi.DTYPE_FLOAT32, abi.OP_SUM, "rand", 1.0),
+            "reduce_fp32_p64_avg": (64, 1048576, torch.float32, abi.DTYPE_FLOAT32, abi.OP_AVG, "rand", 1.0 / 64),
+            "reduce_fp32_p64_max": (64, 1048576, torch.float32, abi.DTYPE_FLOAT32, abi.OP_MAX, "rand", 1.0),
+        }[name]
+        P, N, tdt, code, op, dist, scale = spec
+        isz = torch.empty(0, dtype=tdt).element_size()
+        set_bytes = (P + 1) * N * isz
+        nsets = nsets_for(set_bytes)
+        base = []
+        for r in range(P):
+            torch.manual_seed(r)
+            if dist == "randn":
+                x = torch.randn(N)  # first N draws of rank r's 8*N-element input = its chunk for rank 0
+            elif dist == "randn1e-3":
+                x = (torch.randn(N) * 1e-3).to(tdt)
+            else:
+                x = torch.rand(N) * 2 - 1
+            base.append(x)
+        sets = [[b.to(dev) for b in base] for _ in range(nsets)]
+        outs = [torch.empty(N, dtype=tdt, device=dev) for _ in range(nsets)]
+        tabs = [abi.ptr_table([t.data_ptr() for t in s]) for s in sets]
+
+        def launch(i):
+            k = i % nsets
+            rc = L.mdh_reduce(tabs[k], P, 0, outs[k].data_ptr(), N, code, op, scale, st)
+            if rc:
+                abi.check(rc)
+
+        def check():
+            import numpy as np
+
+            import oracle
+
+            def b(t):
+                t = t.cpu()
+                return t.view(torch.int16).numpy().view(np.uint16) if isz == 2 else t.numpy()
+
+            want = oracle.reduce([b(x) for x in base], 0, code, op, scale)
+            for o in outs:
+                if not np.array_equal(b(o).view(np.uint8), want.view(np.uint8)):
+                    raise SystemExit("bench: result differs from the oracle")
+
+        desc = {"workload": name, "op": "reduce_scatter_tensor local reduction", "sources": P, "numel": N,
+                "dtype": str(tdt).replace("torch.", ""), "fold_first": 0, "buffer_sets": nsets}
+        return desc, set_bytes, launch, check, "reduce_vec_kernel"
+
+    if name == "allgather_bf16_p8" or name == "allgather_bf16_p8_strided":
+        P, n = 8, 16777216
+        rows = cols = 4096
+        pad = 64 if name.endswith("strided") else 0
+        set_bytes = 2 * P * n * 2
+        nsets = nsets_for(set_bytes)
+        base = []
+        for r in range(P):
+            torch.manual_seed(r)
+            base.append(torch.randn(n).bfloat16())
+        sets = [[b.to(dev) for b in base] for _ in range(nsets)]
+        outs = [torch.empty(P, rows, cols + pad, dtype=torch.bfloat16, device=dev) for _ in range(nsets)]
+        tabs = [abi.ptr_table([t.data_ptr() for t in s]) for s in sets]
+
+        def launch(i):
+            k = i % nsets
+            if pad:
+                rc = L.mdh_gather(tabs[k], P, outs[k].data_ptr(), cols * 2, rows, cols * 2, (cols + pad) * 2,
+                                  rows * (cols + pad) * 2, st)
+            else:
+                rc = L.mdh_gather(tabs[k], P, outs[k].data_ptr(), n * 2, 1, n * 2, n * 2, n * 2, st)
+            if rc:
+                abi.check(rc)
+
+        def check():
+            want = torch.stack(base).view(P, rows, cols)
+            for o in outs:
+                if not torch.equal(o[:, :, :cols].cpu(), want):
+                    raise SystemExit("bench: result differs from the expected gather")
+
+        desc = {"workload": name, "op": "all_gather_into_tensor chunk assembly", "sources": P, "numel": n,
+                "dtype": "bfloat16", "buffer_sets": nsets}
+        return desc, set_bytes, launch, check, "copy_boxes_kernel"
+
+    if name.startswith("redistribute"):
+        # redistribute_fp32_8192, redistribute_bf16_8192, redistribute_bf16_3d
+        P = 8
+        if name.endswith("3d"):
+            tdt, shape, box = torch.bfloat16, (64, 512, 1024), [8, 512, 128]
+            sstr, dstr = [512 * 1024, 1024, 1], [512 * 128, 128, 1]
+            out_shape = (64, 512, 128)
+        else:
+            tdt = torch.float32 if "fp32" in name else torch.bfloat16
+            shape, box = (8192, 8192), [1024, 1024]
+            sstr, dstr = [8192, 1], [1024, 1]
+            out_shape = (8192, 1024)
+        isz = torch.empty(0, dtype=tdt).element_size()
+        torch.manual_seed(0)
+        G = torch.randn(*shape).to(tdt)
+        per = shape[0] // P
+        out_numel = 1
+        for s in out_shape:
+            out_numel *= s
+        set_bytes = 2 * out_numel * isz
+        # the slabs are read only in part (this rank's columns), yet all of them must leave the cache
+        nsets = nsets_for(G.numel() * isz)
+        k = 0  # this rank
+        sets = [[G[per * s:per * (s + 1)].contiguous().to(dev) for s in range(P)] for _ in range(nsets)]
+        outs = [torch.empty(out_shape, dtype=tdt, device=dev) for _ in range(nsets)]
+        blk = out_numel // P
+        tabs = []
+        for i in range(nsets):
+            boxes = [abi.make_box(sets[i][s].data_ptr() + box[-1] * k * isz, outs[i].data_ptr() + s * blk * isz, box,
+                                  sstr, dstr) for s in range(P)]
+            tabs.append((abi.Box * P)(*boxes))
+
+        def launch(i):
+            rc = L.mdh_copy_boxes(tabs[i % nsets], P, isz, st)
+            if rc:
+                abi.check(rc)
+
+        def check():
+            want = G[..., box[-1] * k:box[-1] * (k + 1)]
+            for o in outs:
+                if not torch.equal(o.cpu(), want):
+                    raise SystemExit("bench: result differs from the expected redistribution")
+
+        desc = {"workload": name, "op": "compile_op redistribution copies", "sources": P,
+                "global_shape": list(shape), "dtype": str(tdt).replace("torch.", ""), "buffer_sets": nsets}
+        return desc, set_bytes, launch, check, "copy_boxes_kernel"
+
+    raise SystemExit("bench: unknown workload %r" % name)
+
+
+def cpu_baseline(seconds_budget=12.0):
+    """The reference's CPU reduce-scatter, restated in oracle.c, timed on this host: eight
+    rank-threads (one service thread per rank process in the reference), each folding its chunk of
+    all eight inputs with the memcpy + scalar-loop passes of the reference."""
+    import numpy as np
+
+    import oracle
+
+    P, N = 8, 4194304
+    threads = min(P, os.cpu_count() or 1)
+    rng = np.random.RandomState(0)
+    inputs = [rng.standard_normal(P * N).astype(np.float32) for _ in range(P)]
+    outputs = [np.empty(N, dtype=np.float32) for _ in range(P)]
+    alg_bytes = threads * (P + 1) * N * 4
+    oracle.cpu_reduce_scatter_seconds(inputs, outputs, threads, N, oracle.DT_F32, reps=1)  # warm-up, page faults
+    best = None
+    reps = 0
+    t_end = time.time() + seconds_budget
+    while time.time() < t_end and reps < 200:
+        t = oracle.cpu_reduce_scatter_seconds(inputs, outputs, threads, N, oracle.DT_F32, reps=3)
+        best = t if best is None or t < best else best
+        reps += 3
+    single = oracle.cpu_reduce_scatter_seconds(inputs, outputs, 1, N, oracle.DT_F32, reps=3)
+    want = oracle.reduce([x[:N] for x in inputs], 0, oracle.DT_F32, oracle.OP_SUM)
+    assert np.array_equal(outputs[0], want)
+    return {
+        "value": round(alg_bytes / best / 1e9, 2),
+        "unit": "GB/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": "full workload (8 ranks x 8 chunks of 4,194,304 fp32), %d rank-threads at once, best of %d "
+                  "repetitions; one rank-thread alone: %.2f GB/s" % (threads, reps, (P + 1) * N * 4 / single / 1e9),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--workload", default="reduce_fp32_p8")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-check", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        raise SystemExit("bench.py measures one GPU: the path is one rank's share with its peers staged in the "
+                         "same GPU's HBM; run it with --gpus 1")
+
+    import torch
+
+    from moodist_amd import _abi as abi
+
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    desc, alg_bytes, launch, check, kernel = build_workload(args.workload, torch, abi, dev)
+
+    for i in range(args.warmup):
+        launch(i)
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()  # on torch's current stream, the stream every launch above and below uses
+    for i in range(args.steps):
+        launch(i)
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms = e0.elapsed_time(e1)
+    ms_per_step = ms / args.steps
+    if not args.no_check:
+        check()
+    gbs = alg_bytes / (ms_per_step * 1e-3) / 1e9
+    out = {
+        "metric": "achieved HBM GB/s (% of peak) for 1-GPU local reduce-scatter, fp32 P=8"
+        if args.workload == "reduce_fp32_p8" else "achieved HBM GB/s (% of peak), " + args.workload,
+        "value": round(gbs, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": {"float32": "f32", "bfloat16": "bf16"}[desc["dtype"]],
+        "data": "synthetic",
+        "config": desc,
+        "percent_of_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),
+        "host_wall_ms_per_step": round(wall_ms / args.steps, 6),
+        "roofline": {
+            "bound": "hbm",
+            "kernel": kernel,
+            "achieved": round(gbs, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(gbs / HBM_PEAK_GBS, 4),
+            "algorithmic_bytes_per_launch": alg_bytes,
+            "traffic": None,
+        },
+    }
+    if not args.no_cpu_baseline and args.workload == "reduce_fp32_p8":
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

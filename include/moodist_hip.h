@@ -1,0 +1,161 @@
+/*
+ * moodist_hip.h -- thin C ABI between the C++ host side and the hand-written
+ * HIP kernels for gfx950 (MI355X).
+ *
+ * The reference has no such seam: its host code launches run-time generated
+ * kernels directly with cuLaunchKernel (core/processgroup.cc:1240-1242 for
+ * allgather_local, :1651-1657 for reduce_scatter_local, :1556-1557 for
+ * reduce_scatter_direct) after filling AllGatherParameters /
+ * ReduceScatterParameters (core/allgather.h:14-24, core/reduce_scatter.h:14-26).
+ * Each entry point below replaces one of those launches (named per function)
+ * and takes the same facts as plain pointers and sizes.
+ *
+ * Contract shared by every launch function:
+ *   - returns 0 on success, an MDH_E* code otherwise (never throws, never
+ *     aborts); mdh_error_string() names a code, mdh_last_error() holds detail
+ *     for the calling thread;
+ *   - allocates nothing, frees nothing, never synchronises: work is enqueued
+ *     on `stream` (a hipStream_t; NULL is the default stream) and the caller
+ *     owns every buffer until that work has finished;
+ *   - all data pointers are device pointers on the current device; pointer
+ *     TABLES (srcs, boxes) are host memory and are consumed before return;
+ *   - dtype codes are torch ScalarType numbers and op codes are c10d RedOpType
+ *     numbers, the same numbers the reference's API carries
+ *     (api/moodist_api.h:30-55).
+ */
+#ifndef MOODIST_HIP_H
+#define MOODIST_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MDH_ABI_VERSION 1
+
+/* error codes */
+#define MDH_OK 0
+#define MDH_EINVAL 1      /* bad argument (null pointer, count or size out of range) */
+#define MDH_EDTYPE 2      /* "Unsupported dtype for reduce operation" (core/processgroup.cc:277) */
+#define MDH_EOP 3         /* "Unsupported reduce operation" (core/processgroup.cc:294) */
+#define MDH_ELAUNCH 4     /* the HIP runtime refused the launch; see mdh_last_error() */
+#define MDH_ENODEVICE 5   /* no usable gfx950 device */
+
+/* api/moodist_api.h:30-42 */
+#define MDH_DTYPE_INT32 3
+#define MDH_DTYPE_INT64 4
+#define MDH_DTYPE_FLOAT16 5
+#define MDH_DTYPE_FLOAT32 6
+#define MDH_DTYPE_FLOAT64 7
+#define MDH_DTYPE_BFLOAT16 15
+
+/* api/moodist_api.h:45-55 */
+#define MDH_OP_SUM 0
+#define MDH_OP_AVG 1
+#define MDH_OP_MIN 3
+#define MDH_OP_MAX 4
+#define MDH_OP_PREMUL_SUM 8
+
+#define MDH_MAX_SOURCES 64 /* the reference stops at 8 peer slots (core/reduce_scatter.h:22-23) */
+#define MDH_MAX_DIMS 10    /* compile_op accepts up to 10 dimensions (core/processgroup.cc:3110-3141) */
+
+int mdh_abi_version(void);
+const char* mdh_error_string(int code);
+const char* mdh_last_error(void);
+
+/*
+ * Local multi-source reduction: dst[i] = srcs[first][i] (+) srcs[first+1][i]
+ * (+) ... wrapping round to srcs[first-1][i], a left fold in exactly that
+ * order, in one pass over memory.
+ *
+ * Replaces: the reduce_scatter_local kernel launch (core/processgroup.cc:1651-1653;
+ * fold built by core/reduce_scatter.cc:104-142, :180-191 as K-1 two-source
+ * passes), the per-destination reduction of reduce_scatter_direct
+ * (core/reduce_scatter_direct.cc:165-177) and the final sum_out/amax_out/amin_out
+ * over K rows (core/processgroup.cc:1599-1616).  `first` expresses the
+ * reference's peer order: own chunk, then ranks rank+1..P-1, 0..rank-1
+ * (core/group.cc:567-570).
+ *
+ * srcs[j] points at source j's chunk (the caller has already added
+ * pitch*rank); dst may equal srcs[first] exactly (allreduce reduces in place,
+ * core/processgroup.cc:1689-1692) but must not otherwise overlap a source.
+ *
+ * op / scale:
+ *   SUM, MIN, MAX  scale ignored.  MIN/MAX follow std::min/std::max on
+ *                  (running value, next source): ties and NaN keep the
+ *                  running value (core/cputhread.cc:131-143).
+ *   AVG            SUM, then one multiply by `scale` with its own rounding
+ *                  (the caller passes 1.0f/size; core/processgroup.cc:1664-1667).
+ *   PREMUL_SUM     each source times `scale` with its own rounding, then SUM
+ *                  (core/processgroup.cc:1374-1378).
+ *   AVG and PREMUL_SUM need a floating dtype.
+ * float32/float64: IEEE adds in fold order, bit-exact.  int32/int64: wrapping
+ * adds, signed min/max.  bfloat16/float16: sources widened to fp32, folded in
+ * fp32, rounded to nearest even once.
+ *
+ * Pointers and sizes may have any alignment; the 16-byte path is taken when
+ * every pointer is 16-byte aligned.  numel == 0 is a no-op.
+ */
+int mdh_reduce(const void* const* srcs, int nsrc, int first, void* dst, size_t numel, int dtype, int op,
+    float scale, void* stream);
+
+/*
+ * All-gather chunk assembly: for every shard s < nsrc and row r < rows,
+ * copy `width` bytes from srcs[s] + r*src_pitch to
+ * dst + s*dst_shard_stride + r*dst_pitch.
+ *
+ * Replaces: the allgather_local kernel launch (core/processgroup.cc:1240-1242;
+ * P sequential copy_impl calls, core/allgather.cc:381-390) with rows = 1,
+ * width = bytes, dst_shard_stride = pitch; and the copy-engine form
+ * (Copy2d + cuMemcpy2DAsync, core/processgroup.cc:806-820) and the padded
+ * staging copies (:1130-1136, :1273-1283) with rows > 1.
+ *
+ * srcs[s] == dst + s*dst_shard_stride is allowed (a shard already in place is
+ * skipped); other overlap is not.  Any alignment; width == 0 or rows == 0 is a
+ * no-op.
+ */
+int mdh_gather(const void* const* srcs, int nsrc, void* dst, size_t width, size_t rows, size_t src_pitch,
+    size_t dst_pitch, size_t dst_shard_stride, void* stream);
+
+/*
+ * One N-d box to move: shape[d] elements along dimension d, element strides on
+ * each side.  src/dst point at the box's first element (offset already added).
+ */
+typedef struct mdh_box {
+  const void* src;
+  void* dst;
+  int32_t ndim; /* 0..MDH_MAX_DIMS */
+  int32_t reserved;
+  int64_t shape[MDH_MAX_DIMS];
+  int64_t src_strides[MDH_MAX_DIMS]; /* in elements, >= 0 */
+  int64_t dst_strides[MDH_MAX_DIMS]; /* in elements, >= 0 */
+} mdh_box;
+
+/*
+ * Shard redistribution: copy every box, strided on either side, in as few
+ * launches as the table allows (boxes are fused into one grid).
+ *
+ * Replaces: the execution of a compiled custom op -- each Read is a byte-exact
+ * move (core/cputhread.cc:5628-5672) and each Copy an {offset, shape} box of a
+ * tensor to or from contiguous staging (core/cputhread.h:306-310).  A box with
+ * both sides strided is the fused form Copy -> Read -> Copy, so no staging
+ * buffer exists.  Destination boxes must not overlap each other or any source.
+ */
+int mdh_copy_boxes(const mdh_box* boxes, int nboxes, int itemsize, void* stream);
+
+/*
+ * Launch-shape knobs, for measurement.  Names: "reduce_unroll" (1,2,4),
+ * "reduce_max_blocks" (0 = one tile per workgroup), "copy_unroll" (1,2,4,8),
+ * "copy_max_blocks".  Returns MDH_EINVAL for an unknown name or value.
+ * No counterpart in the reference, whose grid is fixed at 4/16/64 blocks
+ * (core/kernels.cc:547-556).
+ */
+int mdh_set_tuning(const char* name, int value);
+int mdh_get_tuning(const char* name, int* value);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOODIST_HIP_H */

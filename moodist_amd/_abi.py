@@ -1,0 +1,121 @@
+"""ctypes binding of the thin C ABI (include/moodist_hip.h) of libmoodist_hip.so.
+
+The library holds the hand-written gfx950 kernels.  There is no fallback: if
+it is missing, loading raises, and every call that fails raises MoodistError
+with the library's own message.
+"""
+
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmoodist_hip.so")
+
+# torch ScalarType / c10d RedOpType numbers (include/moodist_hip.h)
+DTYPE_INT32, DTYPE_INT64, DTYPE_FLOAT16, DTYPE_FLOAT32, DTYPE_FLOAT64, DTYPE_BFLOAT16 = 3, 4, 5, 6, 7, 15
+OP_SUM, OP_AVG, OP_MIN, OP_MAX, OP_PREMUL_SUM = 0, 1, 3, 4, 8
+MAX_SOURCES = 64
+MAX_DIMS = 10
+ABI_VERSION = 1
+
+SYMBOLS = (
+    "mdh_abi_version", "mdh_error_string", "mdh_last_error", "mdh_reduce", "mdh_gather", "mdh_copy_boxes",
+    "mdh_set_tuning", "mdh_get_tuning",
+)
+
+
+class MoodistError(RuntimeError):
+    pass
+
+
+class Box(ctypes.Structure):
+    _fields_ = [
+        ("src", ctypes.c_void_p),
+        ("dst", ctypes.c_void_p),
+        ("ndim", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
+        ("shape", ctypes.c_int64 * MAX_DIMS),
+        ("src_strides", ctypes.c_int64 * MAX_DIMS),
+        ("dst_strides", ctypes.c_int64 * MAX_DIMS),
+    ]
+
+
+_lib = None
+
+
+def lib():
+    """Load libmoodist_hip.so (once). Raises MoodistError if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise MoodistError(
+            "libmoodist_hip.so is not built (%s); run `python -c 'import __graft_entry__ as g; g.build()'` "
+            "or moodist_amd/csrc/build.sh" % LIB_PATH)
+    L = ctypes.CDLL(LIB_PATH)
+    vpp = ctypes.POINTER(ctypes.c_void_p)
+    L.mdh_abi_version.restype = ctypes.c_int
+    L.mdh_error_string.argtypes = [ctypes.c_int]
+    L.mdh_error_string.restype = ctypes.c_char_p
+    L.mdh_last_error.restype = ctypes.c_char_p
+    L.mdh_reduce.argtypes = [vpp, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int,
+                             ctypes.c_int, ctypes.c_float, ctypes.c_void_p]
+    L.mdh_reduce.restype = ctypes.c_int
+    L.mdh_gather.argtypes = [vpp, ctypes.c_int, ctypes.c_void_p] + [ctypes.c_size_t] * 5 + [ctypes.c_void_p]
+    L.mdh_gather.restype = ctypes.c_int
+    L.mdh_copy_boxes.argtypes = [ctypes.POINTER(Box), ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    L.mdh_copy_boxes.restype = ctypes.c_int
+    L.mdh_set_tuning.argtypes = [ctypes.c_char_p, ctypes.c_int]
+    L.mdh_set_tuning.restype = ctypes.c_int
+    L.mdh_get_tuning.argtypes = [ctypes.c_char_p, ctypes.POINTER(ctypes.c_int)]
+    L.mdh_get_tuning.restype = ctypes.c_int
+    if L.mdh_abi_version() != ABI_VERSION:
+        raise MoodistError("libmoodist_hip.so has ABI version %d, expected %d" % (L.mdh_abi_version(), ABI_VERSION))
+    _lib = L
+    return L
+
+
+def check(rc):
+    if rc != 0:
+        L = lib()
+        detail = L.mdh_last_error().decode()
+        raise MoodistError(detail or L.mdh_error_string(rc).decode())
+
+
+def ptr_table(ptrs):
+    tab = (ctypes.c_void_p * max(len(ptrs), 1))()
+    for i, p in enumerate(ptrs):
+        tab[i] = p
+    return tab
+
+
+def reduce(src_ptrs, first, dst_ptr, numel, dtype, op, scale=1.0, stream=0):
+    check(lib().mdh_reduce(ptr_table(src_ptrs), len(src_ptrs), first, dst_ptr, numel, dtype, op, scale, stream))
+
+
+def gather(src_ptrs, dst_ptr, width, rows, src_pitch, dst_pitch, dst_shard_stride, stream=0):
+    check(lib().mdh_gather(ptr_table(src_ptrs), len(src_ptrs), dst_ptr, width, rows, src_pitch, dst_pitch,
+                           dst_shard_stride, stream))
+
+
+def make_box(src_ptr, dst_ptr, shape, src_strides, dst_strides):
+    b = Box()
+    b.src, b.dst, b.ndim = src_ptr, dst_ptr, len(shape)
+    for d in range(len(shape)):
+        b.shape[d], b.src_strides[d], b.dst_strides[d] = shape[d], src_strides[d], dst_strides[d]
+    return b
+
+
+def copy_boxes(boxes, itemsize, stream=0):
+    arr = (Box * max(len(boxes), 1))(*boxes)
+    check(lib().mdh_copy_boxes(arr, len(boxes), itemsize, stream))
+
+
+def set_tuning(name, value):
+    check(lib().mdh_set_tuning(name.encode(), value))
+
+
+def get_tuning(name):
+    v = ctypes.c_int()
+    check(lib().mdh_get_tuning(name.encode(), ctypes.byref(v)))
+    return v.value

@@ -1,0 +1,113 @@
+// Error reporting, launch checking and tuning knobs shared by the C ABI.
+#include "device_common.h"
+
+#include <cstring>
+
+namespace mdh {
+
+namespace {
+thread_local char g_error[512] = "";
+}
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+
+int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    set_error("%s: launch failed: %s", what, hipGetErrorString(e));
+    return MDH_ELAUNCH;
+  }
+  return MDH_OK;
+}
+
+Tuning& tuning() {
+  static Tuning t;
+  return t;
+}
+
+} // namespace mdh
+
+extern "C" int mdh_abi_version(void) {
+  return MDH_ABI_VERSION;
+}
+
+extern "C" const char* mdh_last_error(void) {
+  return mdh::g_error;
+}
+
+extern "C" const char* mdh_error_string(int code) {
+  switch (code) {
+  case MDH_OK:
+    return "success";
+  case MDH_EINVAL:
+    return "invalid argument";
+  case MDH_EDTYPE:
+    return "Unsupported dtype for reduce operation";
+  case MDH_EOP:
+    return "Unsupported reduce operation";
+  case MDH_ELAUNCH:
+    return "kernel launch failed";
+  case MDH_ENODEVICE:
+    return "no usable gfx950 device";
+  default:
+    return "unknown error";
+  }
+}
+
+namespace {
+int* knob(const char* name) {
+  mdh::Tuning& t = mdh::tuning();
+  if (!name) {
+    return nullptr;
+  }
+  if (!std::strcmp(name, "reduce_unroll")) {
+    return &t.reduce_unroll;
+  }
+  if (!std::strcmp(name, "reduce_max_blocks")) {
+    return &t.reduce_max_blocks;
+  }
+  if (!std::strcmp(name, "copy_unroll")) {
+    return &t.copy_unroll;
+  }
+  if (!std::strcmp(name, "copy_max_blocks")) {
+    return &t.copy_max_blocks;
+  }
+  return nullptr;
+}
+} // namespace
+
+extern "C" int mdh_set_tuning(const char* name, int value) {
+  int* k = knob(name);
+  if (!k) {
+    mdh::set_error("mdh_set_tuning: unknown knob");
+    return MDH_EINVAL;
+  }
+  const bool unroll = std::strstr(name, "unroll") != nullptr;
+  const bool reduce = std::strstr(name, "reduce") != nullptr;
+  if (unroll) {
+    if (!(value == 1 || value == 2 || value == 4 || (!reduce && value == 8))) {
+      mdh::set_error("mdh_set_tuning: %s does not take %d", name, value);
+      return MDH_EINVAL;
+    }
+  } else if (value < 0) {
+    mdh::set_error("mdh_set_tuning: %s does not take %d", name, value);
+    return MDH_EINVAL;
+  }
+  *k = value;
+  return MDH_OK;
+}
+
+extern "C" int mdh_get_tuning(const char* name, int* value) {
+  int* k = knob(name);
+  if (!k || !value) {
+    mdh::set_error("mdh_get_tuning: unknown knob");
+    return MDH_EINVAL;
+  }
+  *value = *k;
+  return MDH_OK;
+}

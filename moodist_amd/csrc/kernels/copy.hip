@@ -1,0 +1,504 @@
+// Streaming copies for gfx950: all-gather chunk assembly and the N-d box
+// copies of a shard redistribution, fused into one grid per launch.
+//
+// Where the reference runs P sequential copy_impl calls on at most 64 blocks
+// (core/allgather.cc:381-390, core/kernels.cc:28-169) or hands 2-D shapes to
+// the copy engine (core/processgroup.cc:806-820), this kernel takes a table of
+// up to 32 boxes in its kernel arguments and spreads their tiles over the
+// whole chip.  Every box is reduced on the host to
+//     rows x cols vectors,  rows decomposed over <= 3 strided outer extents,
+// and a tile is kBlock*U vector slots shaped 2^a rows x 2^b columns, so the
+// lane -> (row, column) mapping is shifts and masks; an integer division is
+// paid once per tile, never per vector.  Runs shorter than a wave's 1 KiB still
+// coalesce: consecutive lanes walk a run, then step to the next row.
+#include "device_common.h"
+
+#include <algorithm>
+#include <vector>
+
+namespace mdh {
+namespace {
+
+constexpr int kMaxBoxes = 32;
+constexpr int kMaxOuter = 3;
+
+struct BoxDesc {
+  const char* src;
+  char* dst;
+  int64_t src_stride[kMaxOuter]; // bytes; [0] is the fastest-varying outer extent
+  int64_t dst_stride[kMaxOuter];
+  uint32_t outer[kMaxOuter];
+  uint32_t nouter;
+  uint32_t rows; // product of outer[]
+  uint32_t cols; // vectors per row
+  uint32_t nct;  // column tiles per row of tiles
+  uint32_t log2tc;
+};
+
+struct CopyArgs {
+  BoxDesc box[kMaxBoxes];
+  uint32_t tile_end[kMaxBoxes]; // tiles of boxes 0..k, cumulative; unused entries are ~0
+  uint32_t nboxes;
+  uint32_t total_tiles;
+};
+static_assert(sizeof(CopyArgs) <= 4096, "kernel arguments are limited to 4 KiB");
+
+template<int VEC>
+struct VecType;
+template<>
+struct VecType<16> {
+  using type = u32x4;
+};
+template<>
+struct VecType<8> {
+  using type = u32x2;
+};
+template<>
+struct VecType<4> {
+  using type = uint32_t;
+};
+template<>
+struct VecType<2> {
+  using type = uint16_t;
+};
+template<>
+struct VecType<1> {
+  using type = uint8_t;
+};
+
+constexpr uint32_t ilog2(uint32_t x) {
+  return x <= 1 ? 0 : 1 + ilog2(x >> 1);
+}
+
+template<int VEC, int U>
+__global__ __launch_bounds__(kBlock) void copy_boxes_kernel(CopyArgs a) {
+  using V = typename VecType<VEC>::type;
+  constexpr uint32_t log2slots = ilog2(kBlock * U);
+  for (uint32_t tile = blockIdx.x; tile < a.total_tiles; tile += gridDim.x) {
+    // which box: count the cumulative ends at or below this tile (all scalar,
+    // the table sits in the kernel arguments)
+    uint32_t b = 0, start = 0;
+#pragma unroll
+    for (int k = 0; k < kMaxBoxes - 1; ++k) {
+      const uint32_t e = a.tile_end[k];
+      if (tile >= e) {
+        ++b;
+        start = e;
+      }
+    }
+    const BoxDesc& B = a.box[b];
+    const uint32_t local = tile - start;
+    const uint32_t rt = local / B.nct;
+    const uint32_t ct = local - rt * B.nct;
+    const uint32_t log2tc = B.log2tc;
+    const uint32_t log2tr = log2slots - log2tc;
+    const uint32_t tcmask = (1u << log2tc) - 1u;
+    V v[U];
+    bool ok[U];
+    int64_t doff[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t slot = (uint32_t)u * kBlock + threadIdx.x;
+      const uint32_t col = (ct << log2tc) + (slot & tcmask);
+      uint32_t row = (rt << log2tr) + (slot >> log2tc);
+      ok[u] = col < B.cols && row < B.rows;
+      int64_t so, dof;
+      if (B.nouter <= 1) {
+        so = (int64_t)row * B.src_stride[0];
+        dof = (int64_t)row * B.dst_stride[0];
+      } else {
+        so = 0, dof = 0;
+        for (uint32_t k = 0; k + 1 < B.nouter; ++k) {
+          const uint32_t q = row / B.outer[k];
+          const uint32_t i = row - q * B.outer[k];
+          so += (int64_t)i * B.src_stride[k];
+          dof += (int64_t)i * B.dst_stride[k];
+          row = q;
+        }
+        so += (int64_t)row * B.src_stride[B.nouter - 1];
+        dof += (int64_t)row * B.dst_stride[B.nouter - 1];
+      }
+      so += (int64_t)col * VEC;
+      doff[u] = dof + (int64_t)col * VEC;
+      if (ok[u]) {
+        v[u] = stream_load((const V*)(B.src + so));
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (ok[u]) {
+        stream_store((V*)(B.dst + doff[u]), v[u]);
+      }
+    }
+  }
+}
+
+// ---- host side: reduce a box to the kernel's form ----
+
+struct HostBox {
+  const char* src;
+  char* dst;
+  int nd; // strided extents, slowest first; the contiguous run is separate
+  int64_t shape[MDH_MAX_DIMS + 1];
+  int64_t sstride[MDH_MAX_DIMS + 1]; // bytes
+  int64_t dstride[MDH_MAX_DIMS + 1];
+  int64_t run; // contiguous bytes per row
+};
+
+int vec_width(const HostBox& h) {
+  uint64_t bits = (uint64_t)(uintptr_t)h.src | (uint64_t)(uintptr_t)h.dst | (uint64_t)h.run | 16u;
+  for (int d = 0; d < h.nd; ++d) {
+    bits |= (uint64_t)h.sstride[d] | (uint64_t)h.dstride[d];
+  }
+  return (int)(bits & (~bits + 1)); // lowest set bit: 1, 2, 4, 8 or 16
+}
+
+struct Launcher {
+  hipStream_t stream;
+  std::vector<BoxDesc> pending[5]; // by log2(VEC)
+  int rc = MDH_OK;
+
+  template<int VEC>
+  void launch(CopyArgs& a) {
+    const Tuning& t = tuning();
+    uint32_t grid = a.total_tiles;
+    if (t.copy_max_blocks > 0 && grid > (uint32_t)t.copy_max_blocks) {
+      grid = (uint32_t)t.copy_max_blocks;
+    }
+    if (grid > 0x7fffffffu) {
+      grid = 0x7fffffffu;
+    }
+    dim3 g(grid), b(kBlock);
+    switch (t.copy_unroll) {
+    case 1:
+      hipLaunchKernelGGL((copy_boxes_kernel<VEC, 1>), g, b, 0, stream, a);
+      break;
+    case 2:
+      hipLaunchKernelGGL((copy_boxes_kernel<VEC, 2>), g, b, 0, stream, a);
+      break;
+    case 4:
+      hipLaunchKernelGGL((copy_boxes_kernel<VEC, 4>), g, b, 0, stream, a);
+      break;
+    default:
+      hipLaunchKernelGGL((copy_boxes_kernel<VEC, 8>), g, b, 0, stream, a);
+      break;
+    }
+    int r = check_launch("copy_boxes_kernel");
+    if (r != MDH_OK) {
+      rc = r;
+    }
+  }
+
+  void flush_class(int lg) {
+    auto& list = pending[lg];
+    const int U = tuning().copy_unroll;
+    const uint32_t slots = (uint32_t)kBlock * (uint32_t)U;
+    size_t i = 0;
+    while (i < list.size()) {
+      CopyArgs a;
+      a.nboxes = 0;
+      uint64_t tiles = 0;
+      while (i < list.size() && a.nboxes < (uint32_t)kMaxBoxes) {
+        BoxDesc d = list[i];
+        uint32_t tc = 1, log2tc = 0;
+        while (tc < d.cols && tc < slots) {
+          tc <<= 1, ++log2tc;
+        }
+        const uint32_t tr = slots >> log2tc;
+        d.log2tc = log2tc;
+        d.nct = (d.cols + tc - 1) / tc;
+        const uint64_t n = (uint64_t)d.nct * ((d.rows + tr - 1) / tr);
+        if (tiles + n > 0x7fffffffull) {
+          if (a.nboxes == 0) {
+            set_error("copy: one box needs %llu tiles, more than a grid can index", (unsigned long long)n);
+            rc = MDH_EINVAL;
+            return;
+          }
+          break;
+        }
+        tiles += n;
+        a.tile_end[a.nboxes] = (uint32_t)tiles;
+        a.box[a.nboxes++] = d;
+        ++i;
+      }
+      for (uint32_t k = a.nboxes; k < (uint32_t)kMaxBoxes; ++k) {
+        a.tile_end[k] = 0xffffffffu;
+      }
+      a.total_tiles = (uint32_t)tiles;
+      if (tiles == 0) {
+        continue;
+      }
+      switch (lg) {
+      case 4:
+        launch<16>(a);
+        break;
+      case 3:
+        launch<8>(a);
+        break;
+      case 2:
+        launch<4>(a);
+        break;
+      case 1:
+        launch<2>(a);
+        break;
+      default:
+        launch<1>(a);
+        break;
+      }
+    }
+    list.clear();
+  }
+
+  void flush() {
+    for (int lg = 4; lg >= 0; --lg) {
+      flush_class(lg);
+    }
+  }
+
+  // rows x run with <= kMaxOuter strided extents
+  void emit(const HostBox& h) {
+    const int vec = vec_width(h);
+    int lg = 0;
+    while ((1 << lg) < vec) {
+      ++lg;
+    }
+    BoxDesc d;
+    d.src = h.src;
+    d.dst = h.dst;
+    d.nouter = h.nd > 0 ? (uint32_t)h.nd : 1u;
+    uint64_t rows = 1;
+    for (int k = 0; k < kMaxOuter; ++k) {
+      d.outer[k] = 1;
+      d.src_stride[k] = 0;
+      d.dst_stride[k] = 0;
+    }
+    for (int k = 0; k < h.nd; ++k) {
+      const int dim = h.nd - 1 - k; // fastest first
+      d.outer[k] = (uint32_t)h.shape[dim];
+      d.src_stride[k] = h.sstride[dim];
+      d.dst_stride[k] = h.dstride[dim];
+      rows *= (uint64_t)h.shape[dim];
+    }
+    d.rows = (uint32_t)rows;
+    d.cols = (uint32_t)(h.run / vec);
+    d.nct = d.log2tc = 0;
+    pending[lg].push_back(d);
+  }
+
+  // Splits what the kernel's 32-bit extents or kMaxOuter cannot hold.
+  void add(HostBox h) {
+    if (rc != MDH_OK) {
+      return;
+    }
+    if (h.nd == 0) {
+      // one contiguous run: peel an unaligned head and tail so the body moves
+      // 16 bytes per lane, and cut runs too long for 32-bit column counts
+      const uintptr_t s = (uintptr_t)h.src, d = (uintptr_t)h.dst;
+      if (h.run >= 64 && (s & 15) == (d & 15)) {
+        const int64_t head = (int64_t)((16 - (s & 15)) & 15);
+        const int64_t body = (h.run - head) & ~(int64_t)15;
+        const int64_t tail = h.run - head - body;
+        if (head || tail) {
+          HostBox p = h;
+          if (head) {
+            p.run = head;
+            add(p);
+          }
+          p.src = h.src + head, p.dst = h.dst + head, p.run = body;
+          add(p);
+          if (tail) {
+            p.src = h.src + head + body, p.dst = h.dst + head + body, p.run = tail;
+            add(p);
+          }
+          return;
+        }
+      }
+      const int64_t max_run = (int64_t)1 << 30; // keeps column counts inside 32 bits at any vector width
+      if (h.run > max_run) {
+        HostBox p = h;
+        for (int64_t off = 0; off < h.run; off += max_run) {
+          p.src = h.src + off, p.dst = h.dst + off;
+          p.run = std::min(max_run, h.run - off);
+          add(p);
+        }
+        return;
+      }
+      emit(h);
+      return;
+    }
+    uint64_t rows = 1;
+    for (int d = 0; d < h.nd; ++d) {
+      rows *= (uint64_t)h.shape[d];
+    }
+    if (h.nd > kMaxOuter || rows > 0x7fffffffull || h.run > ((int64_t)1 << 30)) {
+      // walk the slowest extent on the host
+      HostBox p = h;
+      p.nd = h.nd - 1;
+      for (int d = 0; d < p.nd; ++d) {
+        p.shape[d] = h.shape[d + 1];
+        p.sstride[d] = h.sstride[d + 1];
+        p.dstride[d] = h.dstride[d + 1];
+      }
+      for (int64_t i = 0; i < h.shape[0]; ++i) {
+        p.src = h.src + i * h.sstride[0];
+        p.dst = h.dst + i * h.dstride[0];
+        add(p);
+      }
+      return;
+    }
+    emit(h);
+  }
+};
+
+// Drops unit extents, merges extents that are contiguous with each other on
+// both sides, and splits off the innermost extent as the byte run when it is
+// dense on both sides.  Returns false for an empty box.
+bool canonicalise(const char* src, char* dst, int ndim, const int64_t* shape, const int64_t* sstr,
+    const int64_t* dstr, int64_t itemsize, HostBox& h) {
+  h.src = src;
+  h.dst = dst;
+  h.nd = 0;
+  h.run = itemsize;
+  for (int d = 0; d < ndim; ++d) {
+    if (shape[d] == 0) {
+      return false;
+    }
+  }
+  for (int d = 0; d < ndim; ++d) {
+    if (shape[d] == 1) {
+      continue;
+    }
+    const int64_t ss = sstr[d] * itemsize, ds = dstr[d] * itemsize;
+    h.shape[h.nd] = shape[d];
+    h.sstride[h.nd] = ss;
+    h.dstride[h.nd] = ds;
+    ++h.nd;
+  }
+  // merge from the inside out
+  int n = 0;
+  for (int d = 0; d < h.nd; ++d) {
+    if (n > 0 && h.sstride[n - 1] == h.shape[d] * h.sstride[d] && h.dstride[n - 1] == h.shape[d] * h.dstride[d]) {
+      h.shape[n - 1] *= h.shape[d];
+      h.sstride[n - 1] = h.sstride[d];
+      h.dstride[n - 1] = h.dstride[d];
+    } else {
+      h.shape[n] = h.shape[d];
+      h.sstride[n] = h.sstride[d];
+      h.dstride[n] = h.dstride[d];
+      ++n;
+    }
+  }
+  h.nd = n;
+  if (h.nd > 0 && h.sstride[h.nd - 1] == itemsize && h.dstride[h.nd - 1] == itemsize) {
+    h.run = h.shape[h.nd - 1] * itemsize;
+    --h.nd;
+  }
+  return true;
+}
+
+} // namespace
+} // namespace mdh
+
+extern "C" int mdh_copy_boxes(const mdh_box* boxes, int nboxes, int itemsize, void* stream) {
+  using namespace mdh;
+  if (nboxes < 0 || (nboxes > 0 && !boxes)) {
+    set_error("mdh_copy_boxes: bad box table");
+    return MDH_EINVAL;
+  }
+  if (itemsize < 1 || itemsize > 16 || (itemsize & (itemsize - 1))) {
+    set_error("mdh_copy_boxes: itemsize %d is not 1, 2, 4, 8 or 16", itemsize);
+    return MDH_EINVAL;
+  }
+  Launcher L;
+  L.stream = (hipStream_t)stream;
+  for (int i = 0; i < nboxes; ++i) {
+    const mdh_box& b = boxes[i];
+    if (b.ndim < 0 || b.ndim > MDH_MAX_DIMS) {
+      set_error("mdh_copy_boxes: box %d has %d dimensions (0..%d allowed)", i, b.ndim, MDH_MAX_DIMS);
+      return MDH_EINVAL;
+    }
+    int64_t numel = 1;
+    for (int d = 0; d < b.ndim; ++d) {
+      if (b.shape[d] < 0 || b.src_strides[d] < 0 || b.dst_strides[d] < 0) {
+        set_error("mdh_copy_boxes: box %d has a negative extent or stride", i);
+        return MDH_EINVAL;
+      }
+      if (b.shape[d] && numel > ((int64_t)1 << 48) / b.shape[d]) {
+        set_error("mdh_copy_boxes: box %d is not a plausible device size", i);
+        return MDH_EINVAL;
+      }
+      numel *= b.shape[d];
+    }
+    if (numel == 0) {
+      continue;
+    }
+    if (!b.src || !b.dst) {
+      set_error("mdh_copy_boxes: box %d has a null pointer", i);
+      return MDH_EINVAL;
+    }
+    if (((uintptr_t)b.src | (uintptr_t)b.dst) % (unsigned)itemsize) {
+      set_error("mdh_copy_boxes: box %d is not aligned to its element size", i);
+      return MDH_EINVAL;
+    }
+    HostBox h;
+    if (canonicalise((const char*)b.src, (char*)b.dst, b.ndim, b.shape, b.src_strides, b.dst_strides, itemsize, h)) {
+      L.add(h);
+    }
+  }
+  if (L.rc == MDH_OK) {
+    L.flush();
+  }
+  return L.rc;
+}
+
+extern "C" int mdh_gather(const void* const* srcs, int nsrc, void* dst, size_t width, size_t rows, size_t src_pitch,
+    size_t dst_pitch, size_t dst_shard_stride, void* stream) {
+  using namespace mdh;
+  if (nsrc < 0 || nsrc > 65536) {
+    set_error("mdh_gather: nsrc %d out of range", nsrc);
+    return MDH_EINVAL;
+  }
+  if (nsrc == 0 || width == 0 || rows == 0) {
+    return MDH_OK;
+  }
+  if (!srcs || !dst) {
+    set_error("mdh_gather: null pointer");
+    return MDH_EINVAL;
+  }
+  if (rows > 1 && (src_pitch < width || dst_pitch < width)) {
+    set_error("mdh_gather: a row pitch is smaller than the row width");
+    return MDH_EINVAL;
+  }
+  const size_t extent = (rows - 1) * dst_pitch + width;
+  if (nsrc > 1 && dst_shard_stride < extent) {
+    set_error("mdh_gather: shards would overlap in the destination");
+    return MDH_EINVAL;
+  }
+  if (width > ((size_t)1 << 48) || rows > ((size_t)1 << 40)) {
+    set_error("mdh_gather: not a plausible device size");
+    return MDH_EINVAL;
+  }
+  Launcher L;
+  L.stream = (hipStream_t)stream;
+  for (int s = 0; s < nsrc; ++s) {
+    if (!srcs[s]) {
+      set_error("mdh_gather: source %d is null", s);
+      return MDH_EINVAL;
+    }
+    char* out = (char*)dst + (size_t)s * dst_shard_stride;
+    if ((const char*)srcs[s] == out && (rows == 1 || src_pitch == dst_pitch)) {
+      continue; // shard already in place
+    }
+    const int64_t shape[2] = {(int64_t)rows, (int64_t)width};
+    const int64_t ss[2] = {(int64_t)src_pitch, 1};
+    const int64_t ds[2] = {(int64_t)dst_pitch, 1};
+    HostBox h;
+    if (canonicalise((const char*)srcs[s], out, 2, shape, ss, ds, 1, h)) {
+      L.add(h);
+    }
+  }
+  if (L.rc == MDH_OK) {
+    L.flush();
+  }
+  return L.rc;
+}

@@ -1,0 +1,89 @@
+// Device-side helpers shared by the gfx950 kernels: 16-byte streaming loads
+// and stores, and the host-side error plumbing of the C ABI.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "moodist_hip.h"
+
+namespace mdh {
+
+// One lane moves 16 bytes per instruction (global_load_dwordx4 /
+// global_store_dwordx4): a wave64 instruction covers 1 KiB of contiguous HBM.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kBlock = 256; // 4 wave64 per workgroup
+
+#ifndef MDH_NT_LOAD
+#define MDH_NT_LOAD 1
+#endif
+#ifndef MDH_NT_STORE
+#define MDH_NT_STORE 1
+#endif
+
+// Sources are read once and outputs written once, so both bypass cache
+// retention (the `nt` bit) and leave L2 / Infinity Cache to other work.
+template<typename V>
+__device__ __forceinline__ V stream_load(const V* p) {
+#if MDH_NT_LOAD
+  return __builtin_nontemporal_load(p);
+#else
+  return *p;
+#endif
+}
+
+template<typename V>
+__device__ __forceinline__ void stream_store(V* p, V v) {
+#if MDH_NT_STORE
+  __builtin_nontemporal_store(v, p);
+#else
+  *p = v;
+#endif
+}
+
+// Buffer addressing for tiles: the descriptor's base is wave-uniform and its
+// size bounds the tile, so out-of-range lanes load zero and their stores are
+// dropped by the address unit.  Cache-policy bits (gfx940 encoding of the
+// intrinsic's aux operand): 2 = nt, 16 = sc1.
+//   loads  nt   read-once data, evict first;
+//   stores sc1  device-scope write-through: the line leaves L2 at once rather
+//               than waiting as a dirty line (measurably faster than nt here).
+#ifndef MDH_LOAD_AUX
+#define MDH_LOAD_AUX 2
+#endif
+#ifndef MDH_STORE_AUX
+#define MDH_STORE_AUX 16
+#endif
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t tile_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, (int)bytes, 0x00020000);
+}
+
+__device__ __forceinline__ u32x4 tile_load(__amdgpu_buffer_rsrc_t rs, uint32_t byte_offset) {
+  return __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, (int)byte_offset, 0, MDH_LOAD_AUX));
+}
+
+__device__ __forceinline__ void tile_store(__amdgpu_buffer_rsrc_t rs, uint32_t byte_offset, u32x4 v) {
+  __builtin_amdgcn_raw_buffer_store_b128(v, rs, (int)byte_offset, 0, MDH_STORE_AUX);
+}
+
+// ---- host side ----
+
+void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+
+int check_launch(const char* what);
+
+struct Tuning {
+  int reduce_unroll = 4;
+  int reduce_max_blocks = 0;
+  int copy_unroll = 4;
+  int copy_max_blocks = 0;
+};
+Tuning& tuning();
+
+} // namespace mdh

@@ -1,0 +1,135 @@
+// C ABI entry of the K-source reduction: argument checks, fold-order rotation
+// of the pointer table, dispatch on element type.
+#include "reduce_kernels.h"
+
+extern "C" int mdh_reduce(const void* const* srcs, int nsrc, int first, void* dst, size_t numel, int dtype, int op,
+    float scale, void* stream) {
+  using namespace mdh;
+  if (nsrc < 1 || nsrc > MDH_MAX_SOURCES) {
+    set_error("mdh_reduce: nsrc %d outside 1..%d", nsrc, MDH_MAX_SOURCES);
+    return MDH_EINVAL;
+  }
+  if (first < 0 || first >= nsrc) {
+    set_error("mdh_reduce: first %d outside 0..%d", first, nsrc - 1);
+    return MDH_EINVAL;
+  }
+  size_t itemsize;
+  bool floating;
+  switch (dtype) {
+  case MDH_DTYPE_FLOAT32:
+    itemsize = 4, floating = true;
+    break;
+  case MDH_DTYPE_FLOAT64:
+    itemsize = 8, floating = true;
+    break;
+  case MDH_DTYPE_INT32:
+    itemsize = 4, floating = false;
+    break;
+  case MDH_DTYPE_INT64:
+    itemsize = 8, floating = false;
+    break;
+  case MDH_DTYPE_BFLOAT16:
+  case MDH_DTYPE_FLOAT16:
+    itemsize = 2, floating = true;
+    break;
+  default:
+    set_error("Unsupported dtype for reduce operation (%d)", dtype);
+    return MDH_EDTYPE;
+  }
+  int fold_op, mode = kPlain;
+  switch (op) {
+  case MDH_OP_SUM:
+    fold_op = kSum;
+    break;
+  case MDH_OP_AVG:
+    fold_op = kSum, mode = kAvg;
+    break;
+  case MDH_OP_PREMUL_SUM:
+    fold_op = kSum, mode = kPremul;
+    break;
+  case MDH_OP_MIN:
+    fold_op = kMin;
+    break;
+  case MDH_OP_MAX:
+    fold_op = kMax;
+    break;
+  default:
+    set_error("Unsupported reduce operation (%d)", op);
+    return MDH_EOP;
+  }
+  if (mode != kPlain && !floating) {
+    set_error("Unsupported reduce operation (%d) for integer dtype %d", op, dtype);
+    return MDH_EOP;
+  }
+  if (numel == 0) {
+    return MDH_OK;
+  }
+  if (numel > (size_t)1 << 48) {
+    set_error("mdh_reduce: numel %zu is not a plausible device size", numel);
+    return MDH_EINVAL;
+  }
+  if (!srcs || !dst) {
+    set_error("mdh_reduce: null pointer");
+    return MDH_EINVAL;
+  }
+  ReduceArgs a;
+  bool aligned = ((uintptr_t)dst % 16) == 0;
+  const uintptr_t bytes = (uintptr_t)numel * itemsize;
+  for (int j = 0; j < nsrc; ++j) {
+    const void* p = srcs[(first + j) % nsrc];
+    if (!p) {
+      set_error("mdh_reduce: source %d is null", (first + j) % nsrc);
+      return MDH_EINVAL;
+    }
+    if ((uintptr_t)p % itemsize) {
+      set_error("mdh_reduce: source %d is not aligned to its element size", (first + j) % nsrc);
+      return MDH_EINVAL;
+    }
+    // dst may be exactly one source (in-place allreduce); partial overlap would race
+    const uintptr_t s = (uintptr_t)p, d = (uintptr_t)dst;
+    if (s != d && s < d + bytes && d < s + bytes) {
+      set_error("mdh_reduce: destination partially overlaps source %d", (first + j) % nsrc);
+      return MDH_EINVAL;
+    }
+    aligned = aligned && ((uintptr_t)p % 16) == 0;
+    a.src[j] = p;
+  }
+  for (int j = nsrc; j < MDH_MAX_SOURCES; ++j) {
+    a.src[j] = nullptr;
+  }
+  if ((uintptr_t)dst % itemsize) {
+    set_error("mdh_reduce: destination is not aligned to its element size");
+    return MDH_EINVAL;
+  }
+  a.dst = dst;
+  a.numel = numel;
+  a.nvec = aligned ? bytes / 16 : 0;
+  a.scale = scale;
+  a.nsrc = nsrc;
+  a.mode = mode;
+  hipStream_t s = (hipStream_t)stream;
+#define MDH_DISPATCH(tname)                                  \
+  switch (fold_op) {                                         \
+  case kSum:                                                 \
+    return reduce_launch_##tname##_sum(a, aligned, s);       \
+  case kMin:                                                 \
+    return reduce_launch_##tname##_min(a, aligned, s);       \
+  default:                                                   \
+    return reduce_launch_##tname##_max(a, aligned, s);       \
+  }
+  switch (dtype) {
+  case MDH_DTYPE_FLOAT32:
+    MDH_DISPATCH(f32)
+  case MDH_DTYPE_FLOAT64:
+    MDH_DISPATCH(f64)
+  case MDH_DTYPE_INT32:
+    MDH_DISPATCH(i32)
+  case MDH_DTYPE_INT64:
+    MDH_DISPATCH(i64)
+  case MDH_DTYPE_BFLOAT16:
+    MDH_DISPATCH(bf16)
+  default:
+    MDH_DISPATCH(f16)
+  }
+#undef MDH_DISPATCH
+}

@@ -1,0 +1,81 @@
+"""The C-ABI library loads without a GPU, exports what include/moodist_hip.h declares, and
+rejects bad arguments before any launch.  No compute calls here."""
+
+import ctypes
+import os
+import re
+
+import pytest
+
+from moodist_amd import _abi as abi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "moodist_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mdh_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported():
+    L = abi.lib()
+    names = declared_symbols()
+    assert set(names) == set(abi.SYMBOLS)
+    for n in names:
+        assert getattr(L, n) is not None
+
+
+def test_abi_version_and_error_strings():
+    L = abi.lib()
+    assert L.mdh_abi_version() == abi.ABI_VERSION
+    assert L.mdh_error_string(0) == b"success"
+    assert L.mdh_error_string(2) == b"Unsupported dtype for reduce operation"
+    assert L.mdh_error_string(3) == b"Unsupported reduce operation"
+
+
+def test_box_struct_layout_matches_header():
+    # const void*, void*, int32, int32, 3 x int64[10]
+    assert ctypes.sizeof(abi.Box) == 8 + 8 + 4 + 4 + 3 * 8 * abi.MAX_DIMS
+
+
+@pytest.mark.parametrize("call,match", [
+    (lambda: abi.reduce([], 0, 16, 4, abi.DTYPE_FLOAT32, abi.OP_SUM), "nsrc 0 outside"),
+    (lambda: abi.reduce([16] * 65, 0, 16, 4, abi.DTYPE_FLOAT32, abi.OP_SUM), "nsrc 65 outside"),
+    (lambda: abi.reduce([16, 32], 2, 48, 4, abi.DTYPE_FLOAT32, abi.OP_SUM), "first 2 outside"),
+    (lambda: abi.reduce([16], 0, 32, 4, 0, abi.OP_SUM), "Unsupported dtype for reduce operation"),
+    (lambda: abi.reduce([16], 0, 32, 4, abi.DTYPE_FLOAT32, 2), "Unsupported reduce operation"),
+    (lambda: abi.reduce([16], 0, 32, 4, abi.DTYPE_INT32, abi.OP_AVG), "Unsupported reduce operation"),
+    (lambda: abi.reduce([16], 0, 32, 4, abi.DTYPE_INT64, abi.OP_PREMUL_SUM), "Unsupported reduce operation"),
+    (lambda: abi.reduce([0], 0, 32, 4, abi.DTYPE_FLOAT32, abi.OP_SUM), "source 0 is null"),
+    (lambda: abi.reduce([16], 0, 0, 4, abi.DTYPE_FLOAT32, abi.OP_SUM), "null pointer"),
+    (lambda: abi.reduce([18], 0, 64, 4, abi.DTYPE_FLOAT32, abi.OP_SUM), "not aligned to its element size"),
+    (lambda: abi.reduce([64], 0, 72, 4, abi.DTYPE_FLOAT32, abi.OP_SUM), "partially overlaps"),
+    (lambda: abi.gather([16], 1024, 8, 2, 4, 8, 64), "row pitch is smaller"),
+    (lambda: abi.gather([16, 32], 1024, 8, 2, 8, 8, 8), "shards would overlap"),
+    (lambda: abi.gather([0], 1024, 8, 1, 8, 8, 8), "source 0 is null"),
+    (lambda: abi.copy_boxes([abi.make_box(16, 32, [4], [1], [1])], 3), "itemsize 3"),
+    (lambda: abi.copy_boxes([abi.make_box(0, 32, [4], [1], [1])], 4), "null pointer"),
+    (lambda: abi.copy_boxes([abi.make_box(16, 32, [4], [-1], [1])], 4), "negative extent or stride"),
+    (lambda: abi.copy_boxes([abi.make_box(18, 32, [4], [1], [1])], 4), "not aligned to its element size"),
+    (lambda: abi.set_tuning("no_such_knob", 1), "unknown knob"),
+    (lambda: abi.set_tuning("reduce_unroll", 3), "does not take 3"),
+])
+def test_bad_arguments_are_refused_before_launch(call, match):
+    with pytest.raises(abi.MoodistError, match=match):
+        call()
+
+
+def test_empty_work_is_a_no_op_without_a_device():
+    abi.reduce([16], 0, 32, 0, abi.DTYPE_FLOAT32, abi.OP_SUM)  # numel == 0
+    abi.gather([16], 1024, 0, 1, 0, 0, 0)
+    abi.gather([], 1024, 8, 1, 8, 8, 8)
+    abi.copy_boxes([], 4)
+    abi.copy_boxes([abi.make_box(16, 32, [4, 0], [1, 1], [1, 1])], 4)
+
+
+def test_tuning_round_trip():
+    old = abi.get_tuning("copy_unroll")
+    abi.set_tuning("copy_unroll", 2)
+    assert abi.get_tuning("copy_unroll") == 2
+    abi.set_tuning("copy_unroll", old)

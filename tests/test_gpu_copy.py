@@ -1,0 +1,242 @@
+"""Parity of the HIP gather / box-copy kernels against the oracle and torch slicing, through the
+C ABI.  Everything here is byte-exact."""
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from moodist_amd import _abi as abi
+
+pytestmark = pytest.mark.gpu
+
+
+def sync():
+    torch.cuda.synchronize()
+
+
+def st():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def gpu_all_gather(shards, out):
+    b = shards[0].numel() * shards[0].element_size()
+    abi.gather([s.data_ptr() for s in shards], out.data_ptr(), b, 1, b, b, b, st())
+    sync()
+
+
+@pytest.mark.parametrize("P", [1, 2, 8, 33, 64, 100])
+def test_allgather_ragged_byte_sizes(dev, P):
+    for nbytes in (1, 4, 7, 28, 255 * 4, 1020, 4096, 65536 + 12, (1 << 20) + 2):
+        g = torch.Generator().manual_seed(nbytes + P)
+        shards = [torch.randint(0, 256, (nbytes,), dtype=torch.uint8, generator=g) for _ in range(P)]
+        out = torch.zeros(nbytes * P + 16, dtype=torch.uint8, device=dev)
+        gpu_all_gather([s.to(dev) for s in shards], out[:nbytes * P])
+        want = oracle.all_gather([s.numpy() for s in shards])
+        assert np.array_equal(out[:nbytes * P].cpu().numpy(), want)
+        assert (out[nbytes * P:] == 0).all()
+
+
+def test_reference_known_answers(dev):
+    # reference tests/test_processgroup.py:21-48, :82-109, :112-146
+    P = 8
+    shards = [torch.full((4,), float(r), device=dev) for r in range(P)]
+    out = torch.zeros(4 * P, device=dev)
+    gpu_all_gather(shards, out)
+    assert torch.equal(out.cpu(), torch.arange(P).float().repeat_interleave(4))
+    shards = [torch.arange(r * 100, r * 100 + 8, dtype=torch.float32, device=dev) for r in range(P)]
+    out = torch.zeros(8 * P, device=dev)
+    gpu_all_gather(shards, out)
+    for r in range(P):
+        assert torch.equal(out[r * 8:(r + 1) * 8], shards[r])
+    chunk = 256 * 1024
+    cpu = []
+    for r in range(P):
+        torch.manual_seed(r + 42)
+        cpu.append(torch.randn(chunk))
+    out = torch.zeros(chunk * P, device=dev)
+    gpu_all_gather([c.to(dev) for c in cpu], out)
+    assert torch.equal(out.cpu(), torch.cat(cpu))
+
+
+def test_misaligned_shards_and_output(dev):
+    P, n = 5, 10001
+    g = torch.Generator().manual_seed(1)
+    raw = [torch.randint(0, 256, (n + 32,), dtype=torch.uint8, generator=g) for _ in range(P)]
+    dsh = [r.to(dev)[1 + 3 * i:][:n] for i, r in enumerate(raw)]
+    canvas = torch.full((P * n + 64,), 9, dtype=torch.uint8, device=dev)
+    out = canvas[5:5 + P * n]
+    gpu_all_gather(dsh, out)
+    want = torch.cat([r[1 + 3 * i:][:n] for i, r in enumerate(raw)])
+    assert torch.equal(out.cpu(), want)
+    assert (canvas[:5] == 9).all() and (canvas[5 + P * n:] == 9).all()
+
+
+def test_shard_already_in_place_is_skipped(dev):
+    # allreduce gathers into the tensor its own chunk already lives in (core/processgroup.cc:1689-1693)
+    P, n, rank = 4, 1000, 2
+    out = torch.zeros(P * n, device=dev)
+    shards = [torch.full((n,), float(r + 1), device=dev) for r in range(P)]
+    out[rank * n:(rank + 1) * n] = 99.0
+    shards[rank] = out[rank * n:(rank + 1) * n]
+    gpu_all_gather(shards, out)
+    for r in range(P):
+        assert (out[r * n:(r + 1) * n] == (99.0 if r == rank else r + 1)).all()
+
+
+def test_gather_2d_against_oracle(dev):
+    g = torch.Generator().manual_seed(2)
+    for rows, width, sp, dp, pad in ((37, 200, 256, 300, 64), (64, 4096, 4096, 8192, 0), (5, 3, 7, 11, 1),
+                                     (16, 8192, 8192, 8192 + 512, 0)):
+        P = 5
+        stride = rows * dp + pad
+        shards = [torch.randint(0, 256, (rows * sp,), dtype=torch.uint8, generator=g) for _ in range(P)]
+        out = torch.full((P * stride,), 7, dtype=torch.uint8, device=dev)
+        abi.gather([s.to(dev).data_ptr() for s in shards], out.data_ptr(), width, rows, sp, dp, stride, st())
+        keep = [s.to(dev) for s in shards]  # noqa: F841  (the line above must not free them early)
+        sync()
+        d = [s.to(dev) for s in shards]
+        out.fill_(7)
+        abi.gather([s.data_ptr() for s in d], out.data_ptr(), width, rows, sp, dp, stride, st())
+        sync()
+        want = np.full(P * stride, 7, dtype=np.uint8)
+        oracle.gather([s.numpy() for s in shards], want, width, rows, sp, dp, stride)
+        assert np.array_equal(out.cpu().numpy(), want), (rows, width, sp, dp)
+
+
+@pytest.mark.parametrize("unroll", [1, 2, 4, 8])
+@pytest.mark.parametrize("max_blocks", [0, 5])
+def test_copy_parity_under_every_launch_shape(dev, unroll, max_blocks):
+    old = abi.get_tuning("copy_unroll"), abi.get_tuning("copy_max_blocks")
+    try:
+        abi.set_tuning("copy_unroll", unroll)
+        abi.set_tuning("copy_max_blocks", max_blocks)
+        G = torch.randn(96, 200)
+        Gd = G.to(dev)
+        out = torch.zeros(96, 40, device=dev)
+        boxes = [abi.make_box(Gd[12 * s:].data_ptr() + 40 * 2 * 4, out[12 * s:].data_ptr(), [12, 40], [200, 1], [40, 1])
+                 for s in range(8)]
+        abi.copy_boxes(boxes, 4, st())
+        sync()
+        assert torch.equal(out.cpu(), G[:, 80:120])
+        shards = [torch.randn(30000 + 1, device=dev) for _ in range(3)]
+        o = torch.zeros(3 * 30001, device=dev)
+        gpu_all_gather(shards, o)
+        assert torch.equal(o, torch.cat(shards))
+    finally:
+        abi.set_tuning("copy_unroll", old[0])
+        abi.set_tuning("copy_max_blocks", old[1])
+
+
+def _strides(t):
+    return list(t.stride())
+
+
+def test_boxes_against_torch_slicing(dev):
+    g = torch.Generator().manual_seed(5)
+    for dtype in (torch.uint8, torch.bfloat16, torch.float32, torch.float64):
+        isz = torch.empty(0, dtype=dtype).element_size()
+        G = torch.randint(0, 200, (6, 10, 7, 12), generator=g).to(dtype)
+        Gd = G.to(dev)
+        # strided -> contiguous, contiguous -> strided, strided -> strided with transposing strides
+        sl = (slice(1, 5), slice(0, 10), slice(2, 5), slice(3, 11))
+        box = Gd[sl]
+        out = torch.zeros(box.shape, dtype=dtype, device=dev)
+        abi.copy_boxes([abi.make_box(box.data_ptr(), out.data_ptr(), list(box.shape), _strides(box), _strides(out))],
+                       isz, st())
+        sync()
+        assert torch.equal(out.cpu(), G[sl])
+        back = torch.zeros_like(Gd)
+        bb = back[sl]
+        abi.copy_boxes([abi.make_box(out.data_ptr(), bb.data_ptr(), list(bb.shape), _strides(out), _strides(bb))],
+                       isz, st())
+        sync()
+        assert torch.equal(back[sl].cpu(), G[sl]) and back.float().sum().item() == G[sl].float().sum().item()
+        T = torch.zeros(12, 7, 10, 6, dtype=dtype, device=dev)
+        Tv = T.permute(3, 2, 1, 0)
+        abi.copy_boxes([abi.make_box(Gd.data_ptr(), T.data_ptr(), list(G.shape), _strides(Gd), _strides(Tv))],
+                       isz, st())
+        sync()
+        assert torch.equal(T.cpu(), G.permute(3, 2, 1, 0).contiguous())
+
+
+def test_boxes_many_dims_many_boxes_and_empty(dev):
+    A = torch.randn(2, 3, 2, 3, 2, 3, 2, 2)  # 8 dims, box keeps odd extents so nothing merges
+    Ad = A.to(dev)
+    sl = tuple(slice(0, s - 1) if s > 2 else slice(0, s) for s in A.shape)
+    box = Ad[sl]
+    out = torch.zeros(box.shape, device=dev)
+    abi.copy_boxes([abi.make_box(box.data_ptr(), out.data_ptr(), list(box.shape), _strides(box), _strides(out))], 4,
+                   st())
+    sync()
+    assert torch.equal(out.cpu(), A[sl])
+    # 70 boxes in one call (more than one launch's table), one of them empty
+    src = torch.randn(70, 33, device=dev)
+    dst = torch.zeros(70, 40, device=dev)
+    boxes = [abi.make_box(src[i].data_ptr(), dst[i].data_ptr(), [33 if i != 9 else 0], [1], [1]) for i in range(70)]
+    abi.copy_boxes(boxes, 4, st())
+    sync()
+    want = torch.zeros(70, 40)
+    want[:, :33] = src.cpu()
+    want[9] = 0
+    assert torch.equal(dst.cpu(), want)
+    # zero-dimensional box = one element
+    a, b = torch.tensor([5.0], device=dev), torch.zeros(1, device=dev)
+    abi.copy_boxes([abi.make_box(a.data_ptr(), b.data_ptr(), [], [], [])], 4, st())
+    sync()
+    assert b.item() == 5.0
+
+
+# ---- BASELINE configurations at full size ----
+
+def test_config2_allgather_bf16_full_size_contiguous_and_strided(dev):
+    P, n = 8, 16777216
+    cpu = []
+    for r in range(P):
+        torch.manual_seed(r)
+        cpu.append(torch.randn(n).bfloat16())
+    shards = [c.to(dev) for c in cpu]
+    out = torch.zeros(P * n, dtype=torch.bfloat16, device=dev)
+    gpu_all_gather(shards, out)
+    want = torch.cat(cpu)
+    assert torch.equal(out.cpu(), want)
+    del out
+    # strided [8, 4096, 4096] view of a padded buffer
+    rows = cols = 4096
+    pad = 64
+    big = torch.zeros(P, rows, cols + pad, dtype=torch.bfloat16, device=dev)
+    abi.gather([s.data_ptr() for s in shards], big.data_ptr(), cols * 2, rows, cols * 2, (cols + pad) * 2,
+               rows * (cols + pad) * 2, st())
+    sync()
+    assert torch.equal(big[:, :, :cols].cpu(), want.view(P, rows, cols))
+    assert (big[:, :, cols:] == 0).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=str)
+def test_config5_matrix_rows_to_columns_full_size(dev, dtype):
+    P, n = 8, 8192
+    torch.manual_seed(0)
+    G = torch.randn(n, n).to(dtype)
+    slabs = [G[1024 * s:1024 * (s + 1)].contiguous().to(dev) for s in range(P)]
+    isz = G.element_size()
+    for k in (0, 3, 7):
+        out = torch.zeros(n, 1024, dtype=dtype, device=dev)
+        boxes = [abi.make_box(slabs[s].data_ptr() + 1024 * k * isz, out.data_ptr() + s * 1024 * 1024 * isz,
+                              [1024, 1024], [n, 1], [1024, 1]) for s in range(P)]
+        abi.copy_boxes(boxes, isz, st())
+        sync()
+        assert torch.equal(out.cpu(), G[:, 1024 * k:1024 * (k + 1)])
+
+
+def test_config5_3d_dim0_to_dim2_full_size(dev):
+    P = 8
+    torch.manual_seed(0)
+    G3 = torch.randn(64, 512, 1024).bfloat16()
+    slabs = [G3[8 * s:8 * (s + 1)].contiguous().to(dev) for s in range(P)]
+    for k in (0, 5):
+        out = torch.zeros(64, 512, 128, dtype=torch.bfloat16, device=dev)
+        boxes = [abi.make_box(slabs[s].data_ptr() + 128 * k * 2, out.data_ptr() + 8 * s * 512 * 128 * 2,
+                              [8, 512, 128], [512 * 1024, 1024, 1], [512 * 128, 128, 1]) for s in range(P)]
+        abi.copy_boxes(boxes, 2, st())
+        sync()
+        assert torch.equal(out.cpu(), G3[:, :, 128 * k:128 * (k + 1)])

@@ -1,0 +1,221 @@
+"""Pins oracle.c's orc_gather / orc_copy_box and oracle/planner.py.  No GPU."""
+
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle import planner
+
+
+def _u8(a):
+    return np.ascontiguousarray(a).view(np.uint8).reshape(-1)
+
+
+def test_reference_known_answer_allgather_constants():
+    # reference tests/test_processgroup.py:21-48
+    P, chunk = 8, 4
+    shards = [np.full(chunk, float(r), dtype=np.float32) for r in range(P)]
+    out = oracle.all_gather(shards).view(np.float32)
+    assert np.array_equal(out, np.repeat(np.arange(P, dtype=np.float32), chunk))
+
+
+def test_reference_known_answer_allgather_aranges():
+    # reference tests/test_processgroup.py:82-109
+    P, chunk = 8, 8
+    shards = [np.arange(r * 100, r * 100 + chunk, dtype=np.float32) for r in range(P)]
+    out = oracle.all_gather(shards).view(np.float32)
+    for r in range(P):
+        assert np.array_equal(out[r * chunk:(r + 1) * chunk], shards[r])
+
+
+def test_reference_known_answer_allgather_randn():
+    # reference tests/test_processgroup.py:112-146: seed rank+42, 256 Ki elements, torch.equal
+    P, chunk = 8, 256 * 1024
+    shards = []
+    for r in range(P):
+        torch.manual_seed(r + 42)
+        shards.append(torch.randn(chunk, dtype=torch.float32))
+    out = torch.from_numpy(oracle.all_gather([s.numpy() for s in shards]).view(np.float32))
+    assert torch.equal(out, torch.cat(shards))
+
+
+@pytest.mark.parametrize("size", [1, 7, 64, 255, 1024, 4096, 65536])
+def test_reference_known_answer_allgather_ragged(size):
+    # reference tests/test_stress.py:235-280
+    P = 8
+    out = oracle.all_gather([np.full(size, float(r), dtype=np.float32) for r in range(P)]).view(np.float32)
+    for r in range(P):
+        assert (out[r * size:(r + 1) * size] == float(r)).all()
+
+
+def test_gather_2d_against_numpy():
+    rng = np.random.RandomState(1)
+    P, rows, width, sp, dp = 5, 37, 200, 256, 300
+    stride = rows * dp + 64
+    shards = [rng.randint(0, 256, rows * sp).astype(np.uint8) for _ in range(P)]
+    out = np.full(P * stride, 7, dtype=np.uint8)
+    oracle.gather(shards, out, width, rows, sp, dp, stride)
+    want = np.full(P * stride, 7, dtype=np.uint8)
+    for s in range(P):
+        src = shards[s].reshape(rows, sp)[:, :width]
+        want[s * stride:s * stride + rows * dp].reshape(rows, dp)[:, :width] = src
+    assert np.array_equal(out, want)
+
+
+@pytest.mark.parametrize("itemsize", [1, 2, 4, 8])
+def test_copy_box_against_numpy_slicing(itemsize):
+    rng = np.random.RandomState(itemsize)
+    dt = {1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[itemsize]
+    G = rng.randint(0, 255, (6, 5, 7, 4)).astype(dt)
+    out = np.zeros((3, 5, 2, 4), dtype=dt)
+    off = (2, 0, 3, 0)
+    shape = (3, 5, 2, 4)
+    es = lambda a: [s // itemsize for s in a.strides]
+    src_off = sum(o * s for o, s in zip(off, es(G)))
+    oracle.copy_box(_u8(G), src_off, _u8(out), 0, shape, es(G), es(out), itemsize)
+    assert np.array_equal(out, G[2:5, :, 3:5, :])
+    # and back into a strided destination, including a transposing stride order
+    back = np.zeros_like(G)
+    oracle.copy_box(_u8(out), 0, _u8(back), src_off, shape, es(out), es(back), itemsize)
+    assert np.array_equal(back[2:5, :, 3:5, :], out) and back.sum() == out.sum()
+    T = np.zeros((4, 2, 5, 3), dtype=dt)
+    oracle.copy_box(_u8(out), 0, _u8(T), 0, shape, es(out), [es(T)[3 - i] for i in range(4)], itemsize)
+    assert np.array_equal(T, out.transpose(3, 2, 1, 0))
+
+
+# ---------------- planner ----------------
+
+def _run_plan(size, shape, np_dtype, inputs_arg, outputs_arg, G):
+    """Plan, execute with the oracle and return per-rank output arrays (original arg order kept
+    only when sizes are equal, which is all these tests use)."""
+    itemsize = np.dtype(np_dtype).itemsize
+    descs = planner.plan(size, shape, itemsize, inputs_arg, outputs_arg)
+    ins = [[] for _ in range(size)]
+    for r, off, shp in inputs_arg:
+        sl = tuple(slice(o, o + s) for o, s in zip(off, shp))
+        ins[r].append(_u8(G[sl]).copy())
+    outs = [[np.zeros(n, dtype=np.uint8) for n in d.outputs] for d in descs]
+    planner.execute(descs, itemsize, ins, outs)
+    return descs, outs
+
+
+def _check_outputs(outputs_arg, outs, G, np_dtype):
+    counter = {}
+    for r, off, shp in outputs_arg:
+        i = counter.get(r, 0)
+        counter[r] = i + 1
+        sl = tuple(slice(o, o + s) for o, s in zip(off, shp))
+        got = outs[r][i].view(np_dtype).reshape(shp)
+        assert np.array_equal(got, G[sl]), (r, off, shp)
+
+
+def test_planner_hand_derived_4x4_row_to_column():
+    # 4x4 fp32 over 2 ranks, row-sharded -> column-sharded, derived by hand from
+    # core/processgroup.cc:2761-3104
+    inputs = [(0, [0, 0], [2, 4]), (1, [2, 0], [2, 4])]
+    outputs = [(0, [0, 0], [4, 2]), (1, [0, 2], [4, 2])]
+    d = planner.plan(2, [4, 4], 4, inputs, outputs)
+    r0, r1 = d
+    assert r0.inputs == [32] and r0.outputs == [32]
+    assert [(c.index, c.offset, c.shape) for c in r0.inputCopies] == [(0, [0, 0], [2, 2]), (0, [0, 2], [2, 2])]
+    assert [(c.index, c.offset, c.shape) for c in r1.inputCopies] == [(0, [0, 0], [2, 2]), (0, [0, 2], [2, 2])]
+    rd = [(x.rank, x.inputIndex, x.outputIndex, x.inputOffset, x.outputOffset, x.bytes) for x in r0.reads]
+    assert rd == [(0, 1, 0, 0, 0, 16), (1, 1, 0, 0, 16, 16)]
+    rd = [(x.rank, x.inputIndex, x.outputIndex, x.inputOffset, x.outputOffset, x.bytes) for x in r1.reads]
+    assert rd == [(0, 2, 0, 0, 0, 16), (1, 2, 0, 0, 16, 16)]
+    assert r0.outputCopies == [] and r1.outputCopies == []
+    G = np.arange(16, dtype=np.float32).reshape(4, 4)
+    _, outs = _run_plan(2, [4, 4], np.float32, inputs, outputs, G)
+    _check_outputs(outputs, outs, G, np.float32)
+
+
+def test_planner_column_to_row_uses_output_copies():
+    inputs = [(0, [0, 0], [4, 2]), (1, [0, 2], [4, 2])]
+    outputs = [(0, [0, 0], [2, 4]), (1, [2, 0], [2, 4])]
+    d = planner.plan(2, [4, 4], 4, inputs, outputs)
+    assert all(len(x.outputCopies) == 2 and x.inputCopies == [] for x in d)
+    G = np.arange(16, dtype=np.float32).reshape(4, 4)
+    _, outs = _run_plan(2, [4, 4], np.float32, inputs, outputs, G)
+    _check_outputs(outputs, outs, G, np.float32)
+
+
+def test_planner_allgather_1d_plan():
+    # reference tests/test_compile_op.py:190-222
+    P, chunk = 8, 4
+    inputs = [(r, [r * chunk], [chunk]) for r in range(P)]
+    outputs = [(r, [0], [chunk * P]) for r in range(P)]
+    d = planner.plan(P, [chunk * P], 4, inputs, outputs)
+    for r in range(P):
+        assert d[r].inputCopies == [] and d[r].outputCopies == []
+        rd = [(x.rank, x.inputIndex, x.outputIndex, x.inputOffset, x.outputOffset, x.bytes) for x in d[r].reads]
+        assert rd == [(s, 0, 0, 0, s * chunk * 4, chunk * 4) for s in range(P)]
+
+
+def _cases():
+    P = 8
+    yield "p2p", P, [4], np.float32, [(0, [0], [4])], [(1, [0], [4])]  # test_compile_op.py:21-61
+    yield "broadcast", P, [8], np.float32, [(0, [0], [8])], [(r, [0], [8]) for r in range(P)]  # :64-99
+    yield "gather", P, [4 * P], np.float32, [(r, [4 * r], [4]) for r in range(P)], [(0, [0], [4 * P])]  # :102-144
+    yield "scatter", P, [4 * P], np.float32, [(0, [0], [4 * P])], [(r, [4 * r], [4]) for r in range(P)]  # :147-187
+    yield "allgather", P, [4 * P], np.float32, [(r, [4 * r], [4]) for r in range(P)], \
+        [(r, [0], [4 * P]) for r in range(P)]  # :190-222
+    yield "rows2d", P, [P, 4], np.float32, [(r, [r, 0], [1, 4]) for r in range(P)], \
+        [(r, [0, 0], [P, 4]) for r in range(P)]  # :225-258
+    yield "multi_in", P, [4], np.float32, [(0, [0], [2]), (0, [2], [2])], [(1, [0], [4])]  # :261-309
+    for dt in (np.float32, np.float64, np.int32, np.int64):  # :312-343
+        yield "dtype_%s" % np.dtype(dt).name, P, [4], dt, [(0, [0], [4])], [(r, [0], [4]) for r in range(P)]
+    yield "bystanders", P, [4], np.float32, [(0, [0], [4])], [(1, [0], [4])]  # :382-423
+    # beyond the reference's tests: strided slices on either side
+    yield "row_to_col", P, [16, 24], np.float32, [(r, [2 * r, 0], [2, 24]) for r in range(P)], \
+        [(r, [0, 3 * r], [16, 3]) for r in range(P)]
+    yield "col_to_row", P, [16, 24], np.int16, [(r, [0, 3 * r], [16, 3]) for r in range(P)], \
+        [(r, [2 * r, 0], [2, 24]) for r in range(P)]
+    yield "dim0_to_dim2", P, [8, 6, 16], np.uint16, [(r, [r, 0, 0], [1, 6, 16]) for r in range(P)], \
+        [(r, [0, 0, 2 * r], [8, 6, 2]) for r in range(P)]
+    yield "overlapping_outputs", 4, [6, 6], np.float32, [(r % 2, [3 * (r % 2), 0], [3, 6]) for r in range(2)], \
+        [(0, [1, 1], [4, 4]), (1, [0, 0], [6, 6]), (2, [2, 0], [2, 6]), (3, [0, 4], [6, 2])]
+
+
+@pytest.mark.parametrize("case", list(_cases()), ids=lambda c: c[0])
+def test_planner_executes_to_the_global_slice(case):
+    _, size, shape, dt, inputs, outputs = case
+    rng = np.random.RandomState(3)
+    G = rng.randint(-1000, 1000, shape).astype(dt)
+    descs, outs = _run_plan(size, shape, dt, inputs, outputs, G)
+    _check_outputs(outputs, outs, G, dt)
+    itemsize = np.dtype(dt).itemsize
+    for r, d in enumerate(descs):
+        # invariants: the reads cover the outputs exactly once
+        assert sum(x.bytes for x in d.reads) == sum(d.outputs)
+        written = {}
+        for x in d.reads:
+            if x.outputIndex < len(d.outputs):
+                key = x.outputIndex
+                seg = written.setdefault(key, np.zeros(d.outputs[key], dtype=np.int32))
+                seg[x.outputOffset:x.outputOffset + x.bytes] += 1
+        for seg in written.values():
+            assert seg.max() <= 1
+        assert all(x.bytes % itemsize == 0 for x in d.reads)
+
+
+def test_planner_reports_uncovered_outputs():
+    with pytest.raises(planner.PlanError, match="could not find input for all output elements"):
+        planner.plan(2, [8], 4, [(0, [0], [4])], [(1, [0], [8])])
+
+
+def test_shard_box_matches_torch_chunking():
+    # py/moodist/compile.py:21-59 says it matches Shard.local_shard_size_and_offset: check against
+    # torch.chunk-style ceil division on uneven sizes
+    for n, k in itertools.product([1, 7, 8, 9, 64, 65], [1, 2, 3, 8]):
+        chunk = (n + k - 1) // k
+        for c in range(k):
+            off, shp = planner.shard_box([n, 5], [k], [c], [0])
+            start = min(n, chunk * c)
+            stop = min(n, chunk * (c + 1))
+            assert off == [start, 0] or (shp[0] == 0 and off[0] == n)
+            assert shp == [stop - start, 5]
+    assert planner.shard_box([8, 8], [2, 4], [1, 3], [0, 1]) == ([4, 6], [4, 2])
+    assert planner.shard_box([8, 8], [2], None, [0]) == ([0, 0], [0, 0])
