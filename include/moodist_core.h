@@ -1,0 +1,136 @@
+/*
+ * moodist_core.h -- C ABI of the host core (libmoodist.so): the process-group
+ * operator surface for the single-GPU hot path, with the local peers of a
+ * group emulated inside one process.
+ *
+ * The reference exposes this surface as a table of C++ function pointers
+ * obtained through its one extern "C" symbol, moodistGetApi
+ * (api/moodist_api.h:134-271, core/moodist_api.cc:168-179); the functions
+ * below are the members of that table that belong to the path, by the same
+ * names and argument order (api/processgroup_api.h:29-65,
+ * api/moodist_api.h:197-216, :244-255), with
+ *   - TensorPtr (an opaque torch tensor reached through callbacks,
+ *     api/tensor_ptr.h:73-315) replaced by the plain moodist_tensor below,
+ *   - CUstream replaced by a hipStream_t passed as void*,
+ *   - C++ exceptions replaced by a return code (0 = success) plus
+ *     moodist_last_error() for the calling thread; messages are the
+ *     reference's where it has one.
+ *
+ * Peers.  The reference runs one process per rank and obtains its peers'
+ * buffer addresses through shared memory and CUDA IPC
+ * (core/processgroup.cc:1150-1169, :1448-1470).  Here a moodist_world stands
+ * for the node: it owns `size` process groups (ranks 0..size-1) on one
+ * device.  A collective call posts the caller's addresses; when every rank of
+ * the world has posted the same collective, the kernels of all ranks that
+ * asked for an output are launched, each on the stream its rank passed.  A
+ * rank that only contributes (its buffer is a staged peer contribution) posts
+ * with moodist_pg_stage_input().  The returned work is complete once that
+ * launch has happened; as in the reference (wrapper/processgroup_wrapper.cc:63-85)
+ * ordering with later work is by stream, not by the host.
+ *
+ * Nothing here synchronises the host with the device.
+ */
+#ifndef MOODIST_CORE_H
+#define MOODIST_CORE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* api/moodist_version.h:12 (kMoodistApiVersion) */
+#define MOODIST_CORE_API_VERSION 2
+
+typedef struct moodist_tensor {
+  void* data;         /* device pointer */
+  int64_t numel;
+  int32_t itemsize;
+  int32_t dtype;      /* torch ScalarType number (api/moodist_api.h:30-42) */
+  int32_t device;     /* device index, -1 for host memory */
+  int32_t contiguous; /* non-zero if dense row-major */
+  int32_t ndim;
+  int32_t reserved;
+  int64_t shape[10];
+} moodist_tensor;
+
+typedef struct moodist_world moodist_world;
+typedef struct moodist_pg moodist_pg;
+typedef struct moodist_work moodist_work;
+typedef struct moodist_op moodist_op;
+typedef struct moodist_future moodist_future;
+
+/* moodistGetApi's handshake (api/moodist_api.h:265-271): returns 0 unless
+ * expected_version == MOODIST_CORE_API_VERSION. */
+int moodist_core_check_version(uint32_t expected_version);
+const char* moodist_last_error(void);
+
+/* createProcessGroup (api/processgroup_api.h:21) for every local rank at once. */
+int moodist_world_create(int size, int device, moodist_world** world);
+void moodist_world_destroy(moodist_world* world);
+/* Borrowed pointer, valid until the world is destroyed. */
+moodist_pg* moodist_world_group(moodist_world* world, int rank);
+
+/* processGroupRank / processGroupSize (api/processgroup_api.h:30-31) */
+int moodist_pg_rank(moodist_pg* pg);
+int moodist_pg_size(moodist_pg* pg);
+/* processGroupGetOption / processGroupSetOption (api/processgroup_api.h:39-40).
+ * Names as in the reference (core/processgroup.cc:2455-2488): prefer_kernel_less,
+ * force_kernel_less, num_chunks, chunk_size, method.  Unknown name -> error. */
+int moodist_pg_get_option(moodist_pg* pg, const char* name, int64_t* value);
+int moodist_pg_set_option(moodist_pg* pg, const char* name, int64_t value);
+
+/* processGroupAllGather (api/processgroup_api.h:43; core/processgroup.cc:1059-1284) */
+int moodist_pg_all_gather(moodist_pg* pg, const moodist_tensor* output, const moodist_tensor* input, void* stream,
+    moodist_work** work);
+/* processGroupReduceScatter (api/processgroup_api.h:45-46; core/processgroup.cc:1290-1668).
+ * reduce_op is a c10d RedOpType number; premul_value is used by PREMUL_SUM only. */
+int moodist_pg_reduce_scatter(moodist_pg* pg, const moodist_tensor* output, const moodist_tensor* input,
+    int reduce_op, void* stream, float premul_value, moodist_work** work);
+/* processGroupAllreduce (api/processgroup_api.h:48-49; core/processgroup.cc:1674-1722): a
+ * reduce-scatter into the rank's own chunk followed by an all-gather, in place.  When numel
+ * is not a multiple of the group size the reference allocates a padded temporary through
+ * torch (:1694-1697); here the caller passes it as `scratch` (>= roundup(numel, size)
+ * elements, same dtype), or NULL when numel divides evenly. */
+int moodist_pg_allreduce(moodist_pg* pg, const moodist_tensor* tensor, const moodist_tensor* scratch, int reduce_op,
+    void* stream, float premul_value, moodist_work** work);
+/* No counterpart in the reference, where a peer's contribution is whatever that peer's own
+ * collective call passes: posts this rank's input for the next collective without asking
+ * for an output.  kind: 0 = all_gather, 1 = reduce_scatter. */
+int moodist_pg_stage_input(moodist_pg* pg, int kind, const moodist_tensor* input, int reduce_op, void* stream,
+    float premul_value, moodist_work** work);
+
+/* Work: wait() fails if not every rank has posted yet (the launch has not happened). */
+int moodist_work_is_completed(moodist_work* work);
+int moodist_work_wait(moodist_work* work);
+void moodist_work_destroy(moodist_work* work);
+
+/* compileOpFull (api/moodist_api.h:244-248; core/processgroup.cc:2761-3104, :3259-3290):
+ * every rank passes the same full lists; offsets and shapes are ndim ints per slice. */
+int moodist_compile_op_full(moodist_pg* pg, const int* shape, size_t ndim, int dtype, const int* input_ranks,
+    const int* input_offsets, const int* input_shapes, size_t n_inputs, const int* output_ranks,
+    const int* output_offsets, const int* output_shapes, size_t n_outputs, moodist_op** op);
+void moodist_op_destroy(moodist_op* op);
+/* customOpCall (api/moodist_api.h:250-252; core/processgroup.cc:3172-3256) */
+int moodist_op_call(moodist_op* op, const moodist_tensor* inputs, size_t n_inputs, const moodist_tensor* outputs,
+    size_t n_outputs, void* stream, moodist_future** future);
+/* futureWait (api/moodist_api.h:253-255; core/processgroup.cc:2650-2661) */
+int moodist_future_wait(moodist_future* future, void* stream);
+void moodist_future_destroy(moodist_future* future);
+
+/* The plan of the calling rank, as the reference's CustomOpDescriptor holds it
+ * (core/cputhread.h:296-322), for inspection.  what: 0 reads, 1 inputCopies, 2 outputCopies,
+ * 3 inputs, 4 outputs.  moodist_op_plan_count returns the number of entries. */
+int64_t moodist_op_plan_count(moodist_op* op, int what);
+/* reads: out[6] = rank, inputIndex, outputIndex, inputOffset, outputOffset, bytes. */
+int moodist_op_plan_read(moodist_op* op, size_t i, int64_t out[6]);
+/* copies: index, then ndim offsets, then ndim shapes into out (1 + 2*ndim values). */
+int moodist_op_plan_copy(moodist_op* op, int which, size_t i, int64_t* out, size_t out_len);
+/* inputs / outputs: byte size of entry i. */
+int64_t moodist_op_plan_size(moodist_op* op, int which, size_t i);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOODIST_CORE_H */

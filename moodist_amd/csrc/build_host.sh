@@ -1,0 +1,24 @@
+#!/bin/bash
+# Builds the host side in-tree:
+#   libmoodist.so   host core (g++, links neither HIP nor torch; loads both
+#                   libamdhip64.so and libmoodist_hip.so at first GPU use)
+#   _C*.so          pybind11 module on PyTorch-ROCm (skipped with MOODIST_SKIP_WRAPPER=1)
+set -euo pipefail
+here="$(cd "$(dirname "$0")" && pwd)"
+root="$(cd "$here/../.." && pwd)"
+pkg="$here/.."
+cxx="${CXX:-g++}"
+common=(-O2 -std=c++17 -fPIC -Wall -Wextra -fvisibility=hidden -I"$root/include" -I"$here/core")
+mkdir -p "$here/build"
+objs=()
+for f in hip_loader planner processgroup c_api; do
+  o="$here/build/core_$f.o"
+  "$cxx" "${common[@]}" -c "$here/core/$f.cc" -o "$o" &
+  objs+=("$o")
+done
+wait
+"$cxx" -shared -o "$pkg/libmoodist.so" "${objs[@]}" -ldl -lpthread -Wl,--no-undefined
+echo "built $pkg/libmoodist.so"
+if [ "${MOODIST_SKIP_WRAPPER:-0}" != "1" ] && [ -f "$here/wrapper/module.cc" ]; then
+  python3 "$here/wrapper/build_wrapper.py"
+fi

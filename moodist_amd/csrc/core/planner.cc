@@ -1,0 +1,299 @@
+#include "planner.h"
+
+#include <algorithm>
+#include <string>
+
+namespace moodist {
+
+size_t dims_numel(const Dims& d) {
+  size_t n = 1;
+  for (int64_t x : d) {
+    n *= (size_t)x;
+  }
+  return n;
+}
+
+// row-major element offset of `offset` inside a tensor of `shape` (core/processgroup.cc:2788-2796)
+size_t linear_offset(const Dims& offset, const Dims& shape) {
+  size_t result = 0, stride = 1;
+  for (size_t i = shape.size(); i-- > 0;) {
+    result += (size_t)offset[i] * stride;
+    stride *= (size_t)shape[i];
+  }
+  return result;
+}
+
+namespace {
+
+struct Slice {
+  uint32_t rank;
+  uint32_t index; // position among the rank's slices as the caller listed them
+  Dims offset, shape;
+  size_t numel;
+};
+
+struct Hit { // intersection of a destination with entry `index` of some list
+  Dims offset, shape;
+  size_t index;
+};
+
+bool overlaps(const Dims& ao, const Dims& as, const Dims& bo, const Dims& bs) {
+  for (size_t i = 0; i < ao.size(); ++i) {
+    if (ao[i] >= bo[i] + bs[i] || bo[i] >= ao[i] + as[i]) {
+      return false;
+    }
+  }
+  return true;
+}
+
+// a slab that spans every dimension but the first is one contiguous range (:2863-2870)
+bool whole_rows(const Dims& part, const Dims& whole) {
+  for (size_t i = 1; i < part.size(); ++i) {
+    if (part[i] != whole[i]) {
+      return false;
+    }
+  }
+  return true;
+}
+
+Dims minus(const Dims& a, const Dims& b) {
+  Dims r(a.size());
+  for (size_t i = 0; i < a.size(); ++i) {
+    r[i] = a[i] - b[i];
+  }
+  return r;
+}
+
+template<typename List, typename Get>
+std::vector<Hit> intersect(const Dims& doff, const Dims& dshape, const List& list, Get get) {
+  std::vector<Hit> hits;
+  for (size_t i = 0; i < list.size(); ++i) {
+    const auto& [so, ss] = get(list[i]);
+    if (!overlaps(so, ss, doff, dshape)) {
+      continue;
+    }
+    Hit h;
+    h.index = i;
+    h.offset.resize(doff.size());
+    h.shape.resize(doff.size());
+    for (size_t j = 0; j < doff.size(); ++j) {
+      const int64_t lo = std::max(so[j], doff[j]);
+      const int64_t hi = std::min(so[j] + ss[j], doff[j] + dshape[j]);
+      h.offset[j] = lo;
+      h.shape[j] = hi - lo;
+    }
+    hits.push_back(std::move(h));
+  }
+  return hits;
+}
+
+struct Message { // what a sender tells a receiver about one piece (TInput, :2735-2753)
+  Dims offset, shape;
+  uint32_t inputRank, outputRank, inputIndex, outputIndex;
+  size_t inputOffset, outputOffset; // elements
+  bool outputContiguous;
+  uint32_t originInput; // the sender's own tensor the piece really lives in
+};
+
+std::vector<Slice> number_slices(const std::vector<SliceSpec>& specs, int size, size_t ndim, const char* what) {
+  std::vector<uint32_t> counter((size_t)size, 0);
+  std::vector<Slice> out;
+  out.reserve(specs.size());
+  for (const SliceSpec& s : specs) {
+    if (s.rank < 0 || s.rank >= size) {
+      throw std::runtime_error(std::string("moodist.compile_op_full: ") + what + " names rank " +
+                               std::to_string(s.rank) + " outside the group");
+    }
+    if (s.offset.size() != ndim || s.shape.size() != ndim) {
+      throw std::runtime_error(std::string("moodist.compile_op_full: ") + what +
+                               " offset/shape do not have the tensor's number of dimensions");
+    }
+    for (size_t i = 0; i < ndim; ++i) {
+      if (s.offset[i] < 0 || s.shape[i] < 0) {
+        throw std::runtime_error(std::string("moodist.compile_op_full: ") + what + " has a negative offset or shape");
+      }
+    }
+    Slice d;
+    d.rank = (uint32_t)s.rank;
+    d.index = counter[(size_t)s.rank]++;
+    d.offset = s.offset;
+    d.shape = s.shape;
+    d.numel = dims_numel(s.shape);
+    out.push_back(std::move(d));
+  }
+  return out;
+}
+
+} // namespace
+
+std::vector<RankPlan> plan_redistribution(int size, const Dims& shape, size_t itemsize,
+    const std::vector<SliceSpec>& inputs_arg, const std::vector<SliceSpec>& outputs_arg) {
+  const size_t ndim = shape.size();
+  std::vector<Slice> inputs = number_slices(inputs_arg, size, ndim, "an input");
+  std::vector<Slice> outputs = number_slices(outputs_arg, size, ndim, "an output");
+
+  // a rank's outputs as the caller listed them
+  std::vector<std::vector<Slice>> outputsOf((size_t)size);
+  for (const Slice& o : outputs) {
+    outputsOf[o.rank].push_back(o);
+  }
+
+  // largest first, ties in listing order (:2848-2849)
+  auto bigger = [](const Slice& a, const Slice& b) { return a.numel > b.numel; };
+  std::stable_sort(inputs.begin(), inputs.end(), bigger);
+  std::stable_sort(outputs.begin(), outputs.end(), bigger);
+
+  std::vector<RankPlan> plans((size_t)size);
+  std::vector<std::vector<std::vector<Message>>> mail((size_t)size,
+      std::vector<std::vector<Message>>((size_t)size)); // mail[receiver][sender]
+
+  auto slice_box = [](const Slice* s) { return std::pair<const Dims&, const Dims&>(s->offset, s->shape); };
+  auto hit_box = [](const Hit& h) { return std::pair<const Dims&, const Dims&>(h.offset, h.shape); };
+
+  for (int rank = 0; rank < size; ++rank) {
+    std::vector<const Slice*> mine;
+    for (const Slice& s : inputs) {
+      if ((int)s.rank == rank) {
+        mine.push_back(&s);
+      }
+    }
+    std::vector<Hit> staged; // pieces this rank must copy out of a tensor into contiguous staging
+    RankPlan& plan = plans[(size_t)rank];
+
+    for (const Slice& dst : outputs) {
+      if (dst.numel == 0) {
+        continue;
+      }
+      for (const Hit& x : intersect(dst.offset, dst.shape, mine, slice_box)) {
+        const Slice& src = *mine[x.index];
+        const bool inputContiguous = whole_rows(x.shape, src.shape);
+        if (!inputContiguous) {
+          // Does staging made for an earlier destination already hold these elements as
+          // at most three contiguous ranges? (:2931-2962)
+          std::vector<Hit> again = intersect(dst.offset, dst.shape, staged, hit_box);
+          if (!again.empty() && again.size() < 4) {
+            size_t n = 0;
+            bool rows = true;
+            for (const Hit& y : again) {
+              n += dims_numel(y.shape);
+              rows = rows && whole_rows(y.shape, staged[y.index].shape);
+              if (!rows) {
+                break;
+              }
+            }
+            if (rows && n == dims_numel(x.shape)) {
+              for (const Hit& y : again) {
+                const Hit& st = staged[y.index];
+                Message m;
+                m.offset = y.offset;
+                m.shape = y.shape;
+                m.inputRank = (uint32_t)rank;
+                m.outputRank = dst.rank;
+                m.inputIndex = (uint32_t)(mine.size() + y.index);
+                m.outputIndex = dst.index;
+                m.inputOffset = linear_offset(minus(y.offset, st.offset), st.shape);
+                m.outputOffset = linear_offset(minus(y.offset, dst.offset), dst.shape);
+                m.outputContiguous = whole_rows(y.shape, dst.shape);
+                m.originInput = (uint32_t)st.index;
+                mail[dst.rank][(size_t)rank].push_back(std::move(m));
+              }
+              continue;
+            }
+          }
+        }
+        Message m;
+        m.offset = x.offset;
+        m.shape = x.shape;
+        m.inputRank = (uint32_t)rank;
+        m.outputRank = dst.rank;
+        m.inputIndex = (uint32_t)x.index;
+        m.outputIndex = dst.index;
+        m.inputOffset = linear_offset(minus(x.offset, src.offset), src.shape);
+        m.outputOffset = linear_offset(minus(x.offset, dst.offset), dst.shape);
+        m.originInput = (uint32_t)x.index;
+        if (!inputContiguous) {
+          m.inputIndex = (uint32_t)(mine.size() + staged.size());
+          m.inputOffset = 0;
+          staged.push_back(x);
+        }
+        m.outputContiguous = whole_rows(x.shape, dst.shape);
+        mail[dst.rank][(size_t)rank].push_back(std::move(m));
+      }
+    }
+
+    for (const Slice* s : mine) {
+      plan.inputs.push_back(itemsize * s->numel);
+      plan.inputShapes.push_back(s->shape);
+    }
+    for (const Slice& o : outputs) {
+      if ((int)o.rank == rank) {
+        plan.outputs.push_back(itemsize * o.numel);
+        plan.outputShapes.push_back(o.shape);
+      }
+    }
+    for (const Hit& h : staged) {
+      PlanCopy c;
+      c.index = (uint32_t)h.index;
+      c.offset = minus(h.offset, mine[h.index]->offset);
+      c.shape = h.shape;
+      plan.inputCopies.push_back(std::move(c));
+    }
+  }
+
+  // sorted positions of every rank's inputs, to resolve a transfer's source tensor
+  std::vector<std::vector<const Slice*>> inputsOf((size_t)size);
+  for (const Slice& s : inputs) {
+    inputsOf[s.rank].push_back(&s);
+  }
+
+  for (int rank = 0; rank < size; ++rank) {
+    RankPlan& plan = plans[(size_t)rank];
+    size_t want = 0;
+    for (const Slice& o : outputsOf[(size_t)rank]) {
+      want += o.numel;
+    }
+    size_t have = 0;
+    for (int sender = 0; sender < size; ++sender) {
+      for (const Message& m : mail[(size_t)rank][(size_t)sender]) {
+        const Slice& dst = outputsOf[(size_t)rank][m.outputIndex];
+        PlanRead r;
+        r.rank = m.inputRank;
+        r.inputIndex = m.inputIndex;
+        r.outputIndex = m.outputIndex;
+        r.inputOffset = itemsize * m.inputOffset;
+        r.outputOffset = itemsize * m.outputOffset;
+        const size_t n = dims_numel(m.shape);
+        r.bytes = itemsize * n;
+        have += n;
+        if (!m.outputContiguous) {
+          PlanCopy c;
+          c.index = r.outputIndex;
+          c.offset = minus(m.offset, dst.offset);
+          c.shape = m.shape;
+          r.outputIndex = (uint32_t)(plan.outputs.size() + plan.outputCopies.size());
+          r.outputOffset = 0;
+          plan.outputCopies.push_back(std::move(c));
+        }
+        plan.reads.push_back(r);
+
+        const Slice& src = *inputsOf[m.inputRank][m.originInput];
+        Transfer t;
+        t.srcRank = m.inputRank;
+        t.srcInput = m.originInput;
+        t.dstOutput = m.outputIndex;
+        t.shape = m.shape;
+        t.srcOffset = minus(m.offset, src.offset);
+        t.srcShape = src.shape;
+        t.dstOffset = minus(m.offset, dst.offset);
+        t.dstShape = dst.shape;
+        plan.transfers.push_back(std::move(t));
+      }
+    }
+    if (have != want) {
+      throw std::runtime_error("moodist.compile_op_full: could not find input for all output elements");
+    }
+  }
+  return plans;
+}
+
+} // namespace moodist

@@ -1,0 +1,512 @@
+#include "processgroup.h"
+
+#include <stdexcept>
+
+#include "hip_loader.h"
+
+namespace moodist {
+
+namespace {
+
+#define MD_CHECK(cond)                                                                             \
+  do {                                                                                             \
+    if (!(cond)) {                                                                                 \
+      throw std::runtime_error(std::string("moodist: check failed: " #cond " (") + __FILE__ + ":" + \
+                               std::to_string(__LINE__) + ")");                                    \
+    }                                                                                              \
+  } while (0)
+
+// dtypes the reduction kernels take: toInternalDtype (core/processgroup.cc:264-279) plus
+// float16, which the reference's table lacks
+void check_reduce_dtype(int dtype) {
+  switch (dtype) {
+  case MDH_DTYPE_FLOAT32:
+  case MDH_DTYPE_FLOAT64:
+  case MDH_DTYPE_INT32:
+  case MDH_DTYPE_INT64:
+  case MDH_DTYPE_BFLOAT16:
+  case MDH_DTYPE_FLOAT16:
+    return;
+  default:
+    throw std::runtime_error("Unsupported dtype for reduce operation");
+  }
+}
+
+// toInternalReduction (core/processgroup.cc:282-296)
+void check_reduce_op(int op) {
+  switch (op) {
+  case MDH_OP_SUM:
+  case MDH_OP_PREMUL_SUM:
+  case MDH_OP_AVG:
+  case MDH_OP_MIN:
+  case MDH_OP_MAX:
+    return;
+  default:
+    throw std::runtime_error("Unsupported reduce operation");
+  }
+}
+
+void check_device_tensor(const moodist_tensor& t, int device, const char* what) {
+  if (!t.contiguous) {
+    throw std::runtime_error(std::string("moodist: ") + what + " must be contiguous");
+  }
+  if (t.device < 0) {
+    throw std::runtime_error(std::string("moodist: ") + what +
+                             " is a CPU tensor; this build runs the GPU path only (no CPU fallback)");
+  }
+  if (t.device != device) {
+    throw std::runtime_error(std::string("moodist: ") + what + " is on device " + std::to_string(t.device) +
+                             ", the group is on device " + std::to_string(device));
+  }
+  MD_CHECK(t.numel >= 0 && t.itemsize > 0);
+  MD_CHECK(t.numel == 0 || t.data != nullptr);
+}
+
+size_t bytes_of(const moodist_tensor& t) {
+  return (size_t)t.numel * (size_t)t.itemsize;
+}
+
+} // namespace
+
+size_t dtype_size(int dtype) {
+  switch (dtype) {
+  case 0:  // UInt8
+  case 1:  // Int8
+  case 11: // Bool
+    return 1;
+  case 2: // Int16
+  case MDH_DTYPE_FLOAT16:
+  case MDH_DTYPE_BFLOAT16:
+    return 2;
+  case MDH_DTYPE_INT32:
+  case MDH_DTYPE_FLOAT32:
+    return 4;
+  case MDH_DTYPE_INT64:
+  case MDH_DTYPE_FLOAT64:
+    return 8;
+  default:
+    throw std::runtime_error("moodist: unsupported dtype " + std::to_string(dtype));
+  }
+}
+
+// ---------------------------------------------------------------- ProcessGroup
+
+ProcessGroup::Busy::Busy(ProcessGroup& pg) : pg(pg) {
+  if (!pg.busy.try_lock()) {
+    throw std::runtime_error("Concurrent use of process group detected - this is not supported. Moodist process "
+                             "groups are not thread-safe.");
+  }
+}
+
+ProcessGroup::Busy::~Busy() {
+  pg.busy.unlock();
+}
+
+int64_t ProcessGroup::get_option(const std::string& name) const {
+  if (name == "prefer_kernel_less") {
+    return options.preferKernelLess ? 1 : 0;
+  } else if (name == "force_kernel_less") {
+    return options.forceKernelLess ? 1 : 0;
+  } else if (name == "num_chunks") {
+    return options.numChunks;
+  } else if (name == "chunk_size") {
+    return options.chunkSize;
+  } else if (name == "method") {
+    return options.method;
+  }
+  throw std::runtime_error("Unknown option: " + name);
+}
+
+void ProcessGroup::set_option(const std::string& name, int64_t value) {
+  if (name == "prefer_kernel_less") {
+    options.preferKernelLess = value != 0;
+  } else if (name == "force_kernel_less") {
+    options.forceKernelLess = value != 0;
+  } else if (name == "num_chunks") {
+    options.numChunks = value;
+  } else if (name == "chunk_size") {
+    options.chunkSize = value;
+  } else if (name == "method") {
+    options.method = value;
+  } else {
+    throw std::runtime_error("Unknown option: " + name);
+  }
+}
+
+std::shared_ptr<Collective> ProcessGroup::all_gather(const moodist_tensor* output, const moodist_tensor& input,
+    void* stream) {
+  return all_gather_impl(output, input, stream, nullptr);
+}
+
+std::shared_ptr<Collective> ProcessGroup::all_gather_impl(const moodist_tensor* output, const moodist_tensor& input,
+    void* stream, const moodist_tensor* copy_back) {
+  Busy guard(*this);
+  check_device_tensor(input, world->device, "all_gather input");
+  const size_t bytes = bytes_of(input);
+  MD_CHECK(bytes > 0); // core/processgroup.cc:1078
+  Posting p;
+  p.input = input;
+  p.stream = stream;
+  if (output) {
+    check_device_tensor(*output, world->device, "all_gather output");
+    MD_CHECK(bytes_of(*output) == bytes * (size_t)size); // :1079
+    p.output = *output;
+    p.wants_output = true;
+    if (copy_back) {
+      p.copy_back = *copy_back;
+      p.has_copy_back = true;
+    }
+  }
+  const bool kernel_less = options.forceKernelLess || options.preferKernelLess;
+  return world->post(Kind::all_gather, next_seq++, rank, std::move(p), 0, 1.0f, bytes, input.dtype, 0, nullptr,
+      kernel_less);
+}
+
+std::shared_ptr<Collective> ProcessGroup::reduce_scatter(const moodist_tensor* output, const moodist_tensor& input,
+    int reduce_op, void* stream, float premul) {
+  Busy guard(*this);
+  check_device_tensor(input, world->device, "reduce_scatter input");
+  check_reduce_dtype(input.dtype);
+  check_reduce_op(reduce_op);
+  const bool floating = input.dtype == MDH_DTYPE_FLOAT32 || input.dtype == MDH_DTYPE_FLOAT64 ||
+                        input.dtype == MDH_DTYPE_BFLOAT16 || input.dtype == MDH_DTYPE_FLOAT16;
+  if ((reduce_op == MDH_OP_AVG || reduce_op == MDH_OP_PREMUL_SUM) && !floating) {
+    throw std::runtime_error("Unsupported reduce operation");
+  }
+  const size_t in_bytes = bytes_of(input);
+  MD_CHECK(in_bytes > 0 && in_bytes % (size_t)size == 0);
+  const size_t bytes = in_bytes / (size_t)size;
+  MD_CHECK(bytes % (size_t)input.itemsize == 0);
+  Posting p;
+  p.input = input;
+  p.stream = stream;
+  if (output) {
+    check_device_tensor(*output, world->device, "reduce_scatter output");
+    MD_CHECK(output->dtype == input.dtype);   // core/processgroup.cc:1312
+    MD_CHECK(bytes_of(*output) == bytes);     // :1325
+    p.output = *output;
+    p.wants_output = true;
+  }
+  return world->post(Kind::reduce_scatter, next_seq++, rank, std::move(p), reduce_op, premul, bytes, input.dtype, 0,
+      nullptr, false);
+}
+
+std::shared_ptr<Collective> ProcessGroup::allreduce(const moodist_tensor& tensor, const moodist_tensor* scratch,
+    int reduce_op, void* stream, float premul) {
+  check_device_tensor(tensor, world->device, "allreduce tensor");
+  MD_CHECK(tensor.numel > 0); // core/processgroup.cc:1678
+  const int64_t n = tensor.numel;
+  if (n % size == 0) {
+    // in place: reduce into this rank's own chunk, then gather every rank's chunk (:1686-1693)
+    moodist_tensor chunk = tensor;
+    chunk.numel = n / size;
+    chunk.data = (char*)tensor.data + (size_t)rank * (size_t)chunk.numel * (size_t)tensor.itemsize;
+    chunk.ndim = 1;
+    chunk.shape[0] = chunk.numel;
+    reduce_scatter(&chunk, tensor, reduce_op, stream, premul);
+    return all_gather(&tensor, chunk, stream);
+  }
+  // padded temporary (:1694-1720)
+  const int64_t padded = (n + size - 1) / size * size;
+  if (!scratch) {
+    throw std::runtime_error("moodist: allreduce of " + std::to_string(n) + " elements over " + std::to_string(size) +
+                             " ranks needs a scratch tensor of " + std::to_string(padded) + " elements");
+  }
+  check_device_tensor(*scratch, world->device, "allreduce scratch");
+  MD_CHECK(scratch->dtype == tensor.dtype && scratch->numel >= padded);
+  const size_t bytes = bytes_of(tensor);
+  check_hip(hip().MemcpyAsync(scratch->data, tensor.data, bytes, kHipMemcpyDeviceToDevice, stream), "hipMemcpyAsync");
+  moodist_tensor whole = *scratch;
+  whole.numel = padded;
+  whole.ndim = 1;
+  whole.shape[0] = padded;
+  moodist_tensor chunk = whole;
+  chunk.numel = padded / size;
+  chunk.data = (char*)whole.data + (size_t)rank * (size_t)chunk.numel * (size_t)tensor.itemsize;
+  chunk.shape[0] = chunk.numel;
+  reduce_scatter(&chunk, whole, reduce_op, stream, premul);
+  // the copy back into `tensor` follows this rank's gather, wherever that gets launched
+  return all_gather_impl(&whole, chunk, stream, &tensor);
+}
+
+std::shared_ptr<CompiledOp> ProcessGroup::compile_op_full(const Dims& shape, int dtype,
+    const std::vector<SliceSpec>& inputs, const std::vector<SliceSpec>& outputs) {
+  Busy guard(*this);
+  if (shape.size() > MDH_MAX_DIMS) {
+    // core/processgroup.cc:3138-3140
+    throw std::runtime_error("moodist.compile_op_full: ndim " + std::to_string(shape.size()) +
+                             " is too large and not supported!");
+  }
+  auto op = std::make_shared<CompiledOp>();
+  op->id = next_op_id++;
+  op->dtype = dtype;
+  op->itemsize = dtype_size(dtype);
+  op->plans = plan_redistribution(size, shape, op->itemsize, inputs, outputs);
+  // The reference sizes a rank's outputs largest-first (:2999-3004) but numbers its reads by
+  // listing order (:2974); the two agree only when listing order is already largest-first.
+  for (int r = 0; r < size; ++r) {
+    size_t prev = SIZE_MAX;
+    for (const SliceSpec& o : outputs) {
+      if (o.rank == r) {
+        const size_t n = dims_numel(o.shape);
+        if (n > prev) {
+          throw std::runtime_error("moodist.compile_op_full: a rank's outputs must be listed largest first");
+        }
+        prev = n;
+      }
+    }
+  }
+  return op;
+}
+
+std::shared_ptr<Collective> ProcessGroup::custom_op(const std::shared_ptr<CompiledOp>& op,
+    const moodist_tensor* inputs, size_t n_inputs, const moodist_tensor* outputs, size_t n_outputs, void* stream) {
+  Busy guard(*this);
+  const RankPlan& plan = op->plans[(size_t)rank];
+  // core/processgroup.cc:3180-3185, :3205-3216
+  if (n_inputs != plan.inputs.size()) {
+    throw std::runtime_error("moodist: custom op expected different number of inputs");
+  }
+  if (n_outputs != plan.outputs.size()) {
+    throw std::runtime_error("moodist: custom op expected different number of outputs");
+  }
+  Posting p;
+  p.stream = stream;
+  p.wants_output = n_outputs > 0;
+  for (size_t i = 0; i < n_inputs; ++i) {
+    if (!inputs[i].contiguous) {
+      throw std::runtime_error("Got a non-contiguous tensor. All tensors must be contiguous.");
+    }
+    if (bytes_of(inputs[i]) != plan.inputs[i]) {
+      throw std::runtime_error("moodist: custom op input has wrong size");
+    }
+    check_device_tensor(inputs[i], world->device, "custom op input");
+    p.inputs.push_back(inputs[i]);
+  }
+  for (size_t i = 0; i < n_outputs; ++i) {
+    if (!outputs[i].contiguous) {
+      throw std::runtime_error("Got a non-contiguous tensor. All tensors must be contiguous.");
+    }
+    if (bytes_of(outputs[i]) != plan.outputs[i]) {
+      throw std::runtime_error("moodist: custom op output has wrong size");
+    }
+    check_device_tensor(outputs[i], world->device, "custom op output");
+    p.outputs.push_back(outputs[i]);
+  }
+  return world->post(Kind::custom, next_seq++, rank, std::move(p), 0, 1.0f, 0, op->dtype, op->id, op, false);
+}
+
+// ---------------------------------------------------------------- World
+
+World::World(int size, int device) : size(size), device(device) {
+  if (size < 1 || size > MDH_MAX_SOURCES) {
+    throw std::runtime_error("moodist: a local world holds 1.." + std::to_string(MDH_MAX_SOURCES) + " ranks, not " +
+                             std::to_string(size));
+  }
+  for (int r = 0; r < size; ++r) {
+    groups.push_back(std::make_unique<ProcessGroup>(this, r, size));
+  }
+  events.assign((size_t)size, nullptr);
+}
+
+World::~World() {
+  for (void* e : events) {
+    if (e) {
+      hip().EventDestroy(e);
+    }
+  }
+}
+
+std::shared_ptr<Collective> World::post(Kind kind, uint64_t seq, int rank, Posting p, int reduce_op, float premul,
+    size_t bytes, int dtype, uint32_t op_id, const std::shared_ptr<CompiledOp>& op, bool kernel_less) {
+  std::lock_guard<std::mutex> l(mutex);
+  std::shared_ptr<Collective>& slot = pending[seq];
+  if (!slot) {
+    slot = std::make_shared<Collective>();
+    slot->kind = kind;
+    slot->seq = seq;
+    slot->reduce_op = reduce_op;
+    slot->premul = premul;
+    slot->bytes = bytes;
+    slot->dtype = dtype;
+    slot->op_id = op_id;
+    slot->post.resize((size_t)size);
+  }
+  std::shared_ptr<Collective> c = slot;
+  if (c->kind != kind || c->reduce_op != reduce_op || c->bytes != bytes || c->dtype != dtype || c->op_id != op_id ||
+      c->premul != premul) {
+    // the reference detects this across ranks and aborts (CHECK_DYN, core/cputhread.h:100-112)
+    throw std::runtime_error("moodist: rank " + std::to_string(rank) + " issued collective #" + std::to_string(seq) +
+                             " with a different operation, size, dtype or reduction than another rank did");
+  }
+  Posting& mine = c->post[(size_t)rank];
+  MD_CHECK(!mine.arrived);
+  p.arrived = true;
+  mine = std::move(p);
+  ++c->arrived;
+  if (c->arrived == size) {
+    pending.erase(seq);
+    try {
+      launch(*c, op, kernel_less);
+    } catch (const std::exception& e) {
+      c->error = e.what();
+      c->launched = true;
+      throw;
+    }
+    c->launched = true;
+  }
+  return c;
+}
+
+// A rank's launch reads buffers that other ranks' streams may still be producing, and later
+// work on those streams may overwrite what this launch reads.  With one shared stream (the
+// usual case) stream order covers both; otherwise every launch waits for an event recorded
+// on each other rank's stream, and every other stream waits for the launches.
+void World::order_streams_before(Collective& c) {
+  bool same = true;
+  for (const Posting& p : c.post) {
+    same = same && p.stream == c.post[0].stream;
+  }
+  if (same) {
+    return;
+  }
+  const HipRuntime& h = hip();
+  for (int r = 0; r < size; ++r) {
+    if (!events[(size_t)r]) {
+      check_hip(h.EventCreateWithFlags(&events[(size_t)r], kHipEventDisableTiming), "hipEventCreateWithFlags");
+    }
+    check_hip(h.EventRecord(events[(size_t)r], c.post[(size_t)r].stream), "hipEventRecord");
+  }
+  for (int q = 0; q < size; ++q) {
+    if (!c.post[(size_t)q].wants_output) {
+      continue;
+    }
+    for (int r = 0; r < size; ++r) {
+      if (c.post[(size_t)r].stream != c.post[(size_t)q].stream) {
+        check_hip(h.StreamWaitEvent(c.post[(size_t)q].stream, events[(size_t)r], 0), "hipStreamWaitEvent");
+      }
+    }
+  }
+}
+
+void World::order_streams_after(Collective& c) {
+  bool same = true;
+  for (const Posting& p : c.post) {
+    same = same && p.stream == c.post[0].stream;
+  }
+  if (same) {
+    return;
+  }
+  const HipRuntime& h = hip();
+  for (int q = 0; q < size; ++q) {
+    if (c.post[(size_t)q].wants_output) {
+      check_hip(h.EventRecord(events[(size_t)q], c.post[(size_t)q].stream), "hipEventRecord");
+    }
+  }
+  for (int r = 0; r < size; ++r) {
+    for (int q = 0; q < size; ++q) {
+      if (c.post[(size_t)q].wants_output && c.post[(size_t)r].stream != c.post[(size_t)q].stream) {
+        check_hip(h.StreamWaitEvent(c.post[(size_t)r].stream, events[(size_t)q], 0), "hipStreamWaitEvent");
+      }
+    }
+  }
+}
+
+void World::launch(Collective& c, const std::shared_ptr<CompiledOp>& op, bool kernel_less) {
+  const HipRuntime& h = hip();
+  int current = -1;
+  check_hip(h.GetDevice(&current), "hipGetDevice");
+  if (current != device) {
+    check_hip(h.SetDevice(device), "hipSetDevice");
+  }
+  order_streams_before(c);
+  std::vector<const void*> srcs((size_t)size);
+
+  if (c.kind == Kind::reduce_scatter) {
+    // out_q = in_q[q] (+) in_{q+1}[q] (+) ... in rank order starting at q (core/group.cc:567-570;
+    // core/reduce_scatter.cc:180-191), pitch = bytes (core/processgroup.cc:1322)
+    const size_t itemsize = dtype_size(c.dtype);
+    const size_t numel = c.bytes / itemsize;
+    // AVG is SUM then a multiply by 1.0f/size (core/processgroup.cc:1664-1667); PREMUL_SUM
+    // multiplies every input by the factor first (:1374-1378)
+    const float scale = c.reduce_op == MDH_OP_AVG ? 1.0f / (float)size : c.premul;
+    for (int q = 0; q < size; ++q) {
+      const Posting& pq = c.post[(size_t)q];
+      if (!pq.wants_output) {
+        continue;
+      }
+      for (int j = 0; j < size; ++j) {
+        srcs[(size_t)j] = (const char*)c.post[(size_t)j].input.data + c.bytes * (size_t)q;
+      }
+      check_mdh(h.reduce(srcs.data(), size, q, pq.output.data, numel, c.dtype, c.reduce_op, scale, pq.stream));
+    }
+  } else if (c.kind == Kind::all_gather) {
+    // out_q[pitch*j .. +bytes] = in_j for every j (core/allgather.cc:381-390)
+    for (int q = 0; q < size; ++q) {
+      const Posting& pq = c.post[(size_t)q];
+      if (!pq.wants_output) {
+        continue;
+      }
+      for (int j = 0; j < size; ++j) {
+        srcs[(size_t)j] = c.post[(size_t)j].input.data;
+      }
+      if (kernel_less) {
+        // copy-engine form (core/processgroup.cc:706-833): one device-to-device copy per shard
+        for (int j = 0; j < size; ++j) {
+          void* dst = (char*)pq.output.data + c.bytes * (size_t)j;
+          if (dst != srcs[(size_t)j]) {
+            check_hip(h.MemcpyAsync(dst, srcs[(size_t)j], c.bytes, kHipMemcpyDeviceToDevice, pq.stream),
+                "hipMemcpyAsync");
+          }
+        }
+      } else {
+        check_mdh(h.gather(srcs.data(), size, pq.output.data, c.bytes, 1, c.bytes, c.bytes, c.bytes, pq.stream));
+      }
+      if (pq.has_copy_back) {
+        // allreduce through a padded temporary: copy the result back (core/processgroup.cc:1716-1720)
+        const moodist_tensor& back = pq.copy_back;
+        check_hip(h.MemcpyAsync(back.data, pq.output.data, (size_t)back.numel * (size_t)back.itemsize,
+                      kHipMemcpyDeviceToDevice, pq.stream),
+            "hipMemcpyAsync");
+      }
+    }
+  } else {
+    // Every read of every rank, with its staging copies folded in, as strided box copies
+    // straight from the source rank's tensor into the destination tensor.
+    MD_CHECK(op != nullptr);
+    for (int q = 0; q < size; ++q) {
+      const Posting& pq = c.post[(size_t)q];
+      const RankPlan& plan = op->plans[(size_t)q];
+      if (plan.transfers.empty()) {
+        continue;
+      }
+      std::vector<mdh_box> boxes(plan.transfers.size());
+      for (size_t i = 0; i < plan.transfers.size(); ++i) {
+        const Transfer& t = plan.transfers[i];
+        const Posting& ps = c.post[t.srcRank];
+        MD_CHECK(t.srcInput < ps.inputs.size() && t.dstOutput < pq.outputs.size());
+        mdh_box& b = boxes[i];
+        const size_t nd = t.shape.size();
+        b.ndim = (int32_t)nd;
+        b.reserved = 0;
+        int64_t ss = 1, ds = 1;
+        for (size_t d = nd; d-- > 0;) {
+          b.shape[d] = t.shape[d];
+          b.src_strides[d] = ss;
+          b.dst_strides[d] = ds;
+          ss *= t.srcShape[d];
+          ds *= t.dstShape[d];
+        }
+        b.src = (const char*)ps.inputs[t.srcInput].data + linear_offset(t.srcOffset, t.srcShape) * op->itemsize;
+        b.dst = (char*)pq.outputs[t.dstOutput].data + linear_offset(t.dstOffset, t.dstShape) * op->itemsize;
+      }
+      check_mdh(h.copy_boxes(boxes.data(), (int)boxes.size(), (int)op->itemsize, pq.stream));
+    }
+  }
+  order_streams_after(c);
+  if (current != device && current >= 0) {
+    check_hip(h.SetDevice(current), "hipSetDevice");
+  }
+}
+
+} // namespace moodist

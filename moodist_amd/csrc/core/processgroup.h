@@ -1,0 +1,137 @@
+// Host side of the hot path: per-collective validation, the in-process
+// rendezvous that stands in for the reference's peer address exchange, and
+// the launches through the thin C ABI of the kernel library.
+//
+// Follows ProcessGroupImpl in the reference (core/processgroup.cc): all_gather
+// :1059-1284, reduce_scatter :1290-1668, allreduce :1674-1722, compileOpFull
+// :2761-3104 / :3259-3290, customOp :3172-3256, options :334-340 / :2455-2488.
+#pragma once
+
+#include <cstdint>
+#include <map>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "moodist_core.h"
+#include "planner.h"
+
+namespace moodist {
+
+class World;
+
+enum class Kind : int { all_gather = 0, reduce_scatter = 1, custom = 2 };
+
+// What one rank brought to a collective.
+struct Posting {
+  bool arrived = false;
+  bool wants_output = false;
+  moodist_tensor input{};
+  moodist_tensor output{};
+  std::vector<moodist_tensor> inputs; // custom op
+  std::vector<moodist_tensor> outputs;
+  bool has_copy_back = false; // allreduce through a padded temporary
+  moodist_tensor copy_back{};
+  void* stream = nullptr;
+};
+
+struct Collective {
+  Kind kind;
+  uint64_t seq;
+  int reduce_op = 0;
+  float premul = 1.0f;
+  size_t bytes = 0; // per-rank chunk
+  int dtype = 0;
+  uint32_t op_id = 0;
+  int arrived = 0;
+  bool launched = false;
+  std::string error; // set if the launch failed; reported to every waiter
+  std::vector<Posting> post;
+};
+
+struct Options { // core/processgroup.cc:334-340
+  bool preferKernelLess = false;
+  bool forceKernelLess = false;
+  int64_t numChunks = -1;
+  int64_t chunkSize = -1;
+  int64_t method = -1;
+};
+
+struct CompiledOp {
+  uint32_t id;
+  int dtype;
+  size_t itemsize;
+  std::vector<RankPlan> plans; // every rank's, computed identically by every rank
+};
+
+class ProcessGroup {
+public:
+  ProcessGroup(World* world, int rank, int size) : world(world), rank(rank), size(size) {}
+
+  std::shared_ptr<Collective> all_gather(const moodist_tensor* output, const moodist_tensor& input, void* stream);
+  std::shared_ptr<Collective> reduce_scatter(const moodist_tensor* output, const moodist_tensor& input, int reduce_op,
+      void* stream, float premul);
+  std::shared_ptr<Collective> allreduce(const moodist_tensor& tensor, const moodist_tensor* scratch, int reduce_op,
+      void* stream, float premul);
+  std::shared_ptr<CompiledOp> compile_op_full(const Dims& shape, int dtype, const std::vector<SliceSpec>& inputs,
+      const std::vector<SliceSpec>& outputs);
+  std::shared_ptr<Collective> custom_op(const std::shared_ptr<CompiledOp>& op, const moodist_tensor* inputs,
+      size_t n_inputs, const moodist_tensor* outputs, size_t n_outputs, void* stream);
+
+  int64_t get_option(const std::string& name) const;
+  void set_option(const std::string& name, int64_t value);
+
+  World* const world;
+  const int rank;
+  const int size;
+  Options options;
+
+private:
+  std::shared_ptr<Collective> all_gather_impl(const moodist_tensor* output, const moodist_tensor& input, void* stream,
+      const moodist_tensor* copy_back);
+
+  // "Concurrent use of process group detected" guard (core/processgroup.cc:172-183)
+  struct Busy {
+    explicit Busy(ProcessGroup& pg);
+    ~Busy();
+    ProcessGroup& pg;
+  };
+  std::mutex busy;
+  uint64_t next_seq = 0;
+  uint32_t next_op_id = 1;
+};
+
+// The node: `size` local ranks of one group sharing one device.
+class World {
+public:
+  World(int size, int device);
+  ~World();
+
+  ProcessGroup* group(int rank) {
+    return groups.at((size_t)rank).get();
+  }
+
+  // Posts `p` for (kind, seq); launches when the last rank arrives.  Throws if the ranks
+  // disagree about what collective number `seq` is (the reference aborts on this,
+  // core/cputhread.h:100-112).
+  std::shared_ptr<Collective> post(Kind kind, uint64_t seq, int rank, Posting p, int reduce_op, float premul,
+      size_t bytes, int dtype, uint32_t op_id, const std::shared_ptr<CompiledOp>& op, bool kernel_less);
+
+  const int size;
+  const int device;
+
+private:
+  void launch(Collective& c, const std::shared_ptr<CompiledOp>& op, bool kernel_less);
+  void order_streams_before(Collective& c);
+  void order_streams_after(Collective& c);
+
+  std::mutex mutex;
+  std::vector<std::unique_ptr<ProcessGroup>> groups;
+  std::map<uint64_t, std::shared_ptr<Collective>> pending;
+  std::vector<void*> events; // one per rank, created on first cross-stream use
+};
+
+size_t dtype_size(int dtype);
+
+} // namespace moodist

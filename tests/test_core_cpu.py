@@ -1,0 +1,330 @@
+"""Host core without a GPU: the C ABI of libmoodist.so, the planner against the oracle's
+restatement, argument checks and the rendezvous rules.  Nothing here launches a kernel."""
+
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import moodist_amd
+from oracle import planner
+from test_oracle_copy import _cases
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB = os.path.join(ROOT, "moodist_amd", "libmoodist.so")
+
+
+class Tensor(ctypes.Structure):
+    _fields_ = [("data", ctypes.c_void_p), ("numel", ctypes.c_int64), ("itemsize", ctypes.c_int32),
+                ("dtype", ctypes.c_int32), ("device", ctypes.c_int32), ("contiguous", ctypes.c_int32),
+                ("ndim", ctypes.c_int32), ("reserved", ctypes.c_int32), ("shape", ctypes.c_int64 * 10)]
+
+
+def fake(numel, dtype=6, itemsize=4, device=0, data=0x10000, contiguous=1):
+    t = Tensor()
+    t.data, t.numel, t.itemsize, t.dtype, t.device, t.contiguous, t.ndim = data, numel, itemsize, dtype, device, \
+        contiguous, 1
+    t.shape[0] = numel
+    return t
+
+
+@pytest.fixture(scope="module")
+def core():
+    L = ctypes.CDLL(LIB)
+    L.moodist_last_error.restype = ctypes.c_char_p
+    L.moodist_world_group.restype = ctypes.c_void_p
+    L.moodist_world_group.argtypes = [ctypes.c_void_p, ctypes.c_int]
+    L.moodist_world_destroy.argtypes = [ctypes.c_void_p]
+    L.moodist_pg_rank.argtypes = [ctypes.c_void_p]
+    L.moodist_pg_size.argtypes = [ctypes.c_void_p]
+    L.moodist_pg_reduce_scatter.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
+                                            ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p]
+    L.moodist_pg_all_gather.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                        ctypes.c_void_p]
+    L.moodist_pg_allreduce.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
+                                       ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p]
+    L.moodist_work_wait.argtypes = [ctypes.c_void_p]
+    L.moodist_work_is_completed.argtypes = [ctypes.c_void_p]
+    L.moodist_work_destroy.argtypes = [ctypes.c_void_p]
+    L.moodist_pg_get_option.argtypes = [ctypes.c_void_p, ctypes.c_char_p, ctypes.POINTER(ctypes.c_int64)]
+    L.moodist_pg_set_option.argtypes = [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_int64]
+    return L
+
+
+def make_world(core, size):
+    w = ctypes.c_void_p()
+    assert core.moodist_world_create(size, 0, ctypes.byref(w)) == 0, core.moodist_last_error()
+    return w
+
+
+def test_every_declared_symbol_is_exported(core):
+    text = open(os.path.join(ROOT, "include", "moodist_core.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = sorted(set(re.findall(r"\b(moodist_[a-z_0-9]+)\s*\(", text)))
+    assert len(names) >= 25
+    for n in names:
+        assert getattr(core, n) is not None
+
+
+def test_version_handshake(core):
+    # api/moodist_version.h:12: version 2; any other number is refused (api/moodist_api.h:265-271)
+    assert core.moodist_core_check_version(2) == 1
+    assert core.moodist_core_check_version(1) == 0
+    assert core.moodist_core_check_version(3) == 0
+
+
+def test_world_ranks_sizes_and_limits(core):
+    w = make_world(core, 8)
+    for r in range(8):
+        pg = core.moodist_world_group(w, r)
+        assert core.moodist_pg_rank(pg) == r and core.moodist_pg_size(pg) == 8
+    assert core.moodist_world_group(w, 8) is None
+    core.moodist_world_destroy(w)
+    bad = ctypes.c_void_p()
+    assert core.moodist_world_create(0, 0, ctypes.byref(bad)) != 0
+    assert core.moodist_world_create(65, 0, ctypes.byref(bad)) != 0
+    assert b"1..64 ranks" in core.moodist_last_error()
+
+
+def test_options_by_name(core):
+    w = make_world(core, 2)
+    pg = core.moodist_world_group(w, 0)
+    v = ctypes.c_int64()
+    for name, default in ((b"prefer_kernel_less", 0), (b"force_kernel_less", 0), (b"num_chunks", -1),
+                          (b"chunk_size", -1), (b"method", -1)):
+        assert core.moodist_pg_get_option(pg, name, ctypes.byref(v)) == 0 and v.value == default
+    assert core.moodist_pg_set_option(pg, b"chunk_size", 4096) == 0
+    core.moodist_pg_get_option(pg, b"chunk_size", ctypes.byref(v))
+    assert v.value == 4096
+    assert core.moodist_pg_set_option(pg, b"bogus", 1) != 0
+    assert core.moodist_last_error() == b"Unknown option: bogus"  # core/processgroup.cc:2469
+    core.moodist_world_destroy(w)
+
+
+def test_argument_checks_use_the_reference_messages(core):
+    w = make_world(core, 4)
+    pg = core.moodist_world_group(w, 0)
+    work = ctypes.c_void_p()
+
+    def rs(out, inp, op=0):
+        return core.moodist_pg_reduce_scatter(pg, ctypes.byref(out), ctypes.byref(inp), op, None, 0.0,
+                                              ctypes.byref(work))
+
+    assert rs(fake(4, dtype=0, itemsize=1), fake(16, dtype=0, itemsize=1)) != 0
+    assert core.moodist_last_error() == b"Unsupported dtype for reduce operation"  # core/processgroup.cc:277
+    assert rs(fake(4), fake(16), op=2) != 0
+    assert core.moodist_last_error() == b"Unsupported reduce operation"  # :294
+    assert rs(fake(4, dtype=3), fake(16, dtype=3), op=1) != 0  # AVG of int32
+    assert rs(fake(4), fake(16, contiguous=0)) != 0 and b"must be contiguous" in core.moodist_last_error()
+    assert rs(fake(4), fake(16, device=-1)) != 0 and b"no CPU fallback" in core.moodist_last_error()
+    assert rs(fake(4), fake(16, device=1)) != 0 and b"is on device 1" in core.moodist_last_error()
+    assert rs(fake(5), fake(16)) != 0  # output is not input / size
+    assert rs(fake(4, dtype=7, itemsize=8), fake(16)) != 0  # dtype mismatch
+    assert core.moodist_pg_all_gather(pg, ctypes.byref(fake(15)), ctypes.byref(fake(4)), None,
+                                      ctypes.byref(work)) != 0
+    assert core.moodist_pg_allreduce(pg, ctypes.byref(fake(7)), None, 0, None, 0.0, ctypes.byref(work)) != 0
+    assert b"needs a scratch tensor of 8 elements" in core.moodist_last_error()
+    core.moodist_world_destroy(w)
+
+
+def test_work_is_incomplete_until_every_rank_has_posted(core):
+    w = make_world(core, 4)
+    works = []
+    for r in range(3):  # the fourth rank never calls: nothing is launched, so no GPU is needed
+        pg = core.moodist_world_group(w, r)
+        work = ctypes.c_void_p()
+        assert core.moodist_pg_reduce_scatter(pg, ctypes.byref(fake(4)), ctypes.byref(fake(16)), 0, None, 0.0,
+                                              ctypes.byref(work)) == 0, core.moodist_last_error()
+        works.append(work)
+    for work in works:
+        assert core.moodist_work_is_completed(work) == 0
+        assert core.moodist_work_wait(work) != 0
+        assert b"3 of 4 have" in core.moodist_last_error()
+        core.moodist_work_destroy(work)
+    core.moodist_world_destroy(w)
+
+
+def test_mismatched_collectives_are_detected(core):
+    # the reference aborts when ranks disagree about a collective (CHECK_DYN, core/cputhread.h:100-112)
+    w = make_world(core, 4)
+    work = ctypes.c_void_p()
+    pg0, pg1 = core.moodist_world_group(w, 0), core.moodist_world_group(w, 1)
+    assert core.moodist_pg_reduce_scatter(pg0, ctypes.byref(fake(4)), ctypes.byref(fake(16)), 0, None, 0.0,
+                                          ctypes.byref(work)) == 0
+    assert core.moodist_pg_all_gather(pg1, ctypes.byref(fake(16)), ctypes.byref(fake(4)), None,
+                                      ctypes.byref(work)) != 0
+    assert b"different operation" in core.moodist_last_error()
+    pg2 = core.moodist_world_group(w, 2)
+    assert core.moodist_pg_reduce_scatter(pg2, ctypes.byref(fake(8)), ctypes.byref(fake(32)), 0, None, 0.0,
+                                          ctypes.byref(work)) != 0  # other size
+    pg3 = core.moodist_world_group(w, 3)
+    assert core.moodist_pg_reduce_scatter(pg3, ctypes.byref(fake(4)), ctypes.byref(fake(16)), 4, None, 0.0,
+                                          ctypes.byref(work)) != 0  # other reduction
+    core.moodist_world_destroy(w)
+
+
+# ---------------- planner: C++ against the oracle's restatement ----------------
+
+@pytest.mark.parametrize("case", list(_cases()), ids=lambda c: c[0])
+def test_cpp_planner_matches_oracle_planner(case):
+    _, size, shape, dt, inputs, outputs = case
+    tdt = {np.dtype(np.float32): torch.float32, np.dtype(np.float64): torch.float64, np.dtype(np.int32): torch.int32,
+           np.dtype(np.int64): torch.int64, np.dtype(np.int16): torch.int16,
+           np.dtype(np.uint16): torch.bfloat16}[np.dtype(dt)]
+    want = planner.plan(size, shape, np.dtype(dt).itemsize, inputs, outputs)
+    world = moodist_amd.LocalWorld(size, 0)
+    for r, pg in enumerate(world):
+        got = pg.compile_op_full(shape, tdt, inputs, outputs).plan()
+        d = want[r]
+        assert got["reads"] == [(x.rank, x.inputIndex, x.outputIndex, x.inputOffset, x.outputOffset, x.bytes)
+                                for x in d.reads]
+        assert got["inputCopies"] == [(c.index, c.offset, c.shape) for c in d.inputCopies]
+        assert got["outputCopies"] == [(c.index, c.offset, c.shape) for c in d.outputCopies]
+        assert got["inputs"] == d.inputs and got["outputs"] == d.outputs
+
+
+def test_cpp_planner_random_boxes_match_oracle():
+    rng = np.random.RandomState(7)
+    for trial in range(60):
+        ndim = rng.randint(1, 4)
+        shape = [int(rng.randint(2, 9)) for _ in range(ndim)]
+        size = int(rng.randint(2, 5))
+        # inputs: split one random dimension into `size` slabs (covers the tensor); outputs: random boxes
+        d = int(rng.randint(0, ndim))
+        cuts = sorted(set([0, shape[d]] + [int(x) for x in rng.randint(0, shape[d] + 1, size - 1)]))
+        inputs = []
+        for i in range(len(cuts) - 1):
+            off = [0] * ndim
+            shp = list(shape)
+            off[d], shp[d] = cuts[i], cuts[i + 1] - cuts[i]
+            inputs.append((i % size, off, shp))
+        outputs = []
+        for r in range(size):
+            off = [int(rng.randint(0, s)) for s in shape]
+            shp = [int(rng.randint(1, s - o + 1)) for s, o in zip(shape, off)]
+            outputs.append((r, off, shp))
+        want = planner.plan(size, shape, 2, inputs, outputs)
+        world = moodist_amd.LocalWorld(size, 0)
+        for r, pg in enumerate(world):
+            got = pg.compile_op_full(shape, torch.bfloat16, inputs, outputs).plan()
+            assert got["reads"] == [(x.rank, x.inputIndex, x.outputIndex, x.inputOffset, x.outputOffset, x.bytes)
+                                    for x in want[r].reads], (trial, r)
+            assert got["inputCopies"] == [(c.index, c.offset, c.shape) for c in want[r].inputCopies]
+            assert got["outputCopies"] == [(c.index, c.offset, c.shape) for c in want[r].outputCopies]
+
+
+def test_planner_errors():
+    world = moodist_amd.LocalWorld(2, 0)
+    pg = world.groups[0]
+    with pytest.raises(RuntimeError, match="could not find input for all output elements"):
+        pg.compile_op_full([8], torch.float32, [(0, [0], [4])], [(1, [0], [8])])
+    with pytest.raises(RuntimeError, match="ndim 11 is too large and not supported"):
+        pg.compile_op_full([1] * 11, torch.float32, [], [])
+    with pytest.raises(RuntimeError, match="outside the group"):
+        pg.compile_op_full([8], torch.float32, [(2, [0], [8])], [])
+    with pytest.raises(RuntimeError, match="listed largest first"):
+        pg.compile_op_full([8], torch.float32, [(0, [0], [8])], [(1, [0], [2]), (1, [2], [6])])
+
+
+def test_custom_op_argument_checks():
+    world = moodist_amd.LocalWorld(2, 0)
+    op = world.groups[0].compile_op_full([4], torch.float32, [(0, [0], [4])], [(1, [0], [4])])
+    x = torch.zeros(4)
+    with pytest.raises(RuntimeError, match="custom op expected different number of inputs"):
+        op([], [])
+    with pytest.raises(RuntimeError, match="custom op expected different number of outputs"):
+        op([x], [x])
+    with pytest.raises(RuntimeError, match="custom op input has wrong size"):
+        op([torch.zeros(5)], [])
+    with pytest.raises(RuntimeError, match="Got a non-contiguous tensor"):
+        op([torch.zeros(4, 2)[:, 0]], [])
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        op([x], [])
+
+
+# ---------------- compile_op front end (py/moodist/compile.py:104-264) ----------------
+
+def test_compile_op_validation_messages():
+    world = moodist_amd.LocalWorld(2, 0)
+    g = world.groups[0]
+    f32 = torch.float32
+    with pytest.raises(ValueError, match="shape must be provided"):
+        moodist_amd.compile_op(g, dtype=f32)
+    with pytest.raises(ValueError, match="dtype must be provided"):
+        moodist_amd.compile_op(g, shape=[4])
+    with pytest.raises(TypeError, match="dtype must be a torch.dtype"):
+        moodist_amd.compile_op(g, shape=[4], dtype="float32")
+    with pytest.raises(TypeError, match=r"shape\[0\] must be an int"):
+        moodist_amd.compile_op(g, shape=[4.0], dtype=f32)
+    with pytest.raises(TypeError, match="'offset' must be a tuple or list"):
+        moodist_amd.compile_op(g, shape=[4], dtype=f32, inputs=[{"offset": 0, "shape": [4]}])
+    with pytest.raises(TypeError, match="must be a dict"):
+        moodist_amd.compile_op(g, shape=[4], dtype=f32, inputs=[[0, 4]])
+    with pytest.raises(ValueError, match="'shape' is missing"):
+        moodist_amd.compile_op(g, shape=[4], dtype=f32, inputs=[{"offset": [0]}])
+    with pytest.raises(ValueError, match="expected 'offset' with 1 dimensions, but got 2"):
+        moodist_amd.compile_op(g, shape=[4], dtype=f32, inputs=[{"offset": [0, 0], "shape": [4]}])
+    with pytest.raises(TypeError, match=r"shape\[0\] must be an int"):
+        moodist_amd.compile_op(g, shape=[4], dtype=f32, inputs=[{"offset": [0], "shape": [4.0]}])
+
+
+def test_compile_op_waits_for_every_rank_and_checks_agreement():
+    world = moodist_amd.LocalWorld(2, 0)
+    op0 = moodist_amd.compile_op(world.groups[0], shape=[4], dtype=torch.float32,
+                                 inputs=[{"offset": [0], "shape": [4]}])
+    with pytest.raises(RuntimeError, match="1 of 2 ranks have called compile_op"):
+        op0.plan()
+    moodist_amd.compile_op(world.groups[1], shape=[4], dtype=torch.float32, outputs=[{"offset": [0], "shape": [4]}])
+    assert op0.plan()["inputs"] == [16]
+    a = moodist_amd.compile_op(world.groups[0], shape=[4], dtype=torch.float32)
+    moodist_amd.compile_op(world.groups[1], shape=[8], dtype=torch.float32)
+    with pytest.raises(ValueError, match="Ranks specified different shapes"):
+        a.plan()
+    a = moodist_amd.compile_op(world.groups[0], shape=[4], dtype=torch.float32)
+    moodist_amd.compile_op(world.groups[1], shape=[4], dtype=torch.float64)
+    with pytest.raises(ValueError, match="Ranks specified different dtypes"):
+        a.plan()
+
+
+def test_shard_box_matches_oracle_restatement():
+    from moodist_amd.compile import shard_box
+
+    for n in (1, 7, 8, 9, 65):
+        for k in (1, 2, 3, 8):
+            for c in range(k):
+                assert shard_box([n, 5], [k], [c], [0]) == planner.shard_box([n, 5], [k], [c], [0])
+    assert shard_box([8, 8], [2, 4], [1, 3], [0, 1]) == ([4, 6], [4, 2])
+    assert shard_box([8, 8], [2], None, [0]) == ([0, 0], [0, 0])
+
+
+def test_options_object():
+    world = moodist_amd.LocalWorld(2, 0)
+    pg = world.groups[1]
+    assert pg.options().prefer_kernel_less is False and pg.options().num_chunks is None
+    pg.options().prefer_kernel_less = True
+    pg.options().num_chunks = 4
+    assert pg.get_prefer_kernel_less() and pg.options().num_chunks == 4
+    with pg.options(num_chunks=2, force_kernel_less=True) as same:
+        assert same is pg and pg.options().num_chunks == 2 and pg.options().force_kernel_less
+    assert pg.options().num_chunks == 4 and not pg.options().force_kernel_less
+    pg.options().num_chunks = None
+    assert pg._get_option("num_chunks") == -1
+    with pytest.raises(AttributeError):
+        pg.options().bogus
+    with pytest.raises(ValueError):
+        pg.options(bogus=1)
+
+
+def test_process_group_is_a_c10d_process_group():
+    import torch.distributed as dist
+
+    world = moodist_amd.LocalWorld(3, 0)
+    for r, pg in enumerate(world):
+        assert isinstance(pg.c10d, dist.ProcessGroup)
+        assert pg.rank() == r and pg.size() == 3
+        assert pg.moodist_name() == "moodist-local-%d-of-3" % r
+    with pytest.raises(RuntimeError, match="send is not supported"):
+        world.groups[0].send([torch.zeros(1)], 1, 0)

@@ -1,0 +1,283 @@
+"""The process-group operator surface on the GPU, written the way the reference's own tests
+are (tests/test_processgroup.py, tests/test_stress.py): every rank of an 8-rank group makes the
+call, here from one process.  Results are also checked against the CPU oracle, rank by rank, with
+the fold starting at the rank itself."""
+
+import numpy as np
+import pytest
+import torch
+import torch.distributed as dist
+
+import moodist_amd
+import oracle
+from util import TORCH_TO_CODE, bits, random_sources, same_bits
+
+pytestmark = pytest.mark.gpu
+P = 8
+
+
+@pytest.fixture()
+def world(dev):
+    return moodist_amd.LocalWorld(P, dev)
+
+
+def each_rank(world, fn):
+    """Runs fn(rank, pg) for every rank (the body of an SPMD test), then waits on all works."""
+    works = [fn(r, pg) for r, pg in enumerate(world)]
+    for w in works:
+        if w is not None:
+            w.wait()
+    torch.cuda.synchronize()
+
+
+def test_pg_creation(world):
+    # reference tests/test_processgroup.py:13-18
+    for r, pg in enumerate(world):
+        assert pg.rank() == r and pg.size() == P
+
+
+@pytest.mark.parametrize("kernel_less", [False, True])
+def test_pg_allgather_base(world, dev, kernel_less):
+    # reference tests/test_processgroup.py:21-48 (kernel and kernel-less modes)
+    chunk = 4
+    ins = [torch.full((chunk,), float(r), device=dev) for r in range(P)]
+    outs = [torch.zeros(chunk * P, device=dev) for _ in range(P)]
+    for pg in world:
+        pg.options().force_kernel_less = kernel_less
+    each_rank(world, lambda r, pg: pg._allgather_base(outs[r], ins[r]))
+    expected = torch.cat([torch.full((chunk,), float(r), device=dev) for r in range(P)])
+    for r in range(P):
+        assert torch.equal(outs[r], expected)
+
+
+def test_pg_reduce_scatter_base(world, dev):
+    # reference tests/test_processgroup.py:51-79
+    chunk = 4
+    ins = [torch.full((chunk * P,), float(r + 1), device=dev) for r in range(P)]
+    outs = [torch.zeros(chunk, device=dev) for _ in range(P)]
+    each_rank(world, lambda r, pg: pg._reduce_scatter_base(outs[r], ins[r]))
+    for r in range(P):
+        assert torch.equal(outs[r], torch.full((chunk,), P * (P + 1) / 2, device=dev))
+
+
+def test_pg_allgather_varying_data(world, dev):
+    # reference tests/test_processgroup.py:82-109
+    chunk = 8
+    ins = [torch.arange(r * 100, r * 100 + chunk, device=dev, dtype=torch.float32) for r in range(P)]
+    outs = [torch.zeros(chunk * P, device=dev) for _ in range(P)]
+    each_rank(world, lambda r, pg: pg._allgather_base(outs[r], ins[r]))
+    for q in range(P):
+        for r in range(P):
+            assert torch.equal(outs[q][r * chunk:(r + 1) * chunk], ins[r])
+
+
+def test_pg_large_allgather(world, dev):
+    # reference tests/test_processgroup.py:112-146
+    chunk = 256 * 1024
+    ins = []
+    for r in range(P):
+        torch.manual_seed(r + 42)
+        ins.append(torch.randn(chunk).to(dev))
+    outs = [torch.zeros(chunk * P, device=dev) for _ in range(P)]
+    each_rank(world, lambda r, pg: pg._allgather_base(outs[r], ins[r]))
+    for q in range(P):
+        for r in range(P):
+            torch.manual_seed(r + 42)
+            assert torch.equal(outs[q][r * chunk:(r + 1) * chunk].cpu(), torch.randn(chunk))
+
+
+def test_pg_allreduce_sum_and_varying(world, dev):
+    # reference tests/test_processgroup.py:201-248
+    ts = [torch.full((8,), float(r + 1), device=dev) for r in range(P)]
+    each_rank(world, lambda r, pg: pg.allreduce([ts[r]]))
+    for t in ts:
+        assert torch.equal(t, torch.full((8,), P * (P + 1) / 2, device=dev))
+    ts = [torch.arange(r, r + 4, device=dev, dtype=torch.float32) for r in range(P)]
+    each_rank(world, lambda r, pg: pg.allreduce([ts[r]]))
+    want = torch.tensor([P * (P - 1) / 2 + i * P for i in range(4)], device=dev)
+    for t in ts:  # 4 elements over 8 ranks: the padded-temporary path
+        assert torch.equal(t, want)
+
+
+def test_allreduce_matches_oracle_composition(world, dev):
+    # allreduce = reduce_scatter into the rank's own chunk + all_gather (core/processgroup.cc:1674-1722):
+    # chunk c of the result is the fold that starts at rank c
+    for n in (8 * 1000, 8 * 1000 + 3):
+        srcs = random_sources(P, n, torch.float32, seed=n)
+        padded = (n + P - 1) // P * P
+        chunk = padded // P
+        full = [torch.cat([s, torch.zeros(padded - n)]) for s in srcs]
+        want = np.concatenate([oracle.reduce([f[c * chunk:(c + 1) * chunk].numpy() for f in full], c, oracle.DT_F32,
+                                             oracle.OP_SUM) for c in range(P)])[:n]
+        ts = [s.to(dev) for s in srcs]
+        each_rank(world, lambda r, pg: pg.allreduce([ts[r]]))
+        for t in ts:
+            assert same_bits(bits(t), want)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.int32, torch.int64, torch.bfloat16], ids=str)
+def test_reduce_scatter_every_rank_matches_oracle_in_its_own_order(world, dev, dtype):
+    n = 5000 + 3
+    srcs = random_sources(P, P * n, dtype, seed=21)
+    ins = [s.to(dev) for s in srcs]
+    for name, c10d_op, code in (("SUM", dist.ReduceOp.SUM, oracle.OP_SUM), ("MIN", dist.ReduceOp.MIN, oracle.OP_MIN),
+                                ("MAX", dist.ReduceOp.MAX, oracle.OP_MAX), ("AVG", dist.ReduceOp.AVG, oracle.OP_AVG)):
+        if code == oracle.OP_AVG and not dtype.is_floating_point:
+            continue
+        outs = [torch.zeros(n, dtype=dtype, device=dev) for _ in range(P)]
+        opts = dist.ReduceScatterOptions()
+        opts.reduceOp = c10d_op
+        each_rank(world, lambda r, pg: pg._reduce_scatter_base(outs[r], ins[r], opts))
+        scale = float(np.float32(1.0) / np.float32(P))
+        for q in range(P):
+            want = oracle.reduce([bits(s[q * n:(q + 1) * n]) for s in srcs], q, TORCH_TO_CODE[dtype], code, scale)
+            assert same_bits(bits(outs[q]), want), (name, q)
+
+
+def test_reduce_scatter_premul_sum(world, dev):
+    n = 4096
+    srcs = random_sources(P, P * n, torch.float32, seed=5)
+    ins = [s.to(dev) for s in srcs]
+    outs = [torch.zeros(n, device=dev) for _ in range(P)]
+    opts = dist.ReduceScatterOptions()
+    opts.reduceOp = dist._make_nccl_premul_sum(0.37)
+    each_rank(world, lambda r, pg: pg._reduce_scatter_base(outs[r], ins[r], opts))
+    f = float(np.float32(0.37))
+    for q in range(P):
+        want = oracle.reduce([s[q * n:(q + 1) * n].numpy() for s in srcs], q, oracle.DT_F32, oracle.OP_PREMUL_SUM, f)
+        assert same_bits(bits(outs[q]), want)
+
+
+def test_unsupported_requests_raise(world, dev):
+    x = torch.zeros(P * 4, device=dev)
+    o = torch.zeros(4, device=dev)
+    opts = dist.ReduceScatterOptions()
+    opts.reduceOp = dist.ReduceOp.PRODUCT
+    with pytest.raises(RuntimeError, match="Unsupported reduce operation"):
+        world.groups[0]._reduce_scatter_base(o, x, opts)
+    with pytest.raises(RuntimeError, match="Unsupported dtype for reduce operation"):
+        world.groups[0]._reduce_scatter_base(o.to(torch.uint8), x.to(torch.uint8))
+    with pytest.raises(RuntimeError, match="must be contiguous"):
+        world.groups[0]._reduce_scatter_base(o, torch.zeros(P * 4, 2, device=dev)[:, 0])
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        world.groups[0]._reduce_scatter_base(o.cpu(), x.cpu())
+
+
+def test_work_before_all_ranks_called_is_incomplete(world, dev):
+    ins = [torch.ones(P * 4, device=dev) for _ in range(P)]
+    outs = [torch.zeros(4, device=dev) for _ in range(P)]
+    works = [world.groups[r]._reduce_scatter_base(outs[r], ins[r]) for r in range(P - 1)]
+    assert not works[0].is_completed()
+    with pytest.raises(RuntimeError, match="7 of 8 have"):
+        works[0].wait()
+    last = world.groups[P - 1]._reduce_scatter_base(outs[P - 1], ins[P - 1])
+    for w in works + [last]:
+        assert w.is_completed()
+        w.wait()
+    torch.cuda.synchronize()
+    assert all(torch.equal(o, torch.full((4,), float(P), device=dev)) for o in outs)
+
+
+def test_one_ranks_share_with_staged_peers(world, dev):
+    # the benchmark's shape: only rank 0 wants its output; ranks 1..7 are staged contributions
+    n = 100000
+    srcs = random_sources(P, P * n, torch.float32, seed=8)
+    ins = [s.to(dev) for s in srcs]
+    out = torch.zeros(n, device=dev)
+    for r in range(1, P):
+        world.groups[r].stage_input("reduce_scatter", ins[r])
+    world.groups[0]._reduce_scatter_base(out, ins[0]).wait()
+    torch.cuda.synchronize()
+    want = oracle.reduce([s[:n].numpy() for s in srcs], 0, oracle.DT_F32, oracle.OP_SUM)
+    assert same_bits(bits(out), want)
+    # and the gather
+    shards = [s[:n].contiguous().to(dev) for s in srcs]
+    g = torch.zeros(P * n, device=dev)
+    for r in range(1, P):
+        world.groups[r].stage_input("all_gather", shards[r])
+    world.groups[0]._allgather_base(g, shards[0]).wait()
+    torch.cuda.synchronize()
+    assert torch.equal(g.cpu(), torch.cat([s[:n] for s in srcs]))
+
+
+def test_coalesced_variants(world, dev):
+    sizes = (4, 1000, 33)
+    ins = [[torch.full((n,), float(r + 1), device=dev) for n in sizes] for r in range(P)]
+    outs = [[torch.zeros(n * P, device=dev) for n in sizes] for _ in range(P)]
+    each_rank(world, lambda r, pg: pg.allgather_into_tensor_coalesced(outs[r], ins[r]))
+    for r in range(P):
+        for k, n in enumerate(sizes):
+            assert torch.equal(outs[r][k], torch.arange(1, P + 1, device=dev).float().repeat_interleave(n))
+    rins = [[torch.full((n * P,), float(r + 1), device=dev) for n in sizes] for r in range(P)]
+    routs = [[torch.zeros(n, device=dev) for n in sizes] for _ in range(P)]
+    each_rank(world, lambda r, pg: pg.reduce_scatter_tensor_coalesced(routs[r], rins[r]))
+    for r in range(P):
+        for k, n in enumerate(sizes):
+            assert torch.equal(routs[r][k], torch.full((n,), 36.0, device=dev))
+
+
+def test_ranks_on_different_streams(world, dev):
+    # each rank posts on its own stream; the launches must still see every rank's input
+    n = 1 << 20
+    streams = [torch.cuda.Stream(device=dev) for _ in range(P)]
+    ins, outs = [None] * P, [None] * P
+    torch.cuda.synchronize()
+    works = []
+    for r, pg in enumerate(world):
+        with torch.cuda.stream(streams[r]):
+            ins[r] = torch.full((P * n,), float(r + 1), device=dev)  # produced on the rank's own stream
+            outs[r] = torch.zeros(n, device=dev)
+            works.append(pg._reduce_scatter_base(outs[r], ins[r]))
+    for w in works:
+        w.wait()
+    for r in range(P):
+        streams[r].synchronize()
+        assert torch.equal(outs[r], torch.full((n,), 36.0, device=dev))
+
+
+# ---- reference tests/test_stress.py ----
+
+def test_stress_rapid_collectives(world, dev):
+    # :16-82: 100 iterations, pre-allocated tensors, tight loop
+    iters, chunk = 100, 256
+    ag_in = [[torch.full((chunk,), float(r), device=dev) for _ in range(iters)] for r in range(P)]
+    ag_out = [[torch.zeros(chunk * P, device=dev) for _ in range(iters)] for _ in range(P)]
+    rs_in = [[torch.full((chunk * P,), float(r + 1), device=dev) for _ in range(iters)] for r in range(P)]
+    rs_out = [[torch.zeros(chunk, device=dev) for _ in range(iters)] for _ in range(P)]
+    for i in range(iters):
+        for r, pg in enumerate(world):
+            pg._allgather_base(ag_out[r][i], ag_in[r][i])
+        for r, pg in enumerate(world):
+            pg._reduce_scatter_base(rs_out[r][i], rs_in[r][i])
+    torch.cuda.synchronize()
+    want = torch.arange(P, device=dev).float().repeat_interleave(chunk)
+    for r in range(P):
+        for i in range(iters):
+            assert torch.equal(ag_out[r][i], want)
+            assert torch.equal(rs_out[r][i], torch.full((chunk,), 36.0, device=dev))
+
+
+def test_stress_varying_sizes(world, dev):
+    # :235-280
+    for size in (1, 7, 64, 255, 1024, 4096, 65536):
+        ag_in = [torch.full((size,), float(r), device=dev) for r in range(P)]
+        ag_out = [torch.zeros(size * P, device=dev) for _ in range(P)]
+        rs_in = [torch.full((size * P,), float(r + 1), device=dev) for r in range(P)]
+        rs_out = [torch.zeros(size, device=dev) for _ in range(P)]
+        each_rank(world, lambda r, pg: pg._allgather_base(ag_out[r], ag_in[r]))
+        each_rank(world, lambda r, pg: pg._reduce_scatter_base(rs_out[r], rs_in[r]))
+        for q in range(P):
+            for r in range(P):
+                assert (ag_out[q][r * size:(r + 1) * size] == float(r)).all()
+            assert torch.equal(rs_out[q], torch.full((size,), 36.0, device=dev))
+
+
+def test_stress_large_tensors(world, dev):
+    # :283-313: 4 MiB per rank
+    chunk = 1024 * 1024
+    ins = [torch.full((chunk,), float(r), device=dev) for r in range(P)]
+    outs = [torch.zeros(chunk * P, device=dev) for _ in range(P)]
+    for _ in range(3):
+        each_rank(world, lambda r, pg: pg._allgather_base(outs[r], ins[r]))
+    for q in range(P):
+        assert torch.equal(outs[q], torch.arange(P, device=dev).float().repeat_interleave(chunk))
