@@ -299,8 +299,7 @@ public:
       // the padded temporary the reference allocates through torch (core/processgroup.cc:1694-1697)
       scratch = at::empty({(n + size - 1) / size * size}, t.options());
       s = describe(scratch);
-      scratch.record_stream(c10::hip::getCurrentHIPStream(t.device().index()));
-      keep(scratch);
+      keep(scratch); // allocated, used and later reused on this same stream, so stream order protects it
     }
     moodist_work* w = nullptr;
     check(core.moodist_pg_allreduce(pg_, &d, scratch.defined() ? &s : nullptr, reduce_op_code(opts.reduceOp),
