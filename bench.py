@@ -23,11 +23,13 @@ INFINITY_CACHE_BYTES = 256 << 20
 
 
 def build_workload(name, torch, abi, dev):
-    """Returns (describe, algorithmic_bytes, nsets, launch(i), check()) for a named workload.
+    """Returns (describe, algorithmic_bytes, launch(i), check(), kernel name) for a named workload.
     Every workload rotates over enough distinct buffer sets that their footprint exceeds twice
     the 256 MB Infinity Cache, so no launch finds its operands cached by an earlier one."""
-    st = torch.cuda.current_stream().cuda_stream
     L = abi.lib()
+
+    def current():
+        return torch.cuda.current_stream().cuda_stream
 
     def nsets_for(set_bytes):
         return max(2, -(-2 * INFINITY_CACHE_BYTES // set_bytes) + 1)
@@ -61,7 +63,7 @@ def build_workload(name, torch, abi, dev):
 
         def launch(i):
             k = i % nsets
-            rc = L.mdh_reduce(tabs[k], P, 0, outs[k].data_ptr(), N, code, op, scale, st)
+            rc = L.mdh_reduce(tabs[k], P, 0, outs[k].data_ptr(), N, code, op, scale, current())
             if rc:
                 abi.check(rc)
 
@@ -83,6 +85,7 @@ def build_workload(name, torch, abi, dev):
                 "dtype": str(tdt).replace("torch.", ""), "fold_first": 0, "buffer_sets": nsets}
         return desc, set_bytes, launch, check, "reduce_vec_kernel"
 
+
     if name == "allgather_bf16_p8" or name == "allgather_bf16_p8_strided":
         P, n = 8, 16777216
         rows = cols = 4096
@@ -101,9 +104,9 @@ def build_workload(name, torch, abi, dev):
             k = i % nsets
             if pad:
                 rc = L.mdh_gather(tabs[k], P, outs[k].data_ptr(), cols * 2, rows, cols * 2, (cols + pad) * 2,
-                                  rows * (cols + pad) * 2, st)
+                                  rows * (cols + pad) * 2, current())
             else:
-                rc = L.mdh_gather(tabs[k], P, outs[k].data_ptr(), n * 2, 1, n * 2, n * 2, n * 2, st)
+                rc = L.mdh_gather(tabs[k], P, outs[k].data_ptr(), n * 2, 1, n * 2, n * 2, n * 2, current())
             if rc:
                 abi.check(rc)
 
@@ -150,7 +153,7 @@ def build_workload(name, torch, abi, dev):
             tabs.append((abi.Box * P)(*boxes))
 
         def launch(i):
-            rc = L.mdh_copy_boxes(tabs[i % nsets], P, isz, st)
+            rc = L.mdh_copy_boxes(tabs[i % nsets], P, isz, current())
             if rc:
                 abi.check(rc)
 

@@ -133,6 +133,63 @@ __global__ __launch_bounds__(kBlock) void copy_boxes_kernel(CopyArgs a) {
   }
 }
 
+// Contiguous segments (the shards of a dense all-gather, or any box that
+// collapses to one run): no per-lane index arithmetic at all.  A tile is
+// kBlock*U consecutive 16-byte vectors of one segment, addressed through a
+// buffer descriptor based at the tile (wave-uniform), so a lane needs one
+// 32-bit offset and the ragged last tile is clipped by the address unit.
+constexpr int kMaxSegments = 64;
+
+struct FlatArgs {
+  const char* src[kMaxSegments];
+  char* dst[kMaxSegments];
+  uint32_t tile_end[kMaxSegments]; // cumulative tiles; unused entries are ~0
+  uint64_t bytes[kMaxSegments];    // multiples of 16
+  uint32_t nsegs;
+  uint32_t total_tiles;
+  uint32_t tiles_per_seg; // non-zero when every segment has the same tile count
+};
+static_assert(sizeof(FlatArgs) <= 4096, "kernel arguments are limited to 4 KiB");
+
+template<int U>
+__global__ __launch_bounds__(kBlock) void copy_flat_kernel(FlatArgs a) {
+  constexpr uint32_t tile_bytes = kBlock * U * 16;
+  const uint32_t lane_byte = threadIdx.x * 16;
+  for (uint32_t tile = blockIdx.x; tile < a.total_tiles; tile += gridDim.x) {
+    uint32_t seg, local;
+    if (a.tiles_per_seg) {
+      seg = tile / a.tiles_per_seg;
+      local = tile - seg * a.tiles_per_seg;
+    } else {
+      seg = 0;
+      uint32_t start = 0;
+#pragma unroll
+      for (int k = 0; k < kMaxSegments - 1; ++k) {
+        const uint32_t e = a.tile_end[k];
+        if (tile >= e) {
+          ++seg;
+          start = e;
+        }
+      }
+      local = tile - start;
+    }
+    const uint64_t off = (uint64_t)local * tile_bytes;
+    const uint64_t left = a.bytes[seg] - off;
+    const uint32_t n = left < tile_bytes ? (uint32_t)left : tile_bytes;
+    const __amdgpu_buffer_rsrc_t rs = tile_rsrc(a.src[seg] + off, n);
+    const __amdgpu_buffer_rsrc_t rd = tile_rsrc(a.dst[seg] + off, n);
+    u32x4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      v[u] = tile_load(rs, lane_byte + (uint32_t)u * (kBlock * 16));
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      tile_store(rd, lane_byte + (uint32_t)u * (kBlock * 16), v[u]);
+    }
+  }
+}
+
 // ---- host side: reduce a box to the kernel's form ----
 
 struct HostBox {
@@ -156,7 +213,78 @@ int vec_width(const HostBox& h) {
 struct Launcher {
   hipStream_t stream;
   std::vector<BoxDesc> pending[5]; // by log2(VEC)
+  struct Segment {
+    const char* src;
+    char* dst;
+    uint64_t bytes;
+  };
+  std::vector<Segment> flat; // 16-byte aligned contiguous runs
   int rc = MDH_OK;
+
+  void flush_flat() {
+    const Tuning& t = tuning();
+    const int U = t.copy_unroll;
+    const uint64_t tile_bytes = (uint64_t)kBlock * U * 16;
+    size_t i = 0;
+    while (i < flat.size()) {
+      FlatArgs a;
+      a.nsegs = 0;
+      uint64_t tiles = 0;
+      uint64_t first_tiles = 0;
+      bool equal = true;
+      while (i < flat.size() && a.nsegs < (uint32_t)kMaxSegments) {
+        const Segment& g = flat[i];
+        const uint64_t n = (g.bytes + tile_bytes - 1) / tile_bytes;
+        if (tiles + n > 0x7fffffffull) {
+          break; // a segment is at most 2^30 bytes, so the next launch always makes progress
+        }
+        if (a.nsegs == 0) {
+          first_tiles = n;
+        }
+        equal = equal && n == first_tiles;
+        tiles += n;
+        a.src[a.nsegs] = g.src;
+        a.dst[a.nsegs] = g.dst;
+        a.bytes[a.nsegs] = g.bytes;
+        a.tile_end[a.nsegs] = (uint32_t)tiles;
+        ++a.nsegs;
+        ++i;
+      }
+      for (uint32_t k = a.nsegs; k < (uint32_t)kMaxSegments; ++k) {
+        a.src[k] = nullptr, a.dst[k] = nullptr, a.bytes[k] = 0;
+        a.tile_end[k] = 0xffffffffu;
+      }
+      a.total_tiles = (uint32_t)tiles;
+      a.tiles_per_seg = equal ? (uint32_t)first_tiles : 0;
+      if (tiles == 0) {
+        continue;
+      }
+      uint32_t grid = a.total_tiles;
+      if (t.copy_max_blocks > 0 && grid > (uint32_t)t.copy_max_blocks) {
+        grid = (uint32_t)t.copy_max_blocks;
+      }
+      dim3 g(grid), b(kBlock);
+      switch (U) {
+      case 1:
+        hipLaunchKernelGGL((copy_flat_kernel<1>), g, b, 0, stream, a);
+        break;
+      case 2:
+        hipLaunchKernelGGL((copy_flat_kernel<2>), g, b, 0, stream, a);
+        break;
+      case 4:
+        hipLaunchKernelGGL((copy_flat_kernel<4>), g, b, 0, stream, a);
+        break;
+      default:
+        hipLaunchKernelGGL((copy_flat_kernel<8>), g, b, 0, stream, a);
+        break;
+      }
+      int r = check_launch("copy_flat_kernel");
+      if (r != MDH_OK) {
+        rc = r;
+      }
+    }
+    flat.clear();
+  }
 
   template<int VEC>
   void launch(CopyArgs& a) {
@@ -250,6 +378,7 @@ struct Launcher {
   }
 
   void flush() {
+    flush_flat();
     for (int lg = 4; lg >= 0; --lg) {
       flush_class(lg);
     }
@@ -321,6 +450,10 @@ struct Launcher {
           p.run = std::min(max_run, h.run - off);
           add(p);
         }
+        return;
+      }
+      if (vec_width(h) == 16) {
+        flat.push_back(Segment{h.src, h.dst, (uint64_t)h.run});
         return;
       }
       emit(h);

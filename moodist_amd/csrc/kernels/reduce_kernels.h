@@ -315,9 +315,16 @@ __global__ __launch_bounds__(kBlock) void reduce_elem_kernel(ReduceArgs a) {
 template<typename T, int F, int NSRC>
 int launch_vec(const ReduceArgs& a, hipStream_t stream) {
   const Tuning& t = tuning();
-  // 16-bit types widen every vector to eight fp32 accumulators: four sub-tiles
-  // would not fit the register file, so they stop at two.
-  const int U = (sizeof(typename Traits<T>::elem_t) == 2 && t.reduce_unroll > 2) ? 2 : t.reduce_unroll;
+  // 16-bit types widen every vector to eight fp32 accumulators: two sub-tiles at most, and one
+  // when sixteen sources are unrolled (their loads alone fill the register budget; measured
+  // 6.4 TB/s against 5.3 TB/s with two on the bf16 sixteen-source workload).
+  int U = t.reduce_unroll;
+  if (sizeof(typename Traits<T>::elem_t) == 2) {
+    U = U > 2 ? 2 : U;
+    if (NSRC >= 16) {
+      U = 1;
+    }
+  }
   const uint64_t tile_vecs = (uint64_t)kBlock * U;
   uint64_t ntiles = (a.nvec + tile_vecs - 1) / tile_vecs;
   if (ntiles == 0) {
