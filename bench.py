@@ -20,6 +20,8 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 INFINITY_CACHE_BYTES = 256 << 20
+# (65571.59 KiB x 1.99901 fetched + 16384.00 KiB x 0.99914 written) per launch of the fp32 P=8 reduction
+MEASURED_TRAFFIC_BYTES = {"reduce_fp32_p8": 150986752}
 
 
 def build_workload(name, torch, abi, dev):
@@ -270,7 +272,9 @@ def main():
             "unit": "GB/s",
             "frac": round(gbs / HBM_PEAK_GBS, 4),
             "algorithmic_bytes_per_launch": alg_bytes,
-            "traffic": None,
+            # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by the
+            # same counter's reading on a copy of known size (recorded for the headline workload only)
+            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
         },
     }
     if not args.no_cpu_baseline and args.workload == "reduce_fp32_p8":
