@@ -162,7 +162,7 @@ constexpr int per_vec() {
 // buffer descriptor whose base is the tile's first byte (wave-uniform, in
 // SGPRs) and whose size is the bytes left in the tile: the lane offset is one
 // VGPR, and vectors past the end read as zero instead of needing a predicate.
-template<typename T, int F, int CNT, int U>
+template<typename T, int F, int CNT, int U, int MODE>
 __device__ __forceinline__ void fold_chunk(const ReduceArgs& a, int j0, uint64_t tile_byte, uint32_t tile_bytes,
     uint32_t lane_byte, typename Traits<T>::acc_t (&acc)[U][per_vec<T>()]) {
   using Tr = Traits<T>;
@@ -178,6 +178,10 @@ __device__ __forceinline__ void fold_chunk(const ReduceArgs& a, int j0, uint64_t
       v[k][u] = tile_load(rs, lane_byte + (uint32_t)u * (kBlock * 16));
     }
   }
+  // Every load of the chunk is issued before the first add: without this fence the
+  // instruction scheduler interleaves loads with arithmetic to save registers and keeps only
+  // about a dozen loads in flight per lane.
+  __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int k = 0; k < CNT; ++k) {
 #pragma unroll
@@ -187,7 +191,7 @@ __device__ __forceinline__ void fold_chunk(const ReduceArgs& a, int j0, uint64_t
 #pragma unroll
       for (int i = 0; i < N; ++i) {
         acc_t x = Tr::widen(e[i]);
-        if (a.mode == kPremul) {
+        if constexpr (MODE == kPremul) {
           x = Tr::premul(x, a.scale);
         }
         if (k == 0 && j0 == 0) {
@@ -220,7 +224,7 @@ __device__ __forceinline__ void reduce_one_elem(const ReduceArgs& a, int nsrc, u
   ((elem_t*)a.dst)[i] = Tr::template finish<F>(acc, a.mode, a.scale);
 }
 
-template<typename T, int F, int NSRC, int U>
+template<typename T, int F, int NSRC, int U, int MODE>
 __device__ __forceinline__ void reduce_tile(const ReduceArgs& a, int nsrc, uint64_t tile_byte, uint32_t tile_bytes) {
   using Tr = Traits<T>;
   using elem_t = typename Tr::elem_t;
@@ -234,50 +238,56 @@ __device__ __forceinline__ void reduce_tile(const ReduceArgs& a, int nsrc, uint6
     static_assert(NSRC % CH == 0, "unrolled source counts are multiples of the chunk");
 #pragma unroll
     for (int j0 = 0; j0 < NSRC; j0 += CH) {
-      fold_chunk<T, F, CH, U>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
+      fold_chunk<T, F, CH, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
     }
   } else {
     int j0 = 0;
     for (; nsrc - j0 >= CH; j0 += CH) {
-      fold_chunk<T, F, CH, U>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
+      fold_chunk<T, F, CH, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
     }
     switch (nsrc - j0) {
     case 1:
-      fold_chunk<T, F, 1, U>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
+      fold_chunk<T, F, 1, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
       break;
     case 2:
-      fold_chunk<T, F, 2, U>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
+      fold_chunk<T, F, 2, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
       break;
     case 3:
-      fold_chunk<T, F, 3, U>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
+      fold_chunk<T, F, 3, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
       break;
     case 4:
-      fold_chunk<T, F, 4, U>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
+      fold_chunk<T, F, 4, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
       break;
     case 5:
-      fold_chunk<T, F, 5, U>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
+      fold_chunk<T, F, 5, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
       break;
     case 6:
-      fold_chunk<T, F, 6, U>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
+      fold_chunk<T, F, 6, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
       break;
     case 7:
-      fold_chunk<T, F, 7, U>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
+      fold_chunk<T, F, 7, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
       break;
     default:
       break;
     }
   }
   const __amdgpu_buffer_rsrc_t rd = tile_rsrc((const char*)a.dst + tile_byte, tile_bytes);
+  u32x4 out[U];
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     elem_t e[N];
 #pragma unroll
     for (int i = 0; i < N; ++i) {
-      e[i] = Tr::template finish<F>(acc[u][i], a.mode, a.scale);
+      e[i] = Tr::template finish<F>(acc[u][i], MODE, a.scale);
     }
-    u32x4 out;
-    __builtin_memcpy(&out, e, 16);
-    tile_store(rd, lane_byte + (uint32_t)u * (kBlock * 16), out); // dropped by the hardware past the end
+    __builtin_memcpy(&out[u], e, 16);
+  }
+  // results in registers of their own, then the stores back to back (a shared data register
+  // would make each store wait for the one before it)
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    tile_store(rd, lane_byte + (uint32_t)u * (kBlock * 16), out[u]); // dropped by the hardware past the end
   }
 }
 
@@ -293,7 +303,15 @@ __global__ __launch_bounds__(kBlock) void reduce_vec_kernel(ReduceArgs a) {
   for (uint64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
     const uint64_t tile_byte = tile * tile_bytes;
     const uint64_t left = body_bytes - tile_byte;
-    reduce_tile<T, F, NSRC, U>(a, nsrc, tile_byte, (uint32_t)(left < tile_bytes ? left : tile_bytes));
+    const uint32_t n = (uint32_t)(left < tile_bytes ? left : tile_bytes);
+    // the mode is wave-uniform: one branch per tile keeps the scale multiplies out of the plain path
+    if (F != kSum || a.mode == kPlain) {
+      reduce_tile<T, F, NSRC, U, kPlain>(a, nsrc, tile_byte, n);
+    } else if (a.mode == kAvg) {
+      reduce_tile<T, F, NSRC, U, kAvg>(a, nsrc, tile_byte, n);
+    } else {
+      reduce_tile<T, F, NSRC, U, kPremul>(a, nsrc, tile_byte, n);
+    }
   }
   if (blockIdx.x == 0) {
     const uint64_t i = a.nvec * per_vec<T>() + threadIdx.x;
@@ -324,6 +342,8 @@ int launch_vec(const ReduceArgs& a, hipStream_t stream) {
     if (NSRC >= 16) {
       U = 1;
     }
+  } else if (U > 4 && NSRC != 8) {
+    U = 4; // eight sub-tiles exist only for the unrolled eight-source kernel (64 loads in flight)
   }
   const uint64_t tile_vecs = (uint64_t)kBlock * U;
   uint64_t ntiles = (a.nvec + tile_vecs - 1) / tile_vecs;
@@ -342,8 +362,12 @@ int launch_vec(const ReduceArgs& a, hipStream_t stream) {
     hipLaunchKernelGGL((reduce_vec_kernel<T, F, NSRC, 1>), g, b, 0, stream, a);
   } else if (U == 2) {
     hipLaunchKernelGGL((reduce_vec_kernel<T, F, NSRC, 2>), g, b, 0, stream, a);
-  } else {
+  } else if (U == 4) {
     hipLaunchKernelGGL((reduce_vec_kernel<T, F, NSRC, 4>), g, b, 0, stream, a);
+  } else {
+    if constexpr (NSRC == 8 && sizeof(typename Traits<T>::elem_t) >= 4) {
+      hipLaunchKernelGGL((reduce_vec_kernel<T, F, NSRC, 8>), g, b, 0, stream, a);
+    }
   }
   return check_launch("reduce_vec_kernel");
 }

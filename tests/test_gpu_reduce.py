@@ -48,7 +48,7 @@ def test_parity_all_ops_ragged_sizes(dev, dtype, P):
             assert same_bits(bits(out), want), (dtype, P, n, op, first)
 
 
-@pytest.mark.parametrize("unroll", [1, 2, 4])
+@pytest.mark.parametrize("unroll", [1, 2, 4, 8])
 @pytest.mark.parametrize("max_blocks", [0, 3, 256])
 def test_parity_under_every_launch_shape(dev, unroll, max_blocks):
     old = abi.get_tuning("reduce_unroll"), abi.get_tuning("reduce_max_blocks")
@@ -56,7 +56,7 @@ def test_parity_under_every_launch_shape(dev, unroll, max_blocks):
         abi.set_tuning("reduce_unroll", unroll)
         abi.set_tuning("reduce_max_blocks", max_blocks)
         for dtype in (torch.float32, torch.bfloat16, torch.int64):
-            for P, n in ((8, 300000 + 3), (16, 65536), (5, 12345)):
+            for P, n in ((8, 300000 + 3), (8, 8192 * 4 + 4), (16, 65536), (5, 12345)):
                 srcs = random_sources(P, n, dtype, seed=n + P)
                 want = oracle.reduce([bits(s) for s in srcs], 1, TORCH_TO_CODE[dtype], oracle.OP_SUM)
                 out = torch.zeros(n, dtype=dtype, device=dev)
