@@ -239,6 +239,7 @@ def main():
     e0.record()  # on torch's current stream, the stream every launch above and below uses
     for i in range(args.steps):
         launch(i)
+    enqueue_ms = (time.perf_counter() - t0) * 1e3
     e1.record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
@@ -264,6 +265,7 @@ def main():
         "config": desc,
         "percent_of_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),
         "host_wall_ms_per_step": round(wall_ms / args.steps, 6),
+        "host_enqueue_ms_per_step": round(enqueue_ms / args.steps, 6),
         "roofline": {
             "bound": "hbm",
             "kernel": kernel,

@@ -147,8 +147,8 @@ int mdh_copy_boxes(const mdh_box* boxes, int nboxes, int itemsize, void* stream)
 
 /*
  * Launch-shape knobs, for measurement.  Names: "reduce_unroll" (1,2,4,8),
- * "reduce_max_blocks" (0 = one tile per workgroup), "copy_unroll" (1,2,4,8),
- * "copy_max_blocks".  Returns MDH_EINVAL for an unknown name or value.
+ * "reduce_max_blocks" (0 = one tile per workgroup), "copy_unroll" (1,2,4,8;
+ * contiguous segments), "box_unroll" (1,2,4,8; strided boxes), "copy_max_blocks".  Returns MDH_EINVAL for an unknown name or value.
  * No counterpart in the reference, whose grid is fixed at 4/16/64 blocks
  * (core/kernels.cc:547-556).
  */

@@ -74,6 +74,9 @@ int* knob(const char* name) {
   if (!std::strcmp(name, "copy_unroll")) {
     return &t.copy_unroll;
   }
+  if (!std::strcmp(name, "box_unroll")) {
+    return &t.box_unroll;
+  }
   if (!std::strcmp(name, "copy_max_blocks")) {
     return &t.copy_max_blocks;
   }

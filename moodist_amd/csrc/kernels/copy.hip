@@ -33,6 +33,8 @@ struct BoxDesc {
   uint32_t cols; // vectors per row
   uint32_t nct;  // column tiles per row of tiles
   uint32_t log2tc;
+  uint32_t src_span; // bytes from src to the end of the box, when both spans fit 32 bits (else 0)
+  uint32_t dst_span;
 };
 
 struct CopyArgs {
@@ -81,10 +83,10 @@ __global__ __launch_bounds__(kBlock) void copy_boxes_kernel(CopyArgs a) {
 #pragma unroll
     for (int k = 0; k < kMaxBoxes - 1; ++k) {
       const uint32_t e = a.tile_end[k];
-      if (tile >= e) {
-        ++b;
-        start = e;
-      }
+      // ends ascend, so the last one at or below the tile names the box; written as selects
+      // of scalars so that the whole scan stays on the scalar unit
+      b = tile >= e ? (uint32_t)(k + 1) : b;
+      start = tile >= e ? e : start;
     }
     const BoxDesc& B = a.box[b];
     const uint32_t local = tile - start;
@@ -133,6 +135,70 @@ __global__ __launch_bounds__(kBlock) void copy_boxes_kernel(CopyArgs a) {
   }
 }
 
+// The same tiling for boxes whose byte span fits 32 bits on both sides (all but
+// multi-GiB boxes) and whose vectors are 16 bytes: each side is addressed through
+// one buffer descriptor per box (wave-uniform base) and a 32-bit lane offset, so
+// a slot costs two integer multiplies instead of 64-bit address arithmetic, and
+// an out-of-range slot is given an offset past the descriptor's end -- its load
+// returns zero and its store is dropped -- instead of a predicate.
+template<int U>
+__global__ __launch_bounds__(kBlock) void copy_boxes16_kernel(CopyArgs a) {
+  constexpr uint32_t log2slots = ilog2(kBlock * U);
+  for (uint32_t tile = blockIdx.x; tile < a.total_tiles; tile += gridDim.x) {
+    uint32_t b = 0, start = 0;
+#pragma unroll
+    for (int k = 0; k < kMaxBoxes - 1; ++k) {
+      const uint32_t e = a.tile_end[k];
+      // ends ascend, so the last one at or below the tile names the box; written as selects
+      // of scalars so that the whole scan stays on the scalar unit
+      b = tile >= e ? (uint32_t)(k + 1) : b;
+      start = tile >= e ? e : start;
+    }
+    const BoxDesc& B = a.box[b];
+    const uint32_t local = tile - start;
+    const uint32_t rt = local / B.nct;
+    const uint32_t ct = local - rt * B.nct;
+    const uint32_t log2tc = B.log2tc;
+    const uint32_t log2tr = log2slots - log2tc;
+    const uint32_t tcmask = (1u << log2tc) - 1u;
+    const __amdgpu_buffer_rsrc_t rs = tile_rsrc(B.src, B.src_span);
+    const __amdgpu_buffer_rsrc_t rd = tile_rsrc(B.dst, B.dst_span);
+    u32x4 v[U];
+    uint32_t doff[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t slot = (uint32_t)u * kBlock + threadIdx.x;
+      const uint32_t col = (ct << log2tc) + (slot & tcmask);
+      uint32_t row = (rt << log2tr) + (slot >> log2tc);
+      const bool ok = col < B.cols && row < B.rows;
+      uint32_t so, dof;
+      if (B.nouter <= 1) {
+        so = row * (uint32_t)B.src_stride[0];
+        dof = row * (uint32_t)B.dst_stride[0];
+      } else {
+        so = 0, dof = 0;
+        for (uint32_t k = 0; k + 1 < B.nouter; ++k) {
+          const uint32_t q = row / B.outer[k];
+          const uint32_t i = row - q * B.outer[k];
+          so += i * (uint32_t)B.src_stride[k];
+          dof += i * (uint32_t)B.dst_stride[k];
+          row = q;
+        }
+        so += row * (uint32_t)B.src_stride[B.nouter - 1];
+        dof += row * (uint32_t)B.dst_stride[B.nouter - 1];
+      }
+      so += col * 16u;
+      dof += col * 16u;
+      doff[u] = ok ? dof : 0xffffffffu;
+      v[u] = tile_load(rs, ok ? so : 0xffffffffu);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      tile_store(rd, doff[u], v[u]);
+    }
+  }
+}
+
 // Contiguous segments (the shards of a dense all-gather, or any box that
 // collapses to one run): no per-lane index arithmetic at all.  A tile is
 // kBlock*U consecutive 16-byte vectors of one segment, addressed through a
@@ -166,10 +232,8 @@ __global__ __launch_bounds__(kBlock) void copy_flat_kernel(FlatArgs a) {
 #pragma unroll
       for (int k = 0; k < kMaxSegments - 1; ++k) {
         const uint32_t e = a.tile_end[k];
-        if (tile >= e) {
-          ++seg;
-          start = e;
-        }
+        seg = tile >= e ? (uint32_t)(k + 1) : seg;
+        start = tile >= e ? e : start;
       }
       local = tile - start;
     }
@@ -213,6 +277,7 @@ int vec_width(const HostBox& h) {
 struct Launcher {
   hipStream_t stream;
   std::vector<BoxDesc> pending[5]; // by log2(VEC)
+  std::vector<BoxDesc> pending16;  // 16-byte vectors, spans inside 32 bits: copy_boxes16_kernel
   struct Segment {
     const char* src;
     char* dst;
@@ -297,7 +362,7 @@ struct Launcher {
       grid = 0x7fffffffu;
     }
     dim3 g(grid), b(kBlock);
-    switch (t.copy_unroll) {
+    switch (t.box_unroll) {
     case 1:
       hipLaunchKernelGGL((copy_boxes_kernel<VEC, 1>), g, b, 0, stream, a);
       break;
@@ -317,9 +382,36 @@ struct Launcher {
     }
   }
 
+  void launch16(CopyArgs& a) {
+    const Tuning& t = tuning();
+    uint32_t grid = a.total_tiles;
+    if (t.copy_max_blocks > 0 && grid > (uint32_t)t.copy_max_blocks) {
+      grid = (uint32_t)t.copy_max_blocks;
+    }
+    dim3 g(grid), b(kBlock);
+    switch (t.box_unroll) {
+    case 1:
+      hipLaunchKernelGGL((copy_boxes16_kernel<1>), g, b, 0, stream, a);
+      break;
+    case 2:
+      hipLaunchKernelGGL((copy_boxes16_kernel<2>), g, b, 0, stream, a);
+      break;
+    case 4:
+      hipLaunchKernelGGL((copy_boxes16_kernel<4>), g, b, 0, stream, a);
+      break;
+    default:
+      hipLaunchKernelGGL((copy_boxes16_kernel<8>), g, b, 0, stream, a);
+      break;
+    }
+    int r = check_launch("copy_boxes16_kernel");
+    if (r != MDH_OK) {
+      rc = r;
+    }
+  }
+
   void flush_class(int lg) {
-    auto& list = pending[lg];
-    const int U = tuning().copy_unroll;
+    auto& list = lg == 5 ? pending16 : pending[lg];
+    const int U = tuning().box_unroll;
     const uint32_t slots = (uint32_t)kBlock * (uint32_t)U;
     size_t i = 0;
     while (i < list.size()) {
@@ -357,6 +449,9 @@ struct Launcher {
         continue;
       }
       switch (lg) {
+      case 5:
+        launch16(a);
+        break;
       case 4:
         launch<16>(a);
         break;
@@ -379,7 +474,7 @@ struct Launcher {
 
   void flush() {
     flush_flat();
-    for (int lg = 4; lg >= 0; --lg) {
+    for (int lg = 5; lg >= 0; --lg) {
       flush_class(lg);
     }
   }
@@ -411,6 +506,18 @@ struct Launcher {
     d.rows = (uint32_t)rows;
     d.cols = (uint32_t)(h.run / vec);
     d.nct = d.log2tc = 0;
+    d.src_span = d.dst_span = 0;
+    uint64_t sspan = (uint64_t)h.run, dspan = (uint64_t)h.run;
+    for (int k = 0; k < h.nd; ++k) {
+      sspan += (uint64_t)(h.shape[k] - 1) * (uint64_t)h.sstride[k];
+      dspan += (uint64_t)(h.shape[k] - 1) * (uint64_t)h.dstride[k];
+    }
+    if (vec == 16 && sspan < 0xffffff00ull && dspan < 0xffffff00ull) {
+      d.src_span = (uint32_t)sspan;
+      d.dst_span = (uint32_t)dspan;
+      pending16.push_back(d);
+      return;
+    }
     pending[lg].push_back(d);
   }
 

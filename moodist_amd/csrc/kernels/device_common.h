@@ -81,7 +81,8 @@ int check_launch(const char* what);
 struct Tuning {
   int reduce_unroll = 4;
   int reduce_max_blocks = 0;
-  int copy_unroll = 4;
+  int copy_unroll = 4; // contiguous segments
+  int box_unroll = 2;  // strided boxes
   int copy_max_blocks = 0;
 };
 Tuning& tuning();

@@ -107,9 +107,10 @@ def test_gather_2d_against_oracle(dev):
 @pytest.mark.parametrize("unroll", [1, 2, 4, 8])
 @pytest.mark.parametrize("max_blocks", [0, 5])
 def test_copy_parity_under_every_launch_shape(dev, unroll, max_blocks):
-    old = abi.get_tuning("copy_unroll"), abi.get_tuning("copy_max_blocks")
+    old = abi.get_tuning("copy_unroll"), abi.get_tuning("copy_max_blocks"), abi.get_tuning("box_unroll")
     try:
         abi.set_tuning("copy_unroll", unroll)
+        abi.set_tuning("box_unroll", unroll)
         abi.set_tuning("copy_max_blocks", max_blocks)
         G = torch.randn(96, 200)
         Gd = G.to(dev)
@@ -126,6 +127,7 @@ def test_copy_parity_under_every_launch_shape(dev, unroll, max_blocks):
     finally:
         abi.set_tuning("copy_unroll", old[0])
         abi.set_tuning("copy_max_blocks", old[1])
+        abi.set_tuning("box_unroll", old[2])
 
 
 def _strides(t):
