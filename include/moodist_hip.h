@@ -95,8 +95,10 @@ const char* mdh_last_error(void);
  * adds, signed min/max.  bfloat16/float16: sources widened to fp32, folded in
  * fp32, rounded to nearest even once.
  *
- * Pointers and sizes may have any alignment; the 16-byte path is taken when
- * every pointer is 16-byte aligned.  numel == 0 is a no-op.
+ * Pointers need element alignment only, sizes none: no staging copy is ever
+ * made (the reference stages through an aligned buffer when bytes % 16 or
+ * address % 16 is non-zero, core/processgroup.cc:1409-1431).  numel == 0 is a
+ * no-op.
  */
 int mdh_reduce(const void* const* srcs, int nsrc, int first, void* dst, size_t numel, int dtype, int op,
     float scale, void* stream);

@@ -73,7 +73,6 @@ extern "C" int mdh_reduce(const void* const* srcs, int nsrc, int first, void* ds
     return MDH_EINVAL;
   }
   ReduceArgs a;
-  bool aligned = ((uintptr_t)dst % 16) == 0;
   const uintptr_t bytes = (uintptr_t)numel * itemsize;
   for (int j = 0; j < nsrc; ++j) {
     const void* p = srcs[(first + j) % nsrc];
@@ -91,7 +90,6 @@ extern "C" int mdh_reduce(const void* const* srcs, int nsrc, int first, void* ds
       set_error("mdh_reduce: destination partially overlaps source %d", (first + j) % nsrc);
       return MDH_EINVAL;
     }
-    aligned = aligned && ((uintptr_t)p % 16) == 0;
     a.src[j] = p;
   }
   for (int j = nsrc; j < MDH_MAX_SOURCES; ++j) {
@@ -103,7 +101,7 @@ extern "C" int mdh_reduce(const void* const* srcs, int nsrc, int first, void* ds
   }
   a.dst = dst;
   a.numel = numel;
-  a.nvec = aligned ? bytes / 16 : 0;
+  a.nvec = bytes / 16;
   a.scale = scale;
   a.nsrc = nsrc;
   a.mode = mode;
@@ -111,11 +109,11 @@ extern "C" int mdh_reduce(const void* const* srcs, int nsrc, int first, void* ds
 #define MDH_DISPATCH(tname)                                  \
   switch (fold_op) {                                         \
   case kSum:                                                 \
-    return reduce_launch_##tname##_sum(a, aligned, s);       \
+    return reduce_launch_##tname##_sum(a, s);       \
   case kMin:                                                 \
-    return reduce_launch_##tname##_min(a, aligned, s);       \
+    return reduce_launch_##tname##_min(a, s);       \
   default:                                                   \
-    return reduce_launch_##tname##_max(a, aligned, s);       \
+    return reduce_launch_##tname##_max(a, s);       \
   }
   switch (dtype) {
   case MDH_DTYPE_FLOAT32:

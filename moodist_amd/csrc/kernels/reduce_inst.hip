@@ -19,7 +19,7 @@ using f16 = f16_t;
 #define MDH_CAT2(a, b, c, d) a##b##c##d
 #define MDH_CAT(a, b, c, d) MDH_CAT2(a, b, c, d)
 
-int MDH_CAT(reduce_launch_, MDH_TNAME, _, MDH_FNAME)(const ReduceArgs& a, bool aligned, hipStream_t stream) {
-  return launch<MDH_TNAME, MDH_FNAME>(a, aligned, stream);
+int MDH_CAT(reduce_launch_, MDH_TNAME, _, MDH_FNAME)(const ReduceArgs& a, hipStream_t stream) {
+  return launch<MDH_TNAME, MDH_FNAME>(a, stream);
 }
 } // namespace mdh

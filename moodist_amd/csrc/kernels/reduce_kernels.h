@@ -291,9 +291,10 @@ __device__ __forceinline__ void reduce_tile(const ReduceArgs& a, int nsrc, uint6
   }
 }
 
-// Vector path: all pointers 16-byte aligned.  A tile is kBlock*U consecutive
-// 16-byte vectors; tiles are dealt to workgroups round-robin.  Elements past
-// the last whole vector (fewer than 16 bytes) are folded by workgroup 0.
+// A tile is kBlock*U consecutive 16-byte vectors; tiles are dealt to
+// workgroups round-robin.  Pointers need only element alignment: gfx950's
+// 16-byte buffer accesses take any byte address.  Elements past the last whole
+// vector (fewer than 16 bytes) are folded by workgroup 0.
 template<typename T, int F, int NSRC, int U>
 __global__ __launch_bounds__(kBlock) void reduce_vec_kernel(ReduceArgs a) {
   const int nsrc = NSRC ? NSRC : a.nsrc;
@@ -318,15 +319,6 @@ __global__ __launch_bounds__(kBlock) void reduce_vec_kernel(ReduceArgs a) {
     if (i < a.numel) {
       reduce_one_elem<T, F>(a, nsrc, i);
     }
-  }
-}
-
-// Element path: any alignment.
-template<typename T, int F>
-__global__ __launch_bounds__(kBlock) void reduce_elem_kernel(ReduceArgs a) {
-  const uint64_t stride = (uint64_t)gridDim.x * kBlock;
-  for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < a.numel; i += stride) {
-    reduce_one_elem<T, F>(a, a.nsrc, i);
   }
 }
 
@@ -373,15 +365,7 @@ int launch_vec(const ReduceArgs& a, hipStream_t stream) {
 }
 
 template<typename T, int F>
-int launch(const ReduceArgs& a, bool aligned, hipStream_t stream) {
-  if (!aligned) {
-    uint64_t grid = (a.numel + kBlock - 1) / kBlock;
-    if (grid > 65536) {
-      grid = 65536;
-    }
-    hipLaunchKernelGGL((reduce_elem_kernel<T, F>), dim3((unsigned)grid), dim3(kBlock), 0, stream, a);
-    return check_launch("reduce_elem_kernel");
-  }
+int launch(const ReduceArgs& a, hipStream_t stream) {
   // Source counts with a fully unrolled instantiation; anything else takes
   // the run-time loop over chunks of eight.
   if constexpr (std::is_same_v<T, float> || std::is_same_v<T, bf16_t>) {
@@ -398,7 +382,7 @@ int launch(const ReduceArgs& a, bool aligned, hipStream_t stream) {
 // One entry per (element type, fold), each instantiated in its own object
 // file (reduce_inst.hip compiled once per pair) so they build in parallel.
 #define MDH_REDUCE_ENTRY(tname, fname) \
-  int reduce_launch_##tname##_##fname(const ReduceArgs& a, bool aligned, hipStream_t stream)
+  int reduce_launch_##tname##_##fname(const ReduceArgs& a, hipStream_t stream)
 #define MDH_REDUCE_ENTRIES(tname) \
   MDH_REDUCE_ENTRY(tname, sum);   \
   MDH_REDUCE_ENTRY(tname, min);   \
