@@ -79,3 +79,22 @@ def test_tuning_round_trip():
     abi.set_tuning("copy_unroll", 2)
     assert abi.get_tuning("copy_unroll") == 2
     abi.set_tuning("copy_unroll", old)
+
+
+def test_missing_kernel_library_fails_loudly(monkeypatch, tmp_path):
+    # there is no CPU fallback: without the built library every entry raises
+    monkeypatch.setattr(abi, "_lib", None)
+    monkeypatch.setattr(abi, "LIB_PATH", str(tmp_path / "libmoodist_hip.so"))
+    with pytest.raises(abi.MoodistError, match="is not built"):
+        abi.reduce([16], 0, 32, 4, abi.DTYPE_FLOAT32, abi.OP_SUM)
+    with pytest.raises(abi.MoodistError, match="is not built"):
+        abi.gather([16], 32, 4, 1, 4, 4, 4)
+
+
+def test_product_code_never_imports_the_oracle():
+    import glob
+
+    for path in glob.glob(os.path.join(ROOT, "moodist_amd", "**", "*"), recursive=True):
+        if os.path.isfile(path) and path.endswith((".py", ".cc", ".h", ".hip", ".sh")):
+            text = open(path, errors="ignore").read()
+            assert "import oracle" not in text and "from oracle" not in text and "liboracle" not in text, path
