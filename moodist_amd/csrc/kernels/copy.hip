@@ -139,8 +139,8 @@ __global__ __launch_bounds__(kBlock) void copy_boxes_kernel(CopyArgs a) {
 // multi-GiB boxes) and whose vectors are 16 bytes: each side is addressed through
 // one buffer descriptor per box (wave-uniform base) and a 32-bit lane offset, so
 // a slot costs two integer multiplies instead of 64-bit address arithmetic, and
-// an out-of-range slot is given an offset past the descriptor's end -- its load
-// returns zero and its store is dropped -- instead of a predicate.
+// an out-of-range slot is given the offset just past the descriptor's end -- its
+// load returns zero and its store is dropped -- instead of a predicate.
 template<int U>
 __global__ __launch_bounds__(kBlock) void copy_boxes16_kernel(CopyArgs a) {
   constexpr uint32_t log2slots = ilog2(kBlock * U);
@@ -189,8 +189,9 @@ __global__ __launch_bounds__(kBlock) void copy_boxes16_kernel(CopyArgs a) {
       }
       so += col * 16u;
       dof += col * 16u;
-      doff[u] = ok ? dof : 0xffffffffu;
-      v[u] = tile_load(rs, ok ? so : 0xffffffffu);
+      // the span itself is the first offset past the descriptor's end
+      doff[u] = ok ? dof : B.dst_span;
+      v[u] = tile_load(rs, ok ? so : B.src_span);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {

@@ -242,3 +242,73 @@ def test_config5_3d_dim0_to_dim2_full_size(dev):
         abi.copy_boxes(boxes, 2, st())
         sync()
         assert torch.equal(out.cpu(), G3[:, :, 128 * k:128 * (k + 1)])
+
+
+def test_random_boxes_against_oracle(dev):
+    """Random shapes, strides (incl. gaps, transposes, non-unit innermost strides), element sizes and
+    offsets, several boxes per call: the GPU result must equal the oracle's element-by-element copy,
+    and bytes outside the boxes must stay untouched."""
+    rng = np.random.RandomState(11)
+    for trial in range(40):
+        itemsize = int(rng.choice([1, 2, 4, 8, 16]))
+        nboxes = int(rng.randint(1, 5))
+        src_bufs, specs = [], []
+        dst_elems = 0
+        for _ in range(nboxes):
+            nd = int(rng.randint(1, 5))
+            shape = [int(rng.randint(1, 9)) for _ in range(nd)]
+            if rng.rand() < 0.5:
+                shape[-1] = int(rng.choice([4, 16, 33, 64]))
+            # source: a dense parent with padding in every dimension, optionally permuted
+            pshape = [s + int(rng.randint(0, 3)) for s in shape]
+            perm = list(rng.permutation(nd)) if rng.rand() < 0.4 else list(range(nd))
+            dense = [0] * nd
+            acc = 1
+            for d in reversed(range(nd)):
+                dense[perm[d]] = acc
+                acc *= pshape[perm[d]]
+            soff = int(rng.randint(0, 3))
+            src_numel = acc + soff
+            # destination: its own dense parent with padding, natural order
+            dshape = [s + int(rng.randint(0, 2)) for s in shape]
+            dstr = [0] * nd
+            acc2 = 1
+            for d in reversed(range(nd)):
+                dstr[d] = acc2
+                acc2 *= dshape[d]
+            specs.append((shape, dense, soff, src_numel, dstr, dst_elems + int(rng.randint(0, 3)), acc2))
+            dst_elems = specs[-1][5] + acc2
+        dst_elems += 3
+        dst_host = rng.randint(0, 256, dst_elems * itemsize).astype(np.uint8)
+        want = dst_host.copy()
+        dst_dev = torch.from_numpy(dst_host.copy()).to(dev)
+        boxes, keep = [], []
+        for shape, sstr, soff, src_numel, dstr, doff, _ in specs:
+            src_host = rng.randint(0, 256, src_numel * itemsize).astype(np.uint8)
+            src_dev = torch.from_numpy(src_host).to(dev)
+            keep.append(src_dev)
+            oracle.copy_box(src_host, soff, want, doff, shape, sstr, dstr, itemsize)
+            boxes.append(abi.make_box(src_dev.data_ptr() + soff * itemsize, dst_dev.data_ptr() + doff * itemsize, shape,
+                                      sstr, dstr))
+        abi.copy_boxes(boxes, itemsize, st())
+        sync()
+        assert np.array_equal(dst_dev.cpu().numpy(), want), (trial, itemsize, specs)
+
+
+def test_gather_and_boxes_beyond_4_gib(dev):
+    n = (1 << 32) + 4096 + 5  # bytes per shard: past 32-bit offsets, ragged
+    shards = [torch.empty(n, dtype=torch.uint8, device=dev).random_() for _ in range(2)]
+    out = torch.zeros(2 * n + 16, dtype=torch.uint8, device=dev)
+    abi.gather([s.data_ptr() for s in shards], out.data_ptr(), n, 1, n, n, n, st())
+    sync()
+    assert torch.equal(out[:n], shards[0]) and torch.equal(out[n:2 * n], shards[1]) and (out[2 * n:] == 0).all()
+    del out
+    # a strided box whose source spans more than 4 GiB: rows of 1 MiB at a pitch of 5 MiB, 1000 rows
+    pitch, width, rows = 5 << 20, 1 << 20, 1000
+    src = shards[0][:0]  # free references
+    del shards
+    big = torch.empty(rows * pitch, dtype=torch.uint8, device=dev).random_()
+    dst = torch.zeros(rows * width, dtype=torch.uint8, device=dev)
+    abi.copy_boxes([abi.make_box(big.data_ptr(), dst.data_ptr(), [rows, width], [pitch, 1], [width, 1])], 1, st())
+    sync()
+    assert torch.equal(dst.view(rows, width), big.view(rows, pitch)[:, :width])

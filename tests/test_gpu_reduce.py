@@ -253,3 +253,17 @@ def test_config4_fp32_p64_sum_avg_max_full_size(dev):
     # properties: AVG by 2^-6 is SUM / 64 exactly; MAX equals torch's maximum over the stack
     assert torch.equal(outs[oracle.OP_AVG], outs[oracle.OP_SUM] / 64)
     assert torch.equal(outs[oracle.OP_MAX], torch.stack(srcs).amax(dim=0))
+
+
+def test_reduce_beyond_4_gib_per_source(dev):
+    # byte offsets past 2^32: compared on the GPU with torch's own element-wise add (IEEE, same order)
+    n = (1 << 30) + 4099  # 4 GiB + 16 KiB + 12 B of fp32
+    a = torch.empty(n, device=dev).uniform_(-1, 1)
+    b = torch.empty(n, device=dev).uniform_(-1, 1)
+    out = torch.zeros(n, device=dev)
+    gpu_reduce([a, b], 1, out, oracle.OP_SUM)
+    assert torch.equal(out, b + a)
+    del out
+    out = torch.zeros(n, device=dev)
+    gpu_reduce([a, b], 0, out, oracle.OP_MAX)
+    assert torch.equal(out, torch.maximum(a, b))
