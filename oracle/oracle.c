@@ -22,6 +22,11 @@
  *   orc_cpu_reduce_scatter_ranks  timing harness only; its result is checked
  *                   against orc_reduce.
  *
+ * No function here is left unpinned.  What the reference's OWN tests do not
+ * cover -- and what is therefore pinned by the closed forms and torch
+ * witnesses above only -- is: 16-bit floats, MIN/MAX/AVG/PREMUL_SUM, more than
+ * eight sources, and strided (non-contiguous-slice) copies.
+ *
  * dtype codes are torch ScalarType numbers and op codes are c10d RedOpType
  * numbers, as on the reference's API (api/moodist_api.h:30-55).
  */

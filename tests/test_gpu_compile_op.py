@@ -181,7 +181,7 @@ def test_future_before_every_rank_called(world, dev):
     assert all(torch.equal(o, src) for o in outs)
 
 
-# ---- BASELINE configuration 5 through the operator surface ----
+# ---- the full-size redistribution configurations through the operator surface ----
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=str)
 def test_config5_matrix_row_shards_to_column_shards(world, dev, dtype):

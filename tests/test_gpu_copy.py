@@ -189,7 +189,7 @@ def test_boxes_many_dims_many_boxes_and_empty(dev):
     assert b.item() == 5.0
 
 
-# ---- BASELINE configurations at full size ----
+# ---- the benchmark configurations at full size ----
 
 def test_config2_allgather_bf16_full_size_contiguous_and_strided(dev):
     P, n = 8, 16777216

@@ -198,7 +198,7 @@ def test_bf16_within_one_ulp_of_fp32_accumulated_reference(dev):
     assert torch.equal(out.cpu(), ref)  # in fact identical: same order, same single rounding
 
 
-# ---- BASELINE configurations at full size ----
+# ---- the benchmark configurations at full size ----
 
 def _seeded(r, n, kind):
     torch.manual_seed(r)
