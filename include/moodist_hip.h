@@ -148,7 +148,8 @@ typedef struct mdh_box {
 int mdh_copy_boxes(const mdh_box* boxes, int nboxes, int itemsize, void* stream);
 
 /*
- * Launch-shape knobs, for measurement.  Names: "reduce_unroll" (1,2,4,8),
+ * Launch-shape knobs, for measurement; 0 (the default) lets the library choose
+ * by size.  Names: "reduce_unroll" (1,2,4,8),
  * "reduce_max_blocks" (0 = one tile per workgroup), "copy_unroll" (1,2,4,8;
  * contiguous segments), "box_unroll" (1,2,4,8; strided boxes), "copy_max_blocks".  Returns MDH_EINVAL for an unknown name or value.
  * No counterpart in the reference, whose grid is fixed at 4/16/64 blocks

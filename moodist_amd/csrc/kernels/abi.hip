@@ -92,7 +92,7 @@ extern "C" int mdh_set_tuning(const char* name, int value) {
   }
   const bool unroll = std::strstr(name, "unroll") != nullptr;
   if (unroll) {
-    if (!(value == 1 || value == 2 || value == 4 || value == 8)) {
+    if (!(value == 0 || value == 1 || value == 2 || value == 4 || value == 8)) {
       mdh::set_error("mdh_set_tuning: %s does not take %d", name, value);
       return MDH_EINVAL;
     }

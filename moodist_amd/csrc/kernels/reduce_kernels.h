@@ -328,7 +328,7 @@ int launch_vec(const ReduceArgs& a, hipStream_t stream) {
   // 16-bit types widen every vector to eight fp32 accumulators: two sub-tiles at most, and one
   // when sixteen sources are unrolled (their loads alone fill the register budget; measured
   // 6.4 TB/s against 5.3 TB/s with two on the bf16 sixteen-source workload).
-  int U = t.reduce_unroll;
+  int U = t.reduce_unroll ? t.reduce_unroll : auto_unroll(a.nvec, 4);
   if (sizeof(typename Traits<T>::elem_t) == 2) {
     U = U > 2 ? 2 : U;
     if (NSRC >= 16) {

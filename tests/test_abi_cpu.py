@@ -98,3 +98,14 @@ def test_product_code_never_imports_the_oracle():
         if os.path.isfile(path) and path.endswith((".py", ".cc", ".h", ".hip", ".sh")):
             text = open(path, errors="ignore").read()
             assert "import oracle" not in text and "from oracle" not in text and "liboracle" not in text, path
+
+
+def test_launch_without_a_device_is_an_error_not_a_crash():
+    import torch
+
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present; this checks the no-device error path")
+    with pytest.raises(abi.MoodistError, match="launch failed"):
+        abi.reduce([4096, 8192], 0, 16384, 64, abi.DTYPE_FLOAT32, abi.OP_SUM)
+    with pytest.raises(abi.MoodistError, match="launch failed"):
+        abi.gather([4096], 16384, 64, 1, 64, 64, 64)
