@@ -427,7 +427,7 @@ struct Launcher {
     const uint32_t slots = (uint32_t)kBlock * (uint32_t)U;
     size_t i = 0;
     while (i < list.size()) {
-      CopyArgs a;
+      CopyArgs a{};
       a.nboxes = 0;
       uint64_t tiles = 0;
       while (i < list.size() && a.nboxes < (uint32_t)kMaxBoxes) {
