@@ -1,5 +1,9 @@
 #include "processgroup.h"
 
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
 #include <stdexcept>
 
 #include "hip_loader.h"
@@ -7,6 +11,41 @@
 namespace moodist {
 
 namespace {
+
+// MOODIST_LOG_LEVEL = error | info | verbose | debug (the reference's variable and levels,
+// core/logging.h:59-85); at "debug" every launch is reported on stderr.
+int log_level() {
+  static const int level = [] {
+    const char* v = std::getenv("MOODIST_LOG_LEVEL");
+    if (!v) {
+      return 1;
+    }
+    if (!std::strcmp(v, "debug")) {
+      return 4;
+    }
+    if (!std::strcmp(v, "verbose")) {
+      return 3;
+    }
+    if (!std::strcmp(v, "info")) {
+      return 2;
+    }
+    return 1;
+  }();
+  return level;
+}
+
+void log_debug(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+void log_debug(const char* fmt, ...) {
+  if (log_level() < 4) {
+    return;
+  }
+  va_list ap;
+  va_start(ap, fmt);
+  std::fputs("moodist debug: ", stderr);
+  std::vfprintf(stderr, fmt, ap);
+  std::fputc('\n', stderr);
+  va_end(ap);
+}
 
 #define MD_CHECK(cond)                                                                             \
   do {                                                                                             \
@@ -421,6 +460,9 @@ void World::launch(Collective& c, const std::shared_ptr<CompiledOp>& op, bool ke
   }
   order_streams_before(c);
   std::vector<const void*> srcs((size_t)size);
+  log_debug("collective #%llu: launching %s for %d ranks, %zu bytes per rank, dtype %d", (unsigned long long)c.seq,
+      c.kind == Kind::reduce_scatter ? "reduce_scatter" : c.kind == Kind::all_gather ? "all_gather" : "custom op",
+      size, c.bytes, c.dtype);
 
   if (c.kind == Kind::reduce_scatter) {
     // out_q = in_q[q] (+) in_{q+1}[q] (+) ... in rank order starting at q (core/group.cc:567-570;

@@ -328,3 +328,49 @@ def test_process_group_is_a_c10d_process_group():
         assert pg.moodist_name() == "moodist-local-%d-of-3" % r
     with pytest.raises(RuntimeError, match="send is not supported"):
         world.groups[0].send([torch.zeros(1)], 1, 0)
+
+
+def test_compile_op_accepts_dtensor_like_specs():
+    # py/moodist/compile.py:14-59: anything with placements / device_mesh / to_local is read as a
+    # DTensor; Shard(dim) placements turn into offset/shape by ceil-division chunks
+    from torch.distributed.tensor import Replicate, Shard
+
+    class Mesh:
+        def __init__(self, sizes, coord):
+            self.sizes, self.coord = sizes, coord
+
+        def size(self, i):
+            return self.sizes[i]
+
+        def get_coordinate(self):
+            return self.coord
+
+    class FakeDTensor:
+        def __init__(self, shape, dtype, placements, mesh):
+            self.shape, self.dtype, self.placements, self.device_mesh = torch.Size(shape), dtype, placements, mesh
+
+        def to_local(self):
+            raise NotImplementedError
+
+    world = moodist_amd.LocalWorld(2, 0)
+    ops = []
+    for r, pg in enumerate(world):
+        mesh = Mesh([2], [r])
+        src = FakeDTensor([5, 4], torch.float32, [Shard(0)], mesh)  # rows 0-2 on rank 0, rows 3-4 on rank 1
+        dst = FakeDTensor([5, 4], torch.float32, [Shard(1)], mesh)  # columns 0-1 / 2-3
+        ops.append(moodist_amd.compile_op(pg, inputs=[src], outputs=[dst]))
+    p0, p1 = ops[0].plan(), ops[1].plan()
+    assert p0["inputs"] == [3 * 4 * 4] and p1["inputs"] == [2 * 4 * 4]
+    assert p0["outputs"] == [5 * 2 * 4] and p1["outputs"] == [5 * 2 * 4]
+    assert sum(rd[5] for rd in p0["reads"]) == 40 and sum(rd[5] for rd in p1["reads"]) == 40
+    # replicated placement keeps the whole tensor; mismatching global shapes are refused
+    rep = FakeDTensor([5, 4], torch.float32, [Replicate()], Mesh([2], [0]))
+    from moodist_amd.compile import _dtensor_box
+
+    assert _dtensor_box(rep) == {"offset": [0, 0], "shape": [5, 4]}
+    other = FakeDTensor([6, 4], torch.float32, [Shard(0)], Mesh([2], [0]))
+    with pytest.raises(ValueError, match="same global shape"):
+        moodist_amd.compile_op(world.groups[0], inputs=[rep], outputs=[other])
+    with pytest.raises(ValueError, match="same dtype"):
+        moodist_amd.compile_op(world.groups[0], inputs=[rep],
+                               outputs=[FakeDTensor([5, 4], torch.float64, [Shard(0)], Mesh([2], [0]))])
