@@ -196,9 +196,8 @@ std::shared_ptr<Collective> ProcessGroup::all_gather_impl(const moodist_tensor* 
       p.has_copy_back = true;
     }
   }
-  const bool kernel_less = options.forceKernelLess || options.preferKernelLess;
-  return world->post(Kind::all_gather, next_seq++, rank, std::move(p), 0, 1.0f, bytes, input.dtype, 0, nullptr,
-      kernel_less);
+  p.kernel_less = options.forceKernelLess || options.preferKernelLess;
+  return world->post(Kind::all_gather, next_seq++, rank, std::move(p), 0, 1.0f, bytes, input.dtype, 0, nullptr);
 }
 
 std::shared_ptr<Collective> ProcessGroup::reduce_scatter(const moodist_tensor* output, const moodist_tensor& input,
@@ -227,7 +226,7 @@ std::shared_ptr<Collective> ProcessGroup::reduce_scatter(const moodist_tensor* o
     p.wants_output = true;
   }
   return world->post(Kind::reduce_scatter, next_seq++, rank, std::move(p), reduce_op, premul, bytes, input.dtype, 0,
-      nullptr, false);
+      nullptr);
 }
 
 std::shared_ptr<Collective> ProcessGroup::allreduce(const moodist_tensor& tensor, const moodist_tensor* scratch,
@@ -332,7 +331,7 @@ std::shared_ptr<Collective> ProcessGroup::custom_op(const std::shared_ptr<Compil
     check_device_tensor(outputs[i], world->device, "custom op output");
     p.outputs.push_back(outputs[i]);
   }
-  return world->post(Kind::custom, next_seq++, rank, std::move(p), 0, 1.0f, 0, op->dtype, op->id, op, false);
+  return world->post(Kind::custom, next_seq++, rank, std::move(p), 0, 1.0f, 0, op->dtype, op->id, op);
 }
 
 // ---------------------------------------------------------------- World
@@ -357,7 +356,7 @@ World::~World() {
 }
 
 std::shared_ptr<Collective> World::post(Kind kind, uint64_t seq, int rank, Posting p, int reduce_op, float premul,
-    size_t bytes, int dtype, uint32_t op_id, const std::shared_ptr<CompiledOp>& op, bool kernel_less) {
+    size_t bytes, int dtype, uint32_t op_id, const std::shared_ptr<CompiledOp>& op) {
   std::lock_guard<std::mutex> l(mutex);
   std::shared_ptr<Collective>& slot = pending[seq];
   if (!slot) {
@@ -386,7 +385,7 @@ std::shared_ptr<Collective> World::post(Kind kind, uint64_t seq, int rank, Posti
   if (c->arrived == size) {
     pending.erase(seq);
     try {
-      launch(*c, op, kernel_less);
+      launch(*c, op);
     } catch (const std::exception& e) {
       c->error = e.what();
       c->launched = true;
@@ -451,7 +450,7 @@ void World::order_streams_after(Collective& c) {
   }
 }
 
-void World::launch(Collective& c, const std::shared_ptr<CompiledOp>& op, bool kernel_less) {
+void World::launch(Collective& c, const std::shared_ptr<CompiledOp>& op) {
   const HipRuntime& h = hip();
   int current = -1;
   check_hip(h.GetDevice(&current), "hipGetDevice");
@@ -492,7 +491,7 @@ void World::launch(Collective& c, const std::shared_ptr<CompiledOp>& op, bool ke
       for (int j = 0; j < size; ++j) {
         srcs[(size_t)j] = c.post[(size_t)j].input.data;
       }
-      if (kernel_less) {
+      if (pq.kernel_less) {
         // copy-engine form (core/processgroup.cc:706-833): one device-to-device copy per shard
         for (int j = 0; j < size; ++j) {
           void* dst = (char*)pq.output.data + c.bytes * (size_t)j;

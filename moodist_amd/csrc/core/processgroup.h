@@ -31,6 +31,7 @@ struct Posting {
   moodist_tensor output{};
   std::vector<moodist_tensor> inputs; // custom op
   std::vector<moodist_tensor> outputs;
+  bool kernel_less = false;   // this rank asked for the copy-engine form of all_gather
   bool has_copy_back = false; // allreduce through a padded temporary
   moodist_tensor copy_back{};
   void* stream = nullptr;
@@ -116,13 +117,13 @@ public:
   // disagree about what collective number `seq` is (the reference aborts on this,
   // core/cputhread.h:100-112).
   std::shared_ptr<Collective> post(Kind kind, uint64_t seq, int rank, Posting p, int reduce_op, float premul,
-      size_t bytes, int dtype, uint32_t op_id, const std::shared_ptr<CompiledOp>& op, bool kernel_less);
+      size_t bytes, int dtype, uint32_t op_id, const std::shared_ptr<CompiledOp>& op);
 
   const int size;
   const int device;
 
 private:
-  void launch(Collective& c, const std::shared_ptr<CompiledOp>& op, bool kernel_less);
+  void launch(Collective& c, const std::shared_ptr<CompiledOp>& op);
   void order_streams_before(Collective& c);
   void order_streams_after(Collective& c);
 
