@@ -178,9 +178,10 @@ __device__ __forceinline__ void fold_chunk(const ReduceArgs& a, int j0, uint64_t
       v[k][u] = tile_load(rs, lane_byte + (uint32_t)u * (kBlock * 16));
     }
   }
-  // Every load of the chunk is issued before the first add: without this fence the
-  // instruction scheduler interleaves loads with arithmetic to save registers and keeps only
-  // about a dozen loads in flight per lane.
+  // Every load of the chunk is issued before the first add.  Without this fence the
+  // instruction scheduler interleaves loads with arithmetic to save registers (about a dozen
+  // loads in flight per lane instead of 8*U); on the eight-source workload both orders time the
+  // same, the fence just makes the number in flight independent of scheduler heuristics.
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int k = 0; k < CNT; ++k) {
