@@ -84,6 +84,12 @@ int moodist_pg_set_option(moodist_pg* pg, const char* name, int64_t value);
 /* processGroupAllGather (api/processgroup_api.h:43; core/processgroup.cc:1059-1284) */
 int moodist_pg_all_gather(moodist_pg* pg, const moodist_tensor* output, const moodist_tensor* input, void* stream,
     moodist_work** work);
+/* c10d's list form, allgather(output_lists, inputs) (wrapper/processgroup_wrapper.cc:112-129):
+ * outputs[j] receives rank j's input.  The reference gathers into a flat temporary and copies
+ * each row out; here the sources are copied straight into the outputs.  Outputs must be
+ * dense, of the input's dtype and size; n_outputs must equal the group size. */
+int moodist_pg_all_gather_list(moodist_pg* pg, const moodist_tensor* outputs, size_t n_outputs,
+    const moodist_tensor* input, void* stream, moodist_work** work);
 /* processGroupReduceScatter (api/processgroup_api.h:45-46; core/processgroup.cc:1290-1668).
  * reduce_op is a c10d RedOpType number; premul_value is used by PREMUL_SUM only. */
 int moodist_pg_reduce_scatter(moodist_pg* pg, const moodist_tensor* output, const moodist_tensor* input,

@@ -138,6 +138,16 @@ int moodist_pg_all_gather(moodist_pg* pg, const moodist_tensor* output, const mo
   });
 }
 
+int moodist_pg_all_gather_list(moodist_pg* pg, const moodist_tensor* outputs, size_t n_outputs,
+    const moodist_tensor* input, void* stream, moodist_work** work) {
+  return guarded([&] {
+    if (!outputs || !input) {
+      throw std::runtime_error("moodist: null tensor");
+    }
+    give(work, as_pg(pg)->all_gather_list(outputs, n_outputs, *input, stream));
+  });
+}
+
 int moodist_pg_reduce_scatter(moodist_pg* pg, const moodist_tensor* output, const moodist_tensor* input,
     int reduce_op, void* stream, float premul_value, moodist_work** work) {
   return guarded([&] {

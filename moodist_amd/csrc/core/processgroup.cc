@@ -200,6 +200,33 @@ std::shared_ptr<Collective> ProcessGroup::all_gather_impl(const moodist_tensor* 
   return world->post(Kind::all_gather, next_seq++, rank, std::move(p), 0, 1.0f, bytes, input.dtype, 0, nullptr);
 }
 
+// The list form of all_gather (wrapper/processgroup_wrapper.cc:112-129).  The reference gathers
+// into a flat temporary and copies each row out; here every source is copied straight into its
+// destination tensor, so no temporary exists.
+std::shared_ptr<Collective> ProcessGroup::all_gather_list(const moodist_tensor* outputs, size_t n_outputs,
+    const moodist_tensor& input, void* stream) {
+  Busy guard(*this);
+  check_device_tensor(input, world->device, "all_gather input");
+  const size_t bytes = bytes_of(input);
+  MD_CHECK(bytes > 0);
+  if (n_outputs != (size_t)size) {
+    throw std::runtime_error("moodist: all_gather needs one output tensor per rank (" + std::to_string(size) +
+                             "), got " + std::to_string(n_outputs));
+  }
+  Posting p;
+  p.input = input;
+  p.stream = stream;
+  p.wants_output = true;
+  for (size_t i = 0; i < n_outputs; ++i) {
+    check_device_tensor(outputs[i], world->device, "all_gather output");
+    MD_CHECK(outputs[i].dtype == input.dtype);
+    MD_CHECK(bytes_of(outputs[i]) == bytes);
+    p.outputs.push_back(outputs[i]);
+  }
+  p.kernel_less = options.forceKernelLess || options.preferKernelLess;
+  return world->post(Kind::all_gather, next_seq++, rank, std::move(p), 0, 1.0f, bytes, input.dtype, 0, nullptr);
+}
+
 std::shared_ptr<Collective> ProcessGroup::reduce_scatter(const moodist_tensor* output, const moodist_tensor& input,
     int reduce_op, void* stream, float premul) {
   Busy guard(*this);
@@ -491,7 +518,36 @@ void World::launch(Collective& c, const std::shared_ptr<CompiledOp>& op) {
       for (int j = 0; j < size; ++j) {
         srcs[(size_t)j] = c.post[(size_t)j].input.data;
       }
-      if (pq.kernel_less) {
+      if (!pq.outputs.empty()) {
+        // one destination tensor per source rank
+        if (pq.kernel_less) {
+          for (int j = 0; j < size; ++j) {
+            if (pq.outputs[(size_t)j].data != srcs[(size_t)j]) {
+              check_hip(h.MemcpyAsync(pq.outputs[(size_t)j].data, srcs[(size_t)j], c.bytes, kHipMemcpyDeviceToDevice,
+                            pq.stream),
+                  "hipMemcpyAsync");
+            }
+          }
+        } else {
+          std::vector<mdh_box> boxes;
+          boxes.reserve((size_t)size);
+          for (int j = 0; j < size; ++j) {
+            if (pq.outputs[(size_t)j].data == srcs[(size_t)j]) {
+              continue; // already in place
+            }
+            mdh_box b{};
+            b.src = srcs[(size_t)j];
+            b.dst = pq.outputs[(size_t)j].data;
+            b.ndim = 1;
+            b.shape[0] = (int64_t)c.bytes;
+            b.src_strides[0] = b.dst_strides[0] = 1;
+            boxes.push_back(b);
+          }
+          if (!boxes.empty()) {
+            check_mdh(h.copy_boxes(boxes.data(), (int)boxes.size(), 1, pq.stream));
+          }
+        }
+      } else if (pq.kernel_less) {
         // copy-engine form (core/processgroup.cc:706-833): one device-to-device copy per shard
         for (int j = 0; j < size; ++j) {
           void* dst = (char*)pq.output.data + c.bytes * (size_t)j;

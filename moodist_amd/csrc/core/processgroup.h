@@ -29,8 +29,8 @@ struct Posting {
   bool wants_output = false;
   moodist_tensor input{};
   moodist_tensor output{};
-  std::vector<moodist_tensor> inputs; // custom op
-  std::vector<moodist_tensor> outputs;
+  std::vector<moodist_tensor> inputs;  // custom op
+  std::vector<moodist_tensor> outputs; // custom op; all_gather into one tensor per rank
   bool kernel_less = false;   // this rank asked for the copy-engine form of all_gather
   bool has_copy_back = false; // allreduce through a padded temporary
   moodist_tensor copy_back{};
@@ -71,6 +71,8 @@ public:
   ProcessGroup(World* world, int rank, int size) : world(world), rank(rank), size(size) {}
 
   std::shared_ptr<Collective> all_gather(const moodist_tensor* output, const moodist_tensor& input, void* stream);
+  std::shared_ptr<Collective> all_gather_list(const moodist_tensor* outputs, size_t n_outputs,
+      const moodist_tensor& input, void* stream);
   std::shared_ptr<Collective> reduce_scatter(const moodist_tensor* output, const moodist_tensor& input, int reduce_op,
       void* stream, float premul);
   std::shared_ptr<Collective> allreduce(const moodist_tensor& tensor, const moodist_tensor* scratch, int reduce_op,

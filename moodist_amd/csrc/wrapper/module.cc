@@ -42,6 +42,7 @@ struct CoreApi {
   MOODIST_CORE_FN(moodist_pg_get_option)
   MOODIST_CORE_FN(moodist_pg_set_option)
   MOODIST_CORE_FN(moodist_pg_all_gather)
+  MOODIST_CORE_FN(moodist_pg_all_gather_list)
   MOODIST_CORE_FN(moodist_pg_reduce_scatter)
   MOODIST_CORE_FN(moodist_pg_allreduce)
   MOODIST_CORE_FN(moodist_pg_stage_input)
@@ -91,6 +92,7 @@ void load_core() {
   MOODIST_CORE_FN(moodist_pg_get_option)
   MOODIST_CORE_FN(moodist_pg_set_option)
   MOODIST_CORE_FN(moodist_pg_all_gather)
+  MOODIST_CORE_FN(moodist_pg_all_gather_list)
   MOODIST_CORE_FN(moodist_pg_reduce_scatter)
   MOODIST_CORE_FN(moodist_pg_allreduce)
   MOODIST_CORE_FN(moodist_pg_stage_input)
@@ -240,6 +242,24 @@ public:
     return work;
   }
 
+  // wrapper/processgroup_wrapper.cc:112-129
+  c10::intrusive_ptr<c10d::Work> allgather(std::vector<std::vector<at::Tensor>>& outputLists,
+      std::vector<at::Tensor>& inputs, const c10d::AllgatherOptions& = c10d::AllgatherOptions()) override {
+    TORCH_CHECK(outputLists.size() == 1 && inputs.size() == 1);
+    auto work = c10::make_intrusive<WorkImpl>();
+    std::vector<moodist_tensor> outs;
+    for (at::Tensor& t : outputLists[0]) {
+      outs.push_back(describe(t));
+    }
+    moodist_tensor i = describe(inputs[0]);
+    moodist_work* w = nullptr;
+    check(core.moodist_pg_all_gather_list(pg_, outs.data(), outs.size(), &i, stream_of(inputs[0]), &w));
+    work->parts.push_back(w);
+    work->tensors = outputLists[0];
+    keep(inputs[0]);
+    return work;
+  }
+
   c10::intrusive_ptr<c10d::Work> _reduce_scatter_base(at::Tensor& output, at::Tensor& input,
       const c10d::ReduceScatterOptions& opts = c10d::ReduceScatterOptions()) override {
     auto work = c10::make_intrusive<WorkImpl>();
@@ -307,6 +327,23 @@ public:
     work->parts.push_back(w);
     work->tensors = tensors;
     keep(t);
+    return work;
+  }
+
+  // wrapper/processgroup_wrapper.cc:182-191
+  c10::intrusive_ptr<c10d::Work> allreduce_coalesced(std::vector<at::Tensor>& tensors,
+      const c10d::AllreduceCoalescedOptions& opts = c10d::AllreduceCoalescedOptions()) override {
+    auto work = c10::make_intrusive<WorkImpl>();
+    c10d::AllreduceOptions one;
+    one.reduceOp = opts.reduceOp;
+    for (at::Tensor& t : tensors) {
+      std::vector<at::Tensor> single{t};
+      auto part = allreduce(single, one);
+      auto* impl = static_cast<WorkImpl*>(part.get());
+      work->parts.insert(work->parts.end(), impl->parts.begin(), impl->parts.end());
+      impl->parts.clear();
+    }
+    work->tensors = tensors;
     return work;
   }
 

@@ -44,6 +44,8 @@ def core():
                                             ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p]
     L.moodist_pg_all_gather.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                         ctypes.c_void_p]
+    L.moodist_pg_all_gather_list.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p,
+                                             ctypes.c_void_p, ctypes.c_void_p]
     L.moodist_pg_allreduce.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
                                        ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p]
     L.moodist_work_wait.argtypes = [ctypes.c_void_p]
@@ -127,6 +129,18 @@ def test_argument_checks_use_the_reference_messages(core):
                                       ctypes.byref(work)) != 0
     assert core.moodist_pg_allreduce(pg, ctypes.byref(fake(7)), None, 0, None, 0.0, ctypes.byref(work)) != 0
     assert b"needs a scratch tensor of 8 elements" in core.moodist_last_error()
+    # list form of all_gather: one dense output of the input's size and dtype per rank
+    four = (type(fake(4)) * 4)(*[fake(4) for _ in range(4)])
+    three = (type(fake(4)) * 3)(*[fake(4) for _ in range(3)])
+    assert core.moodist_pg_all_gather_list(pg, three, 3, ctypes.byref(fake(4)), None, ctypes.byref(work)) != 0
+    assert b"one output tensor per rank (4), got 3" in core.moodist_last_error()
+    four[2] = fake(5)
+    assert core.moodist_pg_all_gather_list(pg, four, 4, ctypes.byref(fake(4)), None, ctypes.byref(work)) != 0
+    four[2] = fake(4, dtype=7, itemsize=8)
+    assert core.moodist_pg_all_gather_list(pg, four, 4, ctypes.byref(fake(4)), None, ctypes.byref(work)) != 0
+    four[2] = fake(4, contiguous=0)
+    assert core.moodist_pg_all_gather_list(pg, four, 4, ctypes.byref(fake(4)), None, ctypes.byref(work)) != 0
+    assert b"must be contiguous" in core.moodist_last_error()
     core.moodist_world_destroy(w)
 
 

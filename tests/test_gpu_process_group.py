@@ -216,6 +216,44 @@ def test_coalesced_variants(world, dev):
             assert torch.equal(routs[r][k], torch.full((n,), 36.0, device=dev))
 
 
+@pytest.mark.parametrize("kernel_less", [False, True])
+def test_allgather_into_a_list_of_tensors(world, dev, kernel_less):
+    # c10d's list form (reference wrapper/processgroup_wrapper.cc:112-129): outputs[j] = rank j's input.
+    # Sizes with and without a 16-byte body and tail; one output is the rank's own input (in place).
+    for pg in world:
+        pg.options().force_kernel_less = kernel_less
+    for n in (1, 7, 4096, 100003):
+        g = torch.Generator().manual_seed(n)
+        ins = [torch.randn(n, generator=g).to(dev) for _ in range(P)]
+        outs = [[ins[r] if j == r else torch.zeros(n, device=dev) for j in range(P)] for r in range(P)]
+        each_rank(world, lambda r, pg: pg.allgather([outs[r]], [ins[r]]))
+        for r in range(P):
+            for j in range(P):
+                assert torch.equal(outs[r][j], ins[j]), (n, r, j)
+
+
+def test_allgather_list_through_torch_distributed_api_shapes(world, dev):
+    # 2-d inputs, bf16: the list form keeps each output's own shape
+    ins = [torch.full((3, 5), float(r), device=dev, dtype=torch.bfloat16) for r in range(P)]
+    outs = [[torch.empty(3, 5, device=dev, dtype=torch.bfloat16) for _ in range(P)] for _ in range(P)]
+    each_rank(world, lambda r, pg: pg.allgather([outs[r]], [ins[r]]))
+    for r in range(P):
+        for j in range(P):
+            assert torch.equal(outs[r][j], ins[j])
+    with pytest.raises(RuntimeError, match="one output tensor per rank"):
+        world.groups[0].allgather([outs[0][:3]], [ins[0]])
+
+
+def test_allreduce_coalesced(world, dev):
+    # reference wrapper/processgroup_wrapper.cc:182-191: one allreduce per tensor, in order
+    sizes = (8, 1001, 4096)  # 1001 is not a multiple of 8: padded temporary
+    ts = [[torch.arange(n, device=dev, dtype=torch.float32) * (r + 1) for n in sizes] for r in range(P)]
+    each_rank(world, lambda r, pg: pg.allreduce_coalesced(ts[r]))
+    for r in range(P):
+        for k, n in enumerate(sizes):
+            assert torch.equal(ts[r][k], torch.arange(n, device=dev, dtype=torch.float32) * 36.0)
+
+
 def test_ranks_on_different_streams(world, dev):
     # each rank posts on its own stream; the launches must still see every rank's input
     n = 1 << 20
