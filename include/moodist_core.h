@@ -135,6 +135,16 @@ int moodist_op_plan_read(moodist_op* op, size_t i, int64_t out[6]);
 int moodist_op_plan_copy(moodist_op* op, int which, size_t i, int64_t* out, size_t out_len);
 /* inputs / outputs: byte size of entry i. */
 int64_t moodist_op_plan_size(moodist_op* op, int which, size_t i);
+/* The serialized list this rank would put on `receiver`'s queue during compile
+ * (core/processgroup.cc:3022-3033): a 64-bit count, then per piece, packed, little-endian:
+ *   u8 contiguous (always 0); i32 offset[ndim]; i32 shape[ndim]; u32 inputRank, outputRank,
+ *   inputIndex, outputIndex; u64 inputOffset, outputOffset (elements); u8 outputContiguous
+ * (TInput, :2735-2753, written by core/serialization.h's raw-byte serializer).  Returns the
+ * length; copies the bytes when buffer is non-NULL and capacity suffices; -1 on a bad argument. */
+int64_t moodist_op_plan_message(moodist_op* op, int receiver, void* buffer, size_t capacity);
+/* Parses such a list for `ndim` dimensions: 0, or an error with the reference deserializer's
+ * message ("Deserializer: reached end of data", "deserializeBuffer: N trailing bytes"). */
+int moodist_plan_message_check(const void* bytes, size_t length, size_t ndim);
 
 #ifdef __cplusplus
 }

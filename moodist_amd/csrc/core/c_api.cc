@@ -291,6 +291,24 @@ int moodist_op_plan_copy(moodist_op* op, int which, size_t i, int64_t* out, size
   });
 }
 
+int64_t moodist_op_plan_message(moodist_op* op, int receiver, void* buffer, size_t capacity) {
+  if (!op || receiver < 0 || receiver >= op->pg->size) {
+    return -1;
+  }
+  const std::vector<uint8_t>& bytes = op->op->wire[(size_t)op->pg->rank][(size_t)receiver];
+  if (buffer && capacity >= bytes.size()) {
+    std::memcpy(buffer, bytes.data(), bytes.size());
+  }
+  return (int64_t)bytes.size();
+}
+
+int moodist_plan_message_check(const void* bytes, size_t length, size_t ndim) {
+  return guarded([&] {
+    const uint8_t* p = (const uint8_t*)bytes;
+    check_plan_message(std::vector<uint8_t>(p, p + length), ndim);
+  });
+}
+
 int64_t moodist_op_plan_size(moodist_op* op, int which, size_t i) {
   if (!op) {
     return -1;

@@ -1,6 +1,7 @@
 #include "planner.h"
 
 #include <algorithm>
+#include <cstring>
 #include <string>
 
 namespace moodist {
@@ -92,8 +93,90 @@ struct Message { // what a sender tells a receiver about one piece (TInput, :273
   uint32_t inputRank, outputRank, inputIndex, outputIndex;
   size_t inputOffset, outputOffset; // elements
   bool outputContiguous;
-  uint32_t originInput; // the sender's own tensor the piece really lives in
 };
+
+// The bytes a sender puts on a receiver's queue (core/processgroup.cc:3022-3033).  The
+// reference's serializer writes a vector as its 64-bit length followed by the elements, and
+// every trivially copyable member as its raw bytes with no padding (core/serialization.h:148-154,
+// :263-267); TInput lists its members as contiguous, offset, shape, inputRank, outputRank,
+// inputIndex, outputIndex, inputOffset, outputOffset, outputContiguous (:2748-2751), offset and
+// shape being std::array<int, ndim>.  `contiguous` is never set and travels as 0.  One record
+// is 34 + 8*ndim bytes; the number of dimensions is not on the wire.
+template<typename T>
+void put(std::vector<uint8_t>& out, T v) {
+  const uint8_t* p = reinterpret_cast<const uint8_t*>(&v);
+  out.insert(out.end(), p, p + sizeof(T));
+}
+
+std::vector<uint8_t> encode(const std::vector<Message>& list, size_t ndim) {
+  std::vector<uint8_t> out;
+  out.reserve(8 + list.size() * (34 + 8 * ndim));
+  put<uint64_t>(out, list.size());
+  for (const Message& m : list) {
+    put<uint8_t>(out, 0);
+    for (int64_t v : m.offset) {
+      put<int32_t>(out, (int32_t)v);
+    }
+    for (int64_t v : m.shape) {
+      put<int32_t>(out, (int32_t)v);
+    }
+    put<uint32_t>(out, m.inputRank);
+    put<uint32_t>(out, m.outputRank);
+    put<uint32_t>(out, m.inputIndex);
+    put<uint32_t>(out, m.outputIndex);
+    put<uint64_t>(out, m.inputOffset);
+    put<uint64_t>(out, m.outputOffset);
+    put<uint8_t>(out, m.outputContiguous ? 1 : 0);
+  }
+  return out;
+}
+
+struct Reader {
+  const uint8_t* p;
+  size_t left;
+  template<typename T>
+  T get() {
+    if (left < sizeof(T)) {
+      throw std::runtime_error("Deserializer: reached end of data"); // core/serialization.h:287
+    }
+    T v;
+    std::memcpy(&v, p, sizeof(T));
+    p += sizeof(T);
+    left -= sizeof(T);
+    return v;
+  }
+};
+
+std::vector<Message> decode(const std::vector<uint8_t>& bytes, size_t ndim) {
+  Reader r{bytes.data(), bytes.size()};
+  const uint64_t n = r.get<uint64_t>();
+  if (n > r.left / (34 + 8 * ndim)) {
+    throw std::runtime_error("Deserializer: reached end of data");
+  }
+  std::vector<Message> list((size_t)n);
+  for (Message& m : list) {
+    (void)r.get<uint8_t>();
+    m.offset.resize(ndim);
+    m.shape.resize(ndim);
+    for (int64_t& v : m.offset) {
+      v = r.get<int32_t>();
+    }
+    for (int64_t& v : m.shape) {
+      v = r.get<int32_t>();
+    }
+    m.inputRank = r.get<uint32_t>();
+    m.outputRank = r.get<uint32_t>();
+    m.inputIndex = r.get<uint32_t>();
+    m.outputIndex = r.get<uint32_t>();
+    m.inputOffset = (size_t)r.get<uint64_t>();
+    m.outputOffset = (size_t)r.get<uint64_t>();
+    m.outputContiguous = r.get<uint8_t>() != 0;
+  }
+  if (r.left != 0) { // core/serialization.h:677-679
+    throw std::runtime_error("deserializeBuffer: " + std::to_string(r.left) + " trailing bytes");
+  }
+  return list;
+}
 
 std::vector<Slice> number_slices(const std::vector<SliceSpec>& specs, int size, size_t ndim, const char* what) {
   std::vector<uint32_t> counter((size_t)size, 0);
@@ -112,6 +195,10 @@ std::vector<Slice> number_slices(const std::vector<SliceSpec>& specs, int size, 
       if (s.offset[i] < 0 || s.shape[i] < 0) {
         throw std::runtime_error(std::string("moodist.compile_op_full: ") + what + " has a negative offset or shape");
       }
+      if (s.offset[i] > INT32_MAX || s.shape[i] > INT32_MAX) { // `int` in the reference and on the wire
+        throw std::runtime_error(std::string("moodist.compile_op_full: ") + what +
+                                 " has an offset or shape that does not fit a 32-bit int");
+      }
     }
     Slice d;
     d.rank = (uint32_t)s.rank;
@@ -127,8 +214,13 @@ std::vector<Slice> number_slices(const std::vector<SliceSpec>& specs, int size, 
 } // namespace
 
 std::vector<RankPlan> plan_redistribution(int size, const Dims& shape, size_t itemsize,
-    const std::vector<SliceSpec>& inputs_arg, const std::vector<SliceSpec>& outputs_arg) {
+    const std::vector<SliceSpec>& inputs_arg, const std::vector<SliceSpec>& outputs_arg, PlanWire* wire_out) {
   const size_t ndim = shape.size();
+  for (int64_t v : shape) {
+    if (v < 0 || v > INT32_MAX) { // dimensions are `int` in the reference and on the wire
+      throw std::runtime_error("moodist.compile_op_full: a dimension does not fit a 32-bit int");
+    }
+  }
   std::vector<Slice> inputs = number_slices(inputs_arg, size, ndim, "an input");
   std::vector<Slice> outputs = number_slices(outputs_arg, size, ndim, "an output");
 
@@ -194,7 +286,6 @@ std::vector<RankPlan> plan_redistribution(int size, const Dims& shape, size_t it
                 m.inputOffset = linear_offset(minus(y.offset, st.offset), st.shape);
                 m.outputOffset = linear_offset(minus(y.offset, dst.offset), dst.shape);
                 m.outputContiguous = whole_rows(y.shape, dst.shape);
-                m.originInput = (uint32_t)st.index;
                 mail[dst.rank][(size_t)rank].push_back(std::move(m));
               }
               continue;
@@ -210,7 +301,6 @@ std::vector<RankPlan> plan_redistribution(int size, const Dims& shape, size_t it
         m.outputIndex = dst.index;
         m.inputOffset = linear_offset(minus(x.offset, src.offset), src.shape);
         m.outputOffset = linear_offset(minus(x.offset, dst.offset), dst.shape);
-        m.originInput = (uint32_t)x.index;
         if (!inputContiguous) {
           m.inputIndex = (uint32_t)(mine.size() + staged.size());
           m.inputOffset = 0;
@@ -246,6 +336,16 @@ std::vector<RankPlan> plan_redistribution(int size, const Dims& shape, size_t it
     inputsOf[s.rank].push_back(&s);
   }
 
+  // What travels: one byte string per (sender, receiver).  The receivers below work from the
+  // decoded bytes, as a receiver in another process would.
+  PlanWire wire((size_t)size, std::vector<std::vector<uint8_t>>((size_t)size));
+  for (int receiver = 0; receiver < size; ++receiver) {
+    for (int sender = 0; sender < size; ++sender) {
+      wire[(size_t)sender][(size_t)receiver] = encode(mail[(size_t)receiver][(size_t)sender], ndim);
+    }
+  }
+  mail.clear();
+
   for (int rank = 0; rank < size; ++rank) {
     RankPlan& plan = plans[(size_t)rank];
     size_t want = 0;
@@ -254,7 +354,11 @@ std::vector<RankPlan> plan_redistribution(int size, const Dims& shape, size_t it
     }
     size_t have = 0;
     for (int sender = 0; sender < size; ++sender) {
-      for (const Message& m : mail[(size_t)rank][(size_t)sender]) {
+      for (const Message& m : decode(wire[(size_t)sender][(size_t)rank], ndim)) {
+        if (m.outputRank != (uint32_t)rank || m.inputRank != (uint32_t)sender ||
+            m.outputIndex >= outputsOf[(size_t)rank].size()) { // :3052
+          throw std::runtime_error("moodist.compile_op_full: a plan message does not belong to this rank");
+        }
         const Slice& dst = outputsOf[(size_t)rank][m.outputIndex];
         PlanRead r;
         r.rank = m.inputRank;
@@ -276,10 +380,19 @@ std::vector<RankPlan> plan_redistribution(int size, const Dims& shape, size_t it
         }
         plan.reads.push_back(r);
 
-        const Slice& src = *inputsOf[m.inputRank][m.originInput];
+        // An index past the sender's tensors names one of its staging copies; the fused
+        // transfer reads the tensor that copy would have been taken from.
+        const RankPlan& theirs = plans[m.inputRank];
+        const size_t tensors = theirs.inputs.size();
+        if (m.inputIndex >= tensors + theirs.inputCopies.size()) {
+          throw std::runtime_error("moodist.compile_op_full: a plan message names an input the sender does not have");
+        }
+        const uint32_t origin =
+            m.inputIndex < tensors ? m.inputIndex : theirs.inputCopies[m.inputIndex - tensors].index;
+        const Slice& src = *inputsOf[m.inputRank][origin];
         Transfer t;
         t.srcRank = m.inputRank;
-        t.srcInput = m.originInput;
+        t.srcInput = origin;
         t.dstOutput = m.outputIndex;
         t.shape = m.shape;
         t.srcOffset = minus(m.offset, src.offset);
@@ -293,7 +406,14 @@ std::vector<RankPlan> plan_redistribution(int size, const Dims& shape, size_t it
       throw std::runtime_error("moodist.compile_op_full: could not find input for all output elements");
     }
   }
+  if (wire_out) {
+    *wire_out = std::move(wire);
+  }
   return plans;
+}
+
+void check_plan_message(const std::vector<uint8_t>& bytes, size_t ndim) {
+  (void)decode(bytes, ndim);
 }
 
 } // namespace moodist

@@ -5,8 +5,10 @@
 // Behaviour follows the reference's compileOpFullImpl
 // (core/processgroup.cc:2761-3104) and its descriptor (core/cputhread.h:296-322).
 // The reference runs one planner per rank process and exchanges the
-// per-destination lists through queues (:3005-3077); here all ranks live in
-// one process, so one call plans every rank and the exchange is a vector.
+// per-destination lists through queues as serialized bytes (:3005-3077); here
+// all ranks live in one process, so one call plans every rank, but the lists
+// still pass through the reference's byte format between the sender half and
+// the receiver half.
 #pragma once
 
 #include <cstddef>
@@ -66,11 +68,19 @@ struct RankPlan {
   std::vector<Transfer> transfers;
 };
 
+// wire[sender][receiver]: the serialized list the sender puts on the receiver's queue
+// (core/processgroup.cc:3022-3033, format of core/serialization.h).
+using PlanWire = std::vector<std::vector<std::vector<uint8_t>>>;
+
 // Throws std::runtime_error("moodist.compile_op_full: could not find input for
 // all output elements") when some output element has no source
 // (core/processgroup.cc:3079-3081).
 std::vector<RankPlan> plan_redistribution(int size, const Dims& shape, size_t itemsize,
-    const std::vector<SliceSpec>& inputs, const std::vector<SliceSpec>& outputs);
+    const std::vector<SliceSpec>& inputs, const std::vector<SliceSpec>& outputs, PlanWire* wire = nullptr);
+
+// Parses a serialized list for `ndim` dimensions; throws the reference's deserializer errors
+// on a short buffer or trailing bytes.
+void check_plan_message(const std::vector<uint8_t>& bytes, size_t ndim);
 
 size_t dims_numel(const Dims& d);
 size_t linear_offset(const Dims& offset, const Dims& shape);

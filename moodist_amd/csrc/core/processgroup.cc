@@ -306,7 +306,8 @@ std::shared_ptr<CompiledOp> ProcessGroup::compile_op_full(const Dims& shape, int
   op->id = next_op_id++;
   op->dtype = dtype;
   op->itemsize = dtype_size(dtype);
-  op->plans = plan_redistribution(size, shape, op->itemsize, inputs, outputs);
+  op->ndim = shape.size();
+  op->plans = plan_redistribution(size, shape, op->itemsize, inputs, outputs, &op->wire);
   // The reference sizes a rank's outputs largest-first (:2999-3004) but numbers its reads by
   // listing order (:2974); the two agree only when listing order is already largest-first.
   for (int r = 0; r < size; ++r) {

@@ -64,6 +64,8 @@ struct CompiledOp {
   int dtype;
   size_t itemsize;
   std::vector<RankPlan> plans; // every rank's, computed identically by every rank
+  PlanWire wire;               // wire[sender][receiver]
+  size_t ndim = 0;
 };
 
 class ProcessGroup {

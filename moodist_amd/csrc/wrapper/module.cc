@@ -58,6 +58,7 @@ struct CoreApi {
   MOODIST_CORE_FN(moodist_op_plan_read)
   MOODIST_CORE_FN(moodist_op_plan_copy)
   MOODIST_CORE_FN(moodist_op_plan_size)
+  MOODIST_CORE_FN(moodist_op_plan_message)
 #undef MOODIST_CORE_FN
 };
 
@@ -108,6 +109,7 @@ void load_core() {
   MOODIST_CORE_FN(moodist_op_plan_read)
   MOODIST_CORE_FN(moodist_op_plan_copy)
   MOODIST_CORE_FN(moodist_op_plan_size)
+  MOODIST_CORE_FN(moodist_op_plan_message)
 #undef MOODIST_CORE_FN
   if (!core.moodist_core_check_version(MOODIST_CORE_API_VERSION)) {
     throw std::runtime_error("moodist: libmoodist.so speaks a different API version than this module");
@@ -517,6 +519,18 @@ struct CustomOpObj {
     d["outputCopies"] = copies(2);
     d["inputs"] = sizes_in;
     d["outputs"] = sizes_out;
+    // what this rank sends each receiver during compile, in the reference's byte format
+    py::list messages;
+    for (int receiver = 0;; ++receiver) {
+      const int64_t n = core.moodist_op_plan_message(op, receiver, nullptr, 0);
+      if (n < 0) {
+        break;
+      }
+      std::string bytes((size_t)n, '\0');
+      core.moodist_op_plan_message(op, receiver, bytes.data(), bytes.size());
+      messages.append(py::bytes(bytes));
+    }
+    d["messages"] = messages;
     return d;
   }
 };

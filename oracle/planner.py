@@ -13,16 +13,21 @@ core/processgroup.cc:3005-3033; here the exchange is a Python list).
               unchanged (core/cputhread.cc:5628-5672).
   shard_box() follows py/moodist/compile.py:21-59 (DTensor Shard placement ->
               offset/shape).
+  wire()      the serialized per-destination lists the ranks exchange while compiling
+              (TInput, core/processgroup.cc:2735-2753, through core/serialization.h).
 
 Pinned by: the hand-derived plan for a 4x4 row->column reshard over 2 ranks,
 the 1-D all-gather plan (reference tests/test_compile_op.py:191-222), numpy
 slicing of the global tensor for every executed plan (identity
 out[global idx] = in[global idx]), and the invariants sum(read bytes) ==
-sum(output bytes) with no output byte written twice.
+sum(output bytes) with no output byte written twice.  wire() is pinned by a byte string
+written out by hand for the 4x4 example, by the record length 34 + 8*ndim and by
+unpack(pack(x)) == x; no reference test holds serialized plans.
 
 Pure-Python loops: small cases only.
 """
 
+import struct
 from dataclasses import dataclass, field
 from typing import List
 
@@ -121,6 +126,53 @@ def plan(size, shape, itemsize, inputs_arg, outputs_arg):
     Returns one Descriptor per rank.  Reads arrive sender by sender in rank
     order (the reference's arrival order is unspecified).
     """
+    return _plan(size, shape, itemsize, inputs_arg, outputs_arg)[0]
+
+
+def wire(size, shape, itemsize, inputs_arg, outputs_arg):
+    """wire[sender][receiver]: the bytes `sender` puts on `receiver`'s queue while compiling
+    (core/processgroup.cc:3015-3033)."""
+    sent = _plan(size, shape, itemsize, inputs_arg, outputs_arg)[1]
+    return [[pack_messages(sent[s][r], len(shape)) for r in range(size)] for s in range(size)]
+
+
+def pack_messages(messages, ndim):
+    """serializeToBuffer(IVector<TInput<std::array<int, ndim>>>): the vector is its size() as a
+    size_t followed by the elements (core/serialization.h:148-154); an element writes its members
+    in the order TInput::serialize lists them (core/processgroup.cc:2748-2751), each trivially
+    copyable member as its raw object bytes, nothing between them (core/serialization.h:263-267;
+    the header says of itself "not a cross platform serializer": x86-64, little-endian, bool = 1
+    byte, int = 4, size_t = 8).  `contiguous` keeps its initialiser, false (:2737)."""
+    out = [struct.pack("<Q", len(messages))]
+    for m in messages:
+        assert len(m["offset"]) == ndim and len(m["shape"]) == ndim
+        out.append(struct.pack("<?", False))
+        out.append(struct.pack("<%di" % ndim, *m["offset"]))
+        out.append(struct.pack("<%di" % ndim, *m["shape"]))
+        out.append(struct.pack("<IIII", m["inputRank"], m["outputRank"], m["inputIndex"], m["outputIndex"]))
+        out.append(struct.pack("<QQ", m["inputOffset"], m["outputOffset"]))
+        out.append(struct.pack("<?", m["outputContiguous"]))
+    return b"".join(out)
+
+
+def unpack_messages(data, ndim):
+    """deserializeBuffer into IVector<TInput> (core/serialization.h:156-170, :671-680)."""
+    (n,), pos = struct.unpack_from("<Q", data, 0), 8
+    fmt = "<?%di%diIIIIQQ?" % (ndim, ndim)
+    assert struct.calcsize(fmt) == 34 + 8 * ndim
+    out = []
+    for _ in range(n):
+        v = struct.unpack_from(fmt, data, pos)
+        pos += struct.calcsize(fmt)
+        out.append({"offset": list(v[1:1 + ndim]), "shape": list(v[1 + ndim:1 + 2 * ndim]),
+                    "inputRank": v[-7], "outputRank": v[-6], "inputIndex": v[-5], "outputIndex": v[-4],
+                    "inputOffset": v[-3], "outputOffset": v[-2], "outputContiguous": v[-1]})
+    if pos != len(data):
+        raise PlanError("deserializeBuffer: %d trailing bytes" % (len(data) - pos))
+    return out
+
+
+def _plan(size, shape, itemsize, inputs_arg, outputs_arg):
     ndim = len(shape)
     for _, off, shp in list(inputs_arg) + list(outputs_arg):
         assert len(off) == ndim and len(shp) == ndim
@@ -218,7 +270,7 @@ def plan(size, shape, itemsize, inputs_arg, outputs_arg):
                 op.reads.append(r)
         if readNumel != total:  # :3079-3081
             raise PlanError("moodist.compile_op_full: could not find input for all output elements")
-    return descs
+    return descs, sent
 
 
 def _box_view(flat_bytes, tensor_shape, itemsize, offset, shape):

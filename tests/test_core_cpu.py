@@ -198,6 +198,8 @@ def test_cpp_planner_matches_oracle_planner(case):
         assert got["inputCopies"] == [(c.index, c.offset, c.shape) for c in d.inputCopies]
         assert got["outputCopies"] == [(c.index, c.offset, c.shape) for c in d.outputCopies]
         assert got["inputs"] == d.inputs and got["outputs"] == d.outputs
+        # what rank r sends every receiver, byte for byte
+        assert got["messages"] == planner.wire(size, shape, np.dtype(dt).itemsize, inputs, outputs)[r]
 
 
 def test_cpp_planner_random_boxes_match_oracle():
@@ -221,6 +223,7 @@ def test_cpp_planner_random_boxes_match_oracle():
             shp = [int(rng.randint(1, s - o + 1)) for s, o in zip(shape, off)]
             outputs.append((r, off, shp))
         want = planner.plan(size, shape, 2, inputs, outputs)
+        wire = planner.wire(size, shape, 2, inputs, outputs)
         world = moodist_amd.LocalWorld(size, 0)
         for r, pg in enumerate(world):
             got = pg.compile_op_full(shape, torch.bfloat16, inputs, outputs).plan()
@@ -228,6 +231,32 @@ def test_cpp_planner_random_boxes_match_oracle():
                                     for x in want[r].reads], (trial, r)
             assert got["inputCopies"] == [(c.index, c.offset, c.shape) for c in want[r].inputCopies]
             assert got["outputCopies"] == [(c.index, c.offset, c.shape) for c in want[r].outputCopies]
+            assert got["messages"] == wire[r], (trial, r)
+
+
+def test_plan_messages_hand_derived_bytes_and_deserializer_errors(core):
+    from test_oracle_copy import WIRE_4X4_COL_TO_ROW_R0_TO_R1, WIRE_4X4_R0_TO_R1, WIRE_4X4_R1_TO_R0
+
+    rows = [(0, [0, 0], [2, 4]), (1, [2, 0], [2, 4])]
+    cols = [(0, [0, 0], [4, 2]), (1, [0, 2], [4, 2])]
+    world = moodist_amd.LocalWorld(2, 0)
+    ops = [pg.compile_op_full([4, 4], torch.float32, rows, cols) for pg in world]
+    assert ops[1].plan()["messages"][0] == WIRE_4X4_R1_TO_R0
+    assert ops[0].plan()["messages"][1] == WIRE_4X4_R0_TO_R1
+    ops = [pg.compile_op_full([4, 4], torch.float32, cols, rows) for pg in world]
+    assert ops[0].plan()["messages"][1] == WIRE_4X4_COL_TO_ROW_R0_TO_R1
+
+    core.moodist_plan_message_check.argtypes = [ctypes.c_char_p, ctypes.c_size_t, ctypes.c_size_t]
+    m = WIRE_4X4_R1_TO_R0
+    assert core.moodist_plan_message_check(m, len(m), 2) == 0
+    assert core.moodist_plan_message_check(m + b"\0", len(m) + 1, 2) != 0
+    assert core.moodist_last_error() == b"deserializeBuffer: 1 trailing bytes"  # core/serialization.h:677-679
+    assert core.moodist_plan_message_check(m, len(m) - 1, 2) != 0
+    assert core.moodist_last_error() == b"Deserializer: reached end of data"  # :287
+    assert core.moodist_plan_message_check(m, len(m), 3) != 0  # the dimension count is not on the wire
+    assert core.moodist_plan_message_check(m, 4, 2) != 0
+    huge = (2**63).to_bytes(8, "little")
+    assert core.moodist_plan_message_check(huge, 8, 2) != 0
 
 
 def test_planner_errors():

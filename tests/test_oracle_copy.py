@@ -132,6 +132,59 @@ def test_planner_hand_derived_4x4_row_to_column():
     _check_outputs(outputs, outs, G, np.float32)
 
 
+# Written out by hand from the member order of TInput (core/processgroup.cc:2735-2753) and the
+# raw-byte serializer (core/serialization.h:148-154, :263-267): u64 count, then u8 contiguous,
+# i32 offset[2], i32 shape[2], u32 inputRank, outputRank, inputIndex, outputIndex,
+# u64 inputOffset, outputOffset, u8 outputContiguous.
+WIRE_4X4_R1_TO_R0 = bytes.fromhex(
+    "0100000000000000"          # one piece
+    "00"                        # contiguous: never set
+    "02000000" "00000000"       # offset [2, 0] (global coordinates)
+    "02000000" "02000000"       # shape [2, 2]
+    "01000000" "00000000"       # inputRank 1, outputRank 0
+    "01000000" "00000000"       # inputIndex 1 (the sender's first staging copy), outputIndex 0
+    "0000000000000000"          # inputOffset 0 elements
+    "0400000000000000"          # outputOffset linearOffset([2,0],[4,2]) = 4 elements
+    "01")                       # outputContiguous
+WIRE_4X4_R0_TO_R1 = bytes.fromhex(
+    "0100000000000000" "00" "00000000" "02000000" "02000000" "02000000"
+    "00000000" "01000000" "02000000" "00000000" "0000000000000000" "0000000000000000" "01")
+# column -> row, sender 0 to receiver 1: piece [2,0]+[2,2] is contiguous in the sender's [4,2]
+# tensor at element 4 and not contiguous in the receiver's [2,4] tensor
+WIRE_4X4_COL_TO_ROW_R0_TO_R1 = bytes.fromhex(
+    "0100000000000000" "00" "02000000" "00000000" "02000000" "02000000"
+    "00000000" "01000000" "00000000" "00000000" "0400000000000000" "0000000000000000" "00")
+
+
+def test_plan_wire_bytes_hand_derived():
+    inputs = [(0, [0, 0], [2, 4]), (1, [2, 0], [2, 4])]
+    outputs = [(0, [0, 0], [4, 2]), (1, [0, 2], [4, 2])]
+    w = planner.wire(2, [4, 4], 4, inputs, outputs)
+    assert w[1][0] == WIRE_4X4_R1_TO_R0 and len(w[1][0]) == 8 + 34 + 8 * 2
+    assert w[0][1] == WIRE_4X4_R0_TO_R1
+    w = planner.wire(2, [4, 4], 4, outputs, inputs)
+    assert w[0][1] == WIRE_4X4_COL_TO_ROW_R0_TO_R1
+    # a rank with nothing for a receiver still sends an empty list: just the count
+    w = planner.wire(2, [8], 4, [(0, [0], [8])], [(1, [0], [8])])
+    assert w[1][0] == w[1][1] == w[0][0] == bytes(8) and len(w[0][1]) == 8 + 34 + 8
+
+
+def test_plan_wire_round_trip_and_record_length():
+    rng = np.random.RandomState(3)
+    for ndim in (1, 2, 3, 10):
+        msgs = [{"offset": [int(v) for v in rng.randint(0, 2**31 - 1, ndim)],
+                 "shape": [int(v) for v in rng.randint(0, 2**31 - 1, ndim)],
+                 "inputRank": int(rng.randint(0, 2**31)), "outputRank": int(rng.randint(0, 64)),
+                 "inputIndex": int(rng.randint(0, 9)), "outputIndex": int(rng.randint(0, 9)),
+                 "inputOffset": int(rng.randint(0, 2**62)), "outputOffset": int(rng.randint(0, 2**62)),
+                 "outputContiguous": bool(rng.randint(0, 2))} for _ in range(5)]
+        data = planner.pack_messages(msgs, ndim)
+        assert len(data) == 8 + 5 * (34 + 8 * ndim)
+        assert planner.unpack_messages(data, ndim) == msgs
+        with pytest.raises(planner.PlanError, match="1 trailing bytes"):
+            planner.unpack_messages(data + b"\0", ndim)
+
+
 def test_planner_column_to_row_uses_output_copies():
     inputs = [(0, [0, 0], [4, 2]), (1, [0, 2], [4, 2])]
     outputs = [(0, [0, 0], [2, 4]), (1, [2, 0], [2, 4])]
