@@ -12,6 +12,7 @@ from . import _abi  # noqa: F401
 from ._abi import MoodistError  # noqa: F401
 from .compile import compile_op  # noqa: F401
 from .options import MoodistOptions, MoodistOptionsContext  # noqa: F401
-from .process_group import LocalWorld, MoodistProcessGroup  # noqa: F401
+from .process_group import (LocalWorld, MoodistProcessGroup, PreferKernelLessContext,  # noqa: F401
+                            find_process_group)
 
 __version__ = "0.1.0"

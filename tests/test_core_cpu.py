@@ -368,9 +368,35 @@ def test_process_group_is_a_c10d_process_group():
     for r, pg in enumerate(world):
         assert isinstance(pg.c10d, dist.ProcessGroup)
         assert pg.rank() == r and pg.size() == 3
-        assert pg.moodist_name() == "moodist-local-%d-of-3" % r
+        assert pg.moodist_name() == "moodist-local-%d-of-3-world%d" % (r, world.serial)
+        assert moodist_amd.find_process_group(pg.moodist_name()) is pg
     with pytest.raises(RuntimeError, match="send is not supported"):
         world.groups[0].send([torch.zeros(1)], 1, 0)
+
+
+def test_reference_constructor_joins_ranks_through_the_store():
+    # reference: moodist.MoodistProcessGroup(store, rank, size) (wrapper/module.cc:547-566); the ranks that
+    # share a store object are the ranks of one group
+    import torch.distributed as dist
+
+    store = dist.HashStore()
+    pgs = [moodist_amd.MoodistProcessGroup(store, r, 4) for r in range(4)]
+    assert [pg.rank() for pg in pgs] == [0, 1, 2, 3] and all(pg.size() == 4 for pg in pgs)
+    assert len({id(pg.world) for pg in pgs}) == 1
+    assert moodist_amd.MoodistProcessGroup(store, 2, 4) is pgs[2]
+    other = moodist_amd.MoodistProcessGroup(dist.HashStore(), 0, 4)
+    assert other.world is not pgs[0].world
+    with pytest.raises(ValueError, match="already serves a group of 4 ranks"):
+        moodist_amd.MoodistProcessGroup(store, 0, 8)
+    with pytest.raises(ValueError, match="outside a group"):
+        moodist_amd.MoodistProcessGroup(store, 4, 4)
+    # prefer_kernel_less as setter and as context manager (py/moodist/backend.py:17-43)
+    pg = pgs[0]
+    pg.prefer_kernel_less(True)
+    assert pg.get_prefer_kernel_less() is True
+    with pg.prefer_kernel_less(False):
+        assert pg.get_prefer_kernel_less() is False
+    assert pg.get_prefer_kernel_less() is True
 
 
 def test_compile_op_accepts_dtensor_like_specs():

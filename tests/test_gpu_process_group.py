@@ -36,6 +36,20 @@ def test_pg_creation(world):
         assert pg.rank() == r and pg.size() == P
 
 
+def test_groups_built_the_reference_way(dev):
+    # reference tests/framework.py builds each rank's group as MoodistProcessGroup(store, rank, size)
+    store = dist.HashStore()
+    pgs = [moodist_amd.MoodistProcessGroup(store, r, P) for r in range(P)]
+    ins = [torch.full((1024,), float(r + 1), device=dev) for r in range(P)]
+    outs = [torch.zeros(128, device=dev) for _ in range(P)]
+    works = [pg._reduce_scatter_base(outs[r], ins[r]) for r, pg in enumerate(pgs)]
+    for w in works:
+        w.wait()
+    torch.cuda.synchronize()
+    for r in range(P):
+        assert torch.equal(outs[r], torch.full((128,), 36.0, device=dev))
+
+
 @pytest.mark.parametrize("kernel_less", [False, True])
 def test_pg_allgather_base(world, dev, kernel_less):
     # reference tests/test_processgroup.py:21-48 (kernel and kernel-less modes)
