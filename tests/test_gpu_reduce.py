@@ -168,6 +168,40 @@ def test_in_place_on_own_chunk(dev):
             assert torch.equal(d[j].cpu(), srcs[j])  # sources untouched
 
 
+def test_direct_method_chunk_loop_and_final_rows(dev):
+    # The multi-node method (core/reduce_scatter_direct.cc:165-177): for every remote destination
+    # `source`, send[n] = in_self[source] (+) peers' in[source], cut into at most four chunks of
+    # chunkSize bytes (core/processgroup.cc:1496-1503); the receiver then reduces its K rows
+    # (:1599-1616).  Each chunk is one mdh_reduce call on offset pointers; the result must equal
+    # the unchunked fold bit for bit, and the final K-row reduction must equal a fold of folds.
+    local, nodes, rank = 4, 3, 1
+    n = 200000 + 3  # 800,012 bytes: four ragged chunks, the last one short
+    itemsize = 4
+    nbytes = n * itemsize
+    chunks = max(min(nbytes // 131072, 4), 1)
+    chunk_size = ((nbytes + chunks - 1) // chunks + 4095) // 4096 * 4096
+    chunks = (nbytes + chunk_size - 1) // chunk_size
+    assert chunks == 4 and chunk_size % 16 == 0
+    world = local * nodes
+    # inputs of this node's `local` ranks: [world, n] each
+    ins = [torch.stack(random_sources(world, n, torch.float32, seed=100 + r)) for r in range(local)]
+    d = [x.to(dev) for x in ins]
+    send = torch.zeros(world, n, device=dev)
+    for dest in range(world):
+        for c in range(chunks):
+            lo = c * chunk_size // itemsize
+            hi = min((c + 1) * chunk_size // itemsize, n)
+            gpu_reduce([x[dest, lo:hi] for x in d], rank, send[dest, lo:hi], oracle.OP_SUM)
+        want = oracle.reduce([bits(x[dest]) for x in ins], rank, oracle.DT_F32, oracle.OP_SUM)
+        assert same_bits(bits(send[dest]), want), dest
+    # final step on a receiver: rows = [received partials..., own, local peers...], reduced in row order
+    rows = send[:5]
+    out = torch.zeros(n, device=dev)
+    gpu_reduce([rows[k] for k in range(5)], 0, out, oracle.OP_SUM)
+    want = oracle.reduce([bits(rows[k]) for k in range(5)], 0, oracle.DT_F32, oracle.OP_SUM)
+    assert same_bits(bits(out), want)
+
+
 def test_sources_are_not_modified_and_zero_numel_is_a_no_op(dev):
     srcs = random_sources(4, 1000, torch.float32, seed=9)
     d = [s.to(dev) for s in srcs]
