@@ -2,8 +2,9 @@
 // as the library's kernels (256 lanes x U sub-tiles x 16 bytes per workgroup,
 // buffer addressing): read only, write only, copy in one kernel, a read kernel
 // followed by a write kernel, eight streams read only, and eight streams folded
-// into one written stream under several cache policies.  These are the
-// ceilings the kernels' measured rates are judged against.
+// into one written stream under several cache policies, plus the period of
+// back-to-back empty launches.  These are the ceilings the kernels' measured
+// rates are judged against.
 //
 //   hbm_ceilings [MiB per stream, default 16]
 //
@@ -82,6 +83,8 @@ __global__ __launch_bounds__(256) void fill_kernel(char* dst, size_t ntiles) {
   }
 }
 
+__global__ __launch_bounds__(256) void empty_kernel(const char*, size_t, char*, size_t) {}
+
 int main(int argc, char** argv) {
   const size_t mib = argc > 1 ? (size_t)std::atol(argv[1]) : 16;
   const size_t stream = mib << 20; // bytes per stream
@@ -115,6 +118,23 @@ int main(int argc, char** argv) {
   auto set = [&](int s) { return buf + set_bytes * s; };
 
   std::printf("%zu MiB per stream, %d buffer sets of %zu MiB\n", mib, kSets, set_bytes >> 20);
+  {
+    // what a launch costs before it moves a byte: back-to-back empty kernels of the headline grid
+    const int iters = 2000;
+    for (int i = 0; i < 50; ++i) {
+      hipLaunchKernelGGL(empty_kernel, dim3(1024), dim3(256), 0, 0, buf, 0, buf, 0);
+    }
+    CHECK(hipDeviceSynchronize());
+    CHECK(hipEventRecord(e0, 0));
+    for (int i = 0; i < iters; ++i) {
+      hipLaunchKernelGGL(empty_kernel, dim3(1024), dim3(256), 0, 0, buf, 0, buf, 0);
+    }
+    CHECK(hipEventRecord(e1, 0));
+    CHECK(hipEventSynchronize(e1));
+    float ms;
+    CHECK(hipEventElapsedTime(&ms, e0, e1));
+    std::printf("%-58s %9.2f us per launch\n", "empty kernel, 1024 workgroups, back to back", ms * 1e3 / iters);
+  }
   const size_t whole = stream * 8;                 // the eight streams taken as one region
   const size_t t4 = 256 * 4 * 16, t1 = 256 * 16;
   run("read only, one stream of 8x, nt loads", (double)whole,
