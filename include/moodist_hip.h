@@ -149,9 +149,11 @@ int mdh_copy_boxes(const mdh_box* boxes, int nboxes, int itemsize, void* stream)
 
 /*
  * Launch-shape knobs, for measurement; 0 (the default) lets the library choose
- * by size.  Names: "reduce_unroll" (1,2,4,8),
- * "reduce_max_blocks" (0 = one tile per workgroup), "copy_unroll" (1,2,4,8;
- * contiguous segments), "box_unroll" (1,2,4,8; strided boxes), "copy_max_blocks".  Returns MDH_EINVAL for an unknown name or value.
+ * by size.  Names: "reduce_unroll" (sub-tiles per lane: 1, 2, 4; 8 is taken as 4),
+ * "reduce_max_blocks" (0 = one tile per workgroup), "reduce_wg_per_cu" (1..8
+ * caps the workgroups resident on a CU, 9 = never cap), "copy_unroll" (1, 2,
+ * 4, 8; contiguous segments), "box_unroll" (1, 2, 4, 8; strided boxes),
+ * "copy_max_blocks", "copy_wg_per_cu" (2..8, 9 = never cap).  Returns MDH_EINVAL for an unknown name or value.
  * No counterpart in the reference, whose grid is fixed at 4/16/64 blocks
  * (core/kernels.cc:547-556).
  */

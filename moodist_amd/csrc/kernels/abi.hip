@@ -71,11 +71,17 @@ int* knob(const char* name) {
   if (!std::strcmp(name, "reduce_max_blocks")) {
     return &t.reduce_max_blocks;
   }
+  if (!std::strcmp(name, "reduce_wg_per_cu")) {
+    return &t.reduce_wg_per_cu;
+  }
   if (!std::strcmp(name, "copy_unroll")) {
     return &t.copy_unroll;
   }
   if (!std::strcmp(name, "box_unroll")) {
     return &t.box_unroll;
+  }
+  if (!std::strcmp(name, "copy_wg_per_cu")) {
+    return &t.copy_wg_per_cu;
   }
   if (!std::strcmp(name, "copy_max_blocks")) {
     return &t.copy_max_blocks;
@@ -96,7 +102,7 @@ extern "C" int mdh_set_tuning(const char* name, int value) {
       mdh::set_error("mdh_set_tuning: %s does not take %d", name, value);
       return MDH_EINVAL;
     }
-  } else if (value < 0) {
+  } else if (value < 0 || (std::strstr(name, "wg_per_cu") && value > 9)) {
     mdh::set_error("mdh_set_tuning: %s does not take %d", name, value);
     return MDH_EINVAL;
   }

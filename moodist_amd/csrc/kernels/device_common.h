@@ -82,11 +82,17 @@ int check_launch(const char* what);
 struct Tuning {
   int reduce_unroll = 0;
   int reduce_max_blocks = 0;
+  int reduce_wg_per_cu = 0; // cap on resident workgroups per CU (1..8; 9 = none), through an unused LDS allocation
   int copy_unroll = 0; // contiguous segments
   int box_unroll = 0;  // strided boxes
   int copy_max_blocks = 0;
+  int copy_wg_per_cu = 0; // as reduce_wg_per_cu, for the copy kernels
 };
 Tuning& tuning();
+
+// An unused dynamic LDS allocation of this size lets exactly n workgroups share a CU's 160 KiB
+// (index n): the only handle a launch has on how many workgroups a CU holds at once.
+constexpr size_t kLdsForCap[9] = {0, 98304, 65536, 49152, 40960, 32768, 27136, 23296, 20480};
 
 // Sub-tiles per lane.  More sub-tiles mean more loads in flight per lane and longer contiguous
 // pieces per workgroup (faster once the chip is full: 23.6 us with four against 28.5 us with one

@@ -74,12 +74,11 @@ struct Traits<bf16_t> {
   }
   // round to nearest even; NaN stays a quiet NaN
   static __device__ __forceinline__ uint16_t narrow(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) {
-      return (uint16_t)((u >> 16) | 0x0040u);
-    }
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (uint16_t)(u >> 16);
+    // both candidates are computed and one is selected: no divergent branch per element
+    const uint32_t u = __float_as_uint(f);
+    const uint32_t rounded = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+    const uint32_t quiet = (u >> 16) | 0x0040u;
+    return (uint16_t)((u & 0x7fffffffu) > 0x7f800000u ? quiet : rounded);
   }
   static __device__ __forceinline__ float premul(float a, float s) {
     return widen(narrow(a * s));
@@ -202,6 +201,11 @@ __device__ __forceinline__ void fold_chunk(const ReduceArgs& a, int j0, uint64_t
         }
       }
     }
+    if constexpr (sizeof(elem_t) == 2) {
+      // One source at a time: left alone, the scheduler widens every 16-bit value of the chunk
+      // to fp32 before the first add, which doubles the registers the chunk occupies.
+      __builtin_amdgcn_sched_barrier(0);
+    }
   }
 }
 
@@ -214,7 +218,6 @@ __device__ __forceinline__ void reduce_one_elem(const ReduceArgs& a, int nsrc, u
   if (a.mode == kPremul) {
     acc = Tr::premul(acc, a.scale);
   }
-#pragma unroll 4
   for (int j = 1; j < nsrc; ++j) {
     acc_t x = Tr::widen(((const elem_t*)a.src[j])[i]);
     if (a.mode == kPremul) {
@@ -225,7 +228,7 @@ __device__ __forceinline__ void reduce_one_elem(const ReduceArgs& a, int nsrc, u
   ((elem_t*)a.dst)[i] = Tr::template finish<F>(acc, a.mode, a.scale);
 }
 
-template<typename T, int F, int NSRC, int U, int MODE>
+template<typename T, int F, int U, int MODE>
 __device__ __forceinline__ void reduce_tile(const ReduceArgs& a, int nsrc, uint64_t tile_byte, uint32_t tile_bytes) {
   using Tr = Traits<T>;
   using elem_t = typename Tr::elem_t;
@@ -234,43 +237,34 @@ __device__ __forceinline__ void reduce_tile(const ReduceArgs& a, int nsrc, uint6
   constexpr int CH = 8;
   const uint32_t lane_byte = threadIdx.x * 16;
   acc_t acc[U][N];
-  if constexpr (NSRC != 0) {
-    // compile-time source count: fully unrolled chunks
-    static_assert(NSRC % CH == 0, "unrolled source counts are multiples of the chunk");
-#pragma unroll
-    for (int j0 = 0; j0 < NSRC; j0 += CH) {
-      fold_chunk<T, F, CH, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
-    }
-  } else {
-    int j0 = 0;
-    for (; nsrc - j0 >= CH; j0 += CH) {
-      fold_chunk<T, F, CH, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
-    }
-    switch (nsrc - j0) {
-    case 1:
-      fold_chunk<T, F, 1, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
-      break;
-    case 2:
-      fold_chunk<T, F, 2, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
-      break;
-    case 3:
-      fold_chunk<T, F, 3, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
-      break;
-    case 4:
-      fold_chunk<T, F, 4, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
-      break;
-    case 5:
-      fold_chunk<T, F, 5, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
-      break;
-    case 6:
-      fold_chunk<T, F, 6, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
-      break;
-    case 7:
-      fold_chunk<T, F, 7, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
-      break;
-    default:
-      break;
-    }
+  int j0 = 0;
+  for (; nsrc - j0 >= CH; j0 += CH) {
+    fold_chunk<T, F, CH, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
+  }
+  switch (nsrc - j0) {
+  case 1:
+    fold_chunk<T, F, 1, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
+    break;
+  case 2:
+    fold_chunk<T, F, 2, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
+    break;
+  case 3:
+    fold_chunk<T, F, 3, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
+    break;
+  case 4:
+    fold_chunk<T, F, 4, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
+    break;
+  case 5:
+    fold_chunk<T, F, 5, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
+    break;
+  case 6:
+    fold_chunk<T, F, 6, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
+    break;
+  case 7:
+    fold_chunk<T, F, 7, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
+    break;
+  default:
+    break;
   }
   const __amdgpu_buffer_rsrc_t rd = tile_rsrc((const char*)a.dst + tile_byte, tile_bytes);
   u32x4 out[U];
@@ -279,7 +273,7 @@ __device__ __forceinline__ void reduce_tile(const ReduceArgs& a, int nsrc, uint6
     elem_t e[N];
 #pragma unroll
     for (int i = 0; i < N; ++i) {
-      e[i] = Tr::template finish<F>(acc[u][i], MODE, a.scale);
+      e[i] = Tr::template finish<F>(acc[u][i], MODE == kPremul ? (int)kPremul : a.mode, a.scale);
     }
     __builtin_memcpy(&out[u], e, 16);
   }
@@ -296,9 +290,9 @@ __device__ __forceinline__ void reduce_tile(const ReduceArgs& a, int nsrc, uint6
 // workgroups round-robin.  Pointers need only element alignment: gfx950's
 // 16-byte buffer accesses take any byte address.  Elements past the last whole
 // vector (fewer than 16 bytes) are folded by workgroup 0.
-template<typename T, int F, int NSRC, int U>
+template<typename T, int F, int U, bool PREMUL>
 __global__ __launch_bounds__(kBlock) void reduce_vec_kernel(ReduceArgs a) {
-  const int nsrc = NSRC ? NSRC : a.nsrc;
+  const int nsrc = a.nsrc;
   constexpr uint64_t tile_bytes = (uint64_t)kBlock * U * 16;
   const uint64_t body_bytes = a.nvec * 16;
   const uint64_t ntiles = (body_bytes + tile_bytes - 1) / tile_bytes;
@@ -306,14 +300,11 @@ __global__ __launch_bounds__(kBlock) void reduce_vec_kernel(ReduceArgs a) {
     const uint64_t tile_byte = tile * tile_bytes;
     const uint64_t left = body_bytes - tile_byte;
     const uint32_t n = (uint32_t)(left < tile_bytes ? left : tile_bytes);
-    // the mode is wave-uniform: one branch per tile keeps the scale multiplies out of the plain path
-    if (F != kSum || a.mode == kPlain) {
-      reduce_tile<T, F, NSRC, U, kPlain>(a, nsrc, tile_byte, n);
-    } else if (a.mode == kAvg) {
-      reduce_tile<T, F, NSRC, U, kAvg>(a, nsrc, tile_byte, n);
-    } else {
-      reduce_tile<T, F, NSRC, U, kPremul>(a, nsrc, tile_byte, n);
-    }
+    // PREMUL_SUM is a kernel of its own: for 16-bit types every source element is rounded to the
+    // element type after the multiply, which takes several times the registers of the plain
+    // fold, and a kernel's register budget is that of its hungriest path.  AVG is the plain
+    // fold with one more multiply when the result is written (a wave-uniform test there).
+    reduce_tile<T, F, U, PREMUL ? kPremul : kPlain>(a, nsrc, tile_byte, n);
   }
   if (blockIdx.x == 0) {
     const uint64_t i = a.nvec * per_vec<T>() + threadIdx.x;
@@ -323,21 +314,51 @@ __global__ __launch_bounds__(kBlock) void reduce_vec_kernel(ReduceArgs a) {
   }
 }
 
-template<typename T, int F, int NSRC>
+struct LaunchShape {
+  int unroll;    // sub-tiles per lane: 1, 2 or 4
+  int wg_per_cu; // 0 = as many as the registers allow
+};
+
+// Chosen by measurement on MI355X (TB/s of algorithmic bytes on one box; sub-tiles/workgroups
+// per CU, "-" = no cap):
+//   fp32  8 x 16 MiB   4/-: 6.34   2/-: 5.26   1/2: 5.36   2/2: 5.56
+//   fp32  8 x 32 MiB   4/-: 6.40   1/2: 6.08        8 x 48 MiB   4/-: 6.37   1/2: 6.52
+//   fp32  8 x 64 MiB   4/-: 6.34   1/2: 6.56        8 x 128 MiB  4/-: 6.30   1/2: 6.68
+//   fp32 16 x 32 MiB   4/-: 6.40   1/2: 6.23       16 x 48 MiB   4/-: 6.30   1/2: 6.69
+//   fp32 32 x 64 MiB   4/-: 5.97   1/2: 6.53       64 x 64 MiB   4/-: 6.42   1/2: 6.55
+//   bf16 16 x 16 MiB   4/-: 6.27   1/2: 5.35       16 x 64 MiB   4/-: 6.13   1/2: 6.64
+//   bf16  8 x 16 MiB   4/-: 6.10   2/2: 5.54        8 x 64 MiB   4/-: 6.32   2/2: 6.61   1/2: 6.08
+//   fp16  8 x 64 MiB   4/-: 6.30   1/2: 6.47   2/2: 5.96
+//   fp32  4 x 32 MiB   4/-: 6.48   1/2: 5.21   (few sources: a cap starves the CU)
+// Four sub-tiles and no cap is best or equal below about 48 MiB per source and with fewer
+// than eight sources.  Above that a launch spends most of its time in a steady state in
+// which reads and writes interleave at the DRAM, and two workgroups per CU with eight loads
+// in flight per lane do better (bf16 with eight or nine sources: sixteen).
+template<typename T, bool PREMUL>
+LaunchShape choose_shape(const ReduceArgs& a) {
+  const Tuning& t = tuning();
+  constexpr bool half = sizeof(typename Traits<T>::elem_t) == 2;
+  LaunchShape s{auto_unroll(a.nvec, 4), 0};
+  if (PREMUL && half) {
+    s.unroll = 1; // the per-element rounding of PREMUL_SUM fills the register file on its own
+  } else if (!PREMUL && a.nvec >= ((uint64_t)48 << 20) / 16 && a.nsrc >= 8) {
+    s.unroll = (std::is_same_v<T, bf16_t> && a.nsrc < 10) ? 2 : 1;
+    s.wg_per_cu = 2;
+  }
+  if (t.reduce_unroll) {
+    s.unroll = t.reduce_unroll > 4 ? 4 : t.reduce_unroll;
+  }
+  if (t.reduce_wg_per_cu) {
+    s.wg_per_cu = t.reduce_wg_per_cu > 8 ? 0 : t.reduce_wg_per_cu; // 9 = no cap
+  }
+  return s;
+}
+
+template<typename T, int F, bool PREMUL = false>
 int launch_vec(const ReduceArgs& a, hipStream_t stream) {
   const Tuning& t = tuning();
-  // 16-bit types widen every vector to eight fp32 accumulators: two sub-tiles at most, and one
-  // when sixteen sources are unrolled (their loads alone fill the register budget; measured
-  // 6.4 TB/s against 5.3 TB/s with two on the bf16 sixteen-source workload).
-  int U = t.reduce_unroll ? t.reduce_unroll : auto_unroll(a.nvec, 4);
-  if (sizeof(typename Traits<T>::elem_t) == 2) {
-    U = U > 2 ? 2 : U;
-    if (NSRC >= 16) {
-      U = 1;
-    }
-  } else if (U > 4 && NSRC != 8) {
-    U = 4; // eight sub-tiles exist only for the unrolled eight-source kernel (64 loads in flight)
-  }
+  const LaunchShape shape = choose_shape<T, PREMUL>(a);
+  const int U = shape.unroll;
   const uint64_t tile_vecs = (uint64_t)kBlock * U;
   uint64_t ntiles = (a.nvec + tile_vecs - 1) / tile_vecs;
   if (ntiles == 0) {
@@ -351,33 +372,43 @@ int launch_vec(const ReduceArgs& a, hipStream_t stream) {
     grid = 0x7fffffffull;
   }
   dim3 g((unsigned)grid), b(kBlock);
+  const size_t lds = kLdsForCap[shape.wg_per_cu];
+#define MDH_LAUNCH_REDUCE(UU)                                                                            \
+  do {                                                                                                   \
+    auto* fn = reduce_vec_kernel<T, F, UU, PREMUL>;                                                      \
+    if (lds > 65536) {                                                                                   \
+      /* more than 64 KiB of dynamic LDS has to be allowed once per kernel */                            \
+      static bool raised = false;                                                                        \
+      if (!raised) {                                                                                     \
+        if (hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) { \
+          (void)hipGetLastError();                                                                       \
+          set_error("reduce_vec_kernel: the device refused %zu bytes of dynamic LDS", lds);              \
+          return MDH_ELAUNCH;                                                                            \
+        }                                                                                                \
+        raised = true;                                                                                   \
+      }                                                                                                  \
+    }                                                                                                    \
+    hipLaunchKernelGGL(fn, g, b, lds, stream, a);                                                        \
+  } while (0)
   if (U == 1) {
-    hipLaunchKernelGGL((reduce_vec_kernel<T, F, NSRC, 1>), g, b, 0, stream, a);
+    MDH_LAUNCH_REDUCE(1);
   } else if (U == 2) {
-    hipLaunchKernelGGL((reduce_vec_kernel<T, F, NSRC, 2>), g, b, 0, stream, a);
-  } else if (U == 4) {
-    hipLaunchKernelGGL((reduce_vec_kernel<T, F, NSRC, 4>), g, b, 0, stream, a);
+    MDH_LAUNCH_REDUCE(2);
   } else {
-    if constexpr (NSRC == 8 && sizeof(typename Traits<T>::elem_t) >= 4) {
-      hipLaunchKernelGGL((reduce_vec_kernel<T, F, NSRC, 8>), g, b, 0, stream, a);
-    }
+    MDH_LAUNCH_REDUCE(4);
   }
+#undef MDH_LAUNCH_REDUCE
   return check_launch("reduce_vec_kernel");
 }
 
 template<typename T, int F>
 int launch(const ReduceArgs& a, hipStream_t stream) {
-  // Source counts with a fully unrolled instantiation; anything else takes
-  // the run-time loop over chunks of eight.
-  if constexpr (std::is_same_v<T, float> || std::is_same_v<T, bf16_t>) {
-    if (a.nsrc == 8) {
-      return launch_vec<T, F, 8>(a, stream);
-    }
-    if (a.nsrc == 16) {
-      return launch_vec<T, F, 16>(a, stream);
+  if constexpr (F == kSum && (std::is_floating_point_v<T> || sizeof(typename Traits<T>::elem_t) == 2)) {
+    if (a.mode == kPremul) {
+      return launch_vec<T, F, true>(a, stream);
     }
   }
-  return launch_vec<T, F, 0>(a, stream);
+  return launch_vec<T, F>(a, stream);
 }
 
 // One entry per (element type, fold), each instantiated in its own object

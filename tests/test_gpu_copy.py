@@ -105,13 +105,14 @@ def test_gather_2d_against_oracle(dev):
 
 
 @pytest.mark.parametrize("unroll", [1, 2, 4, 8])
-@pytest.mark.parametrize("max_blocks", [0, 5])
-def test_copy_parity_under_every_launch_shape(dev, unroll, max_blocks):
+@pytest.mark.parametrize("max_blocks,wg_per_cu", [(0, 0), (5, 0), (0, 2), (0, 4), (0, 8), (0, 9)])
+def test_copy_parity_under_every_launch_shape(dev, unroll, max_blocks, wg_per_cu):
     old = abi.get_tuning("copy_unroll"), abi.get_tuning("copy_max_blocks"), abi.get_tuning("box_unroll")
     try:
         abi.set_tuning("copy_unroll", unroll)
         abi.set_tuning("box_unroll", unroll)
         abi.set_tuning("copy_max_blocks", max_blocks)
+        abi.set_tuning("copy_wg_per_cu", wg_per_cu)
         G = torch.randn(96, 200)
         Gd = G.to(dev)
         out = torch.zeros(96, 40, device=dev)
@@ -128,6 +129,7 @@ def test_copy_parity_under_every_launch_shape(dev, unroll, max_blocks):
         abi.set_tuning("copy_unroll", old[0])
         abi.set_tuning("copy_max_blocks", old[1])
         abi.set_tuning("box_unroll", old[2])
+        abi.set_tuning("copy_wg_per_cu", 0)
 
 
 def _strides(t):

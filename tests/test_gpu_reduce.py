@@ -67,6 +67,38 @@ def test_parity_under_every_launch_shape(dev, unroll, max_blocks):
         abi.set_tuning("reduce_max_blocks", old[1])
 
 
+@pytest.mark.parametrize("wg_per_cu", [1, 2, 3, 5, 8, 9])
+def test_parity_under_every_residency_cap(dev, wg_per_cu):
+    # the cap is an unused LDS allocation; 1 needs the kernel's dynamic-LDS limit raised
+    old = abi.get_tuning("reduce_wg_per_cu")
+    try:
+        abi.set_tuning("reduce_wg_per_cu", wg_per_cu)
+        for dtype, op in ((torch.float32, oracle.OP_SUM), (torch.bfloat16, oracle.OP_AVG), (torch.float16, oracle.OP_PREMUL_SUM),
+                          (torch.int32, oracle.OP_MAX)):
+            P, n = 8, 700000 + 5
+            srcs = random_sources(P, n, dtype, seed=wg_per_cu)
+            scale = scale_for(op, P)
+            want = oracle.reduce([bits(s) for s in srcs], 2, TORCH_TO_CODE[dtype], op, scale)
+            out = torch.zeros(n, dtype=dtype, device=dev)
+            gpu_reduce([s.to(dev) for s in srcs], 2, out, op, scale)
+            assert same_bits(bits(out), want), (dtype, op)
+    finally:
+        abi.set_tuning("reduce_wg_per_cu", old)
+
+
+def test_large_sources_take_the_capped_shape_and_match(dev):
+    # 64 MiB per source and 8..16 sources select one or two sub-tiles with two workgroups per CU
+    for dtype, P in ((torch.float32, 8), (torch.bfloat16, 9), (torch.float16, 12)):
+        n = (64 << 20) // torch.empty(0, dtype=dtype).element_size() + 3
+        g = torch.Generator().manual_seed(P)
+        srcs = [(torch.randn(n, generator=g) * 3).to(dtype) for _ in range(P)]
+        want = oracle.reduce([bits(s) for s in srcs], 5, TORCH_TO_CODE[dtype], oracle.OP_SUM)
+        out = torch.zeros(n, dtype=dtype, device=dev)
+        gpu_reduce([s.to(dev) for s in srcs], 5, out, oracle.OP_SUM)
+        assert same_bits(bits(out), want), (dtype, P)
+        del srcs, want, out
+
+
 def test_golden_fixtures(dev):
     z = np.load(os.path.join(HERE, "golden", "reduce_cases.npz"))
     code_to_torch = {v: k for k, v in TORCH_TO_CODE.items()}
