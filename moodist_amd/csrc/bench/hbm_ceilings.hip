@@ -148,6 +148,9 @@ int main(int argc, char** argv) {
   const size_t half = whole / 2;
   run("copy 4x -> 4x in one kernel, nt loads, sc1 stores", (double)whole,
       [&](int s) { hipLaunchKernelGGL((fold_kernel<1, 4, kNt, kSc1, true>), dim3(half / t4), dim3(256), 0, 0, set(s), 0, set(s) + half, half / t4); });
+  // an unused dynamic LDS allocation caps the workgroups resident on a CU: 40 KiB -> four, 64 KiB -> two
+  run("copy 4x -> 4x, nt/sc1, two sub-tiles, four workgroups per CU", (double)whole,
+      [&](int s) { hipLaunchKernelGGL((fold_kernel<1, 2, kNt, kSc1, true>), dim3(half / (t4 / 2)), dim3(256), 40960, 0, set(s), 0, set(s) + half, half / (t4 / 2)); });
   run("copy 4x -> 4x in one kernel, plain loads and stores", (double)whole,
       [&](int s) { hipLaunchKernelGGL((fold_kernel<1, 4, 0, 0, true>), dim3(half / t4), dim3(256), 0, 0, set(s), 0, set(s) + half, half / t4); });
   run("read kernel (4x) then write kernel (4x), same stream", (double)whole, [&](int s) {
@@ -169,7 +172,9 @@ int main(int argc, char** argv) {
       [&](int s) { hipLaunchKernelGGL((fold_kernel<8, 2, kNt, kSc1, true>), dim3(stream / (t4 / 2)), dim3(256), 0, 0, set(s), stream, set(s) + stream * 8, stream / (t4 / 2)); });
   run("8 streams -> 1, nt loads, sc1 stores, one sub-tile", nine,
       [&](int s) { hipLaunchKernelGGL((fold_kernel<8, 1, kNt, kSc1, true>), dim3(stream / t1), dim3(256), 0, 0, set(s), stream, set(s) + stream * 8, stream / t1); });
-  run("8 streams -> 1, nt/sc1, four sub-tiles, one workgroup per CU", nine,
+  run("8 streams -> 1, nt/sc1, one sub-tile, two workgroups per CU", nine,
+      [&](int s) { hipLaunchKernelGGL((fold_kernel<8, 1, kNt, kSc1, true>), dim3(stream / t1), dim3(256), 65536, 0, set(s), stream, set(s) + stream * 8, stream / t1); });
+  run("8 streams -> 1, nt/sc1, four sub-tiles, persistent grid of 256", nine,
       [&](int s) { hipLaunchKernelGGL((fold_kernel<8, 4, kNt, kSc1, true>), dim3(256), dim3(256), 0, 0, set(s), stream, set(s) + stream * 8, stream / t4); });
   return 0;
 }
