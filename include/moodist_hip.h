@@ -16,7 +16,9 @@
  *     for the calling thread;
  *   - allocates nothing, frees nothing, never synchronises: work is enqueued
  *     on `stream` (a hipStream_t; NULL is the default stream) and the caller
- *     owns every buffer until that work has finished;
+ *     owns every buffer until that work has finished.  Long launches ask for
+ *     40-64 KiB of dynamic LDS per workgroup that the kernels never touch: it
+ *     limits how many workgroups a CU holds at once;
  *   - all data pointers are device pointers on the current device; pointer
  *     TABLES (srcs, boxes) are host memory and are consumed before return;
  *   - dtype codes are torch ScalarType numbers and op codes are c10d RedOpType
