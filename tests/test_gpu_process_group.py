@@ -309,6 +309,30 @@ def test_stress_rapid_collectives(world, dev):
             assert torch.equal(rs_out[r][i], torch.full((chunk,), 36.0, device=dev))
 
 
+def test_stress_mixed_collectives(world, dev):
+    # :146-232 without the broadcast (outside this path): all_gather, reduce_scatter, allreduce and
+    # barrier interleaved in a tight loop
+    iters, chunk = 50, 32
+    ag_in = [[torch.full((chunk,), float(r), device=dev) for _ in range(iters)] for r in range(P)]
+    ag_out = [[torch.zeros(chunk * P, device=dev) for _ in range(iters)] for _ in range(P)]
+    rs_in = [[torch.full((chunk * P,), float(r + 1), device=dev) for _ in range(iters)] for r in range(P)]
+    rs_out = [[torch.zeros(chunk, device=dev) for _ in range(iters)] for _ in range(P)]
+    ar = [[torch.full((chunk,), float(r + 1), device=dev) for _ in range(iters)] for r in range(P)]
+    for i in range(iters):
+        each_rank(world, lambda r, pg: pg._allgather_base(ag_out[r][i], ag_in[r][i]))
+        each_rank(world, lambda r, pg: pg._reduce_scatter_base(rs_out[r][i], rs_in[r][i]))
+        each_rank(world, lambda r, pg: pg.allreduce([ar[r][i]]))
+        each_rank(world, lambda r, pg: pg.barrier())
+    want = torch.arange(P, device=dev).float().repeat_interleave(chunk)
+    for r in range(P):
+        for i in range(iters):
+            assert torch.equal(ag_out[r][i], want)
+            assert torch.equal(rs_out[r][i], torch.full((chunk,), 36.0, device=dev))
+            assert torch.equal(ar[r][i], torch.full((chunk,), 36.0, device=dev))
+    with pytest.raises(RuntimeError, match="broadcast .* is not supported"):
+        world.groups[0].broadcast([ar[0][0]])
+
+
 def test_stress_varying_sizes(world, dev):
     # :235-280
     for size in (1, 7, 64, 255, 1024, 4096, 65536):
