@@ -609,6 +609,20 @@ struct Launcher {
       }
       return;
     }
+    if ((h.run & 15) && h.run >= 32) {
+      // Rows that are not a multiple of 16 bytes long would move as 1-, 2-, 4- or 8-byte vectors
+      // (0.6-1.7 TB/s on 4 KiB rows).  Their first run & ~15 bytes go as 16-byte vectors, which
+      // the buffer path takes at any alignment, and the last < 16 bytes of every row as a box
+      // of its own.
+      HostBox body = h, tail = h;
+      body.run = h.run & ~(int64_t)15;
+      tail.src = h.src + body.run;
+      tail.dst = h.dst + body.run;
+      tail.run = h.run & 15;
+      emit(body);
+      emit(tail);
+      return;
+    }
     emit(h);
   }
 };

@@ -136,6 +136,28 @@ def _strides(t):
     return list(t.stride())
 
 
+@pytest.mark.parametrize("itemsize", [1, 2, 4])
+def test_strided_rows_of_ragged_byte_length(dev, itemsize):
+    # rows whose byte length is not a multiple of 16 move as a 16-byte body plus a narrow tail;
+    # every byte of the destination outside the boxes must stay untouched
+    dtype = {1: torch.uint8, 2: torch.int16, 4: torch.int32}[itemsize]
+    g = torch.Generator().manual_seed(itemsize)
+    for rows, cols, src_pitch, dst_pitch, col0 in ((37, 1025, 1031, 1100, 3), (5, 33, 40, 35, 1), (64, 259, 259, 300, 0),
+                                                    (3, 8, 9, 9, 0), (129, 4097, 4099, 4200, 2)):
+        if itemsize == 4:
+            cols, src_pitch, dst_pitch = cols // 4 + 1, src_pitch // 4 + 3, dst_pitch // 4 + 3
+        src = torch.randint(0, 100, (rows, src_pitch), generator=g).to(dtype)
+        sd = src.to(dev)
+        out = torch.full((rows, dst_pitch), 7, dtype=dtype, device=dev)
+        boxes = [abi.make_box(sd.data_ptr() + col0 * itemsize, out.data_ptr() + itemsize, [rows, cols],
+                              [src_pitch, 1], [dst_pitch, 1])]
+        abi.copy_boxes(boxes, itemsize, st())
+        sync()
+        want = torch.full((rows, dst_pitch), 7, dtype=dtype)
+        want[:, 1:1 + cols] = src[:, col0:col0 + cols]
+        assert torch.equal(out.cpu(), want), (itemsize, rows, cols)
+
+
 def test_boxes_against_torch_slicing(dev):
     g = torch.Generator().manual_seed(5)
     for dtype in (torch.uint8, torch.bfloat16, torch.float32, torch.float64):
