@@ -1,0 +1,131 @@
+"""Seeded randomized differential tests on the GPU, through the C ABI.
+
+The reduction is compared bit for bit with the CPU oracle over random element types, ops, source
+counts, sizes, fold starts, element misalignments of every buffer, in-place destinations, special
+values (NaN, infinities, -0) and launch-shape knobs; guard elements round the destination must
+stay untouched.  The box copy is compared with torch slicing on the CPU over random N-d boxes
+(1..6 dims, four element sizes, ragged inner runs, padded destinations, several boxes per call in
+random order) and knobs.
+"""
+
+import random
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from moodist_amd import _abi as abi
+from util import ALL_DTYPES, TORCH_TO_CODE, bits, same_bits
+
+pytestmark = pytest.mark.gpu
+OPS = [oracle.OP_SUM, oracle.OP_MIN, oracle.OP_MAX, oracle.OP_AVG, oracle.OP_PREMUL_SUM]
+KNOBS = ("reduce_unroll", "reduce_max_blocks", "reduce_wg_per_cu", "box_unroll", "copy_unroll", "copy_max_blocks",
+         "copy_wg_per_cu")
+
+
+@pytest.fixture()
+def knobs():
+    yield
+    for k in KNOBS:
+        abi.set_tuning(k, 0)
+
+
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_reduce_random_cases_match_the_oracle(dev, knobs, seed):
+    st = torch.cuda.current_stream().cuda_stream
+    rng = random.Random(seed)
+    for case in range(120):
+        dtype = rng.choice(ALL_DTYPES)
+        op = rng.choice(OPS)
+        if op in (oracle.OP_AVG, oracle.OP_PREMUL_SUM) and not dtype.is_floating_point:
+            op = oracle.OP_SUM
+        P = rng.choice([1, 2, 3, 4, 5, 7, 8, 9, 12, 15, 16, 17, 24, 31, 32, 33, 63, 64])
+        n = rng.choice([1, 2, 3, 5, 8, 15, 16, 17, 100, 1023, 1024, 4099, 65536, 70001, rng.randint(1, 300000),
+                        rng.randint(1, 2000000) // max(1, P // 8)])
+        first = rng.randrange(P)
+        offs = [rng.randrange(0, 9) for _ in range(P + 1)]  # element misalignment of every buffer
+        abi.set_tuning("reduce_unroll", rng.choice([0, 0, 1, 2, 4, 8]))
+        abi.set_tuning("reduce_max_blocks", rng.choice([0, 0, 1, 7, 300]))
+        abi.set_tuning("reduce_wg_per_cu", rng.choice([0, 0, 1, 2, 3, 6, 9]))
+        g = torch.Generator().manual_seed(seed * 100000 + case)
+        srcs = []
+        for _ in range(P):
+            if dtype.is_floating_point:
+                t = (torch.randn(n, generator=g) * 4).to(dtype)
+                if rng.random() < 0.1 and n > 3:
+                    t[rng.randrange(n)] = float("nan")
+                    t[rng.randrange(n)] = float("inf")
+                    t[rng.randrange(n)] = -0.0
+            else:
+                t = torch.randint(-2**30, 2**30, (n,), generator=g).to(dtype) * 3
+            srcs.append(t)
+        scale = float(np.float32(1.0) / np.float32(P)) if op == oracle.OP_AVG else \
+            float(np.float32(rng.choice([0.37, 2.0, -1.5, 1e-3])))
+        want = oracle.reduce([bits(s) for s in srcs], first, TORCH_TO_CODE[dtype], op, scale)
+        dbuf = []
+        for j in range(P):
+            b = torch.zeros(n + 16, dtype=dtype, device=dev)
+            b[offs[j]:offs[j] + n] = srcs[j].to(dev)
+            dbuf.append(b)
+        inplace = rng.random() < 0.2
+        if inplace:
+            out_full, o = dbuf[first], offs[first]
+        else:
+            out_full, o = torch.full((n + 16,), 5, dtype=dtype, device=dev), offs[P]
+        isz = out_full.element_size()
+        abi.reduce([dbuf[j].data_ptr() + offs[j] * isz for j in range(P)], first, out_full.data_ptr() + o * isz, n,
+                   TORCH_TO_CODE[dtype], op, scale, st)
+        torch.cuda.synchronize()
+        what = (seed, case, dtype, op, P, n, first, offs, inplace)
+        assert same_bits(bits(out_full[o:o + n]), want), what
+        if not inplace:
+            assert bool((torch.cat([out_full[:o], out_full[o + n:]]).cpu() == 5).all()), what
+
+
+@pytest.mark.parametrize("seed", [1, 2])
+def test_copy_random_boxes_match_torch_slicing(dev, knobs, seed):
+    st = torch.cuda.current_stream().cuda_stream
+    rng = random.Random(seed)
+    dtypes = {1: torch.uint8, 2: torch.int16, 4: torch.int32, 8: torch.int64}
+    for case in range(250):
+        itemsize = rng.choice([1, 2, 4, 8])
+        dtype = dtypes[itemsize]
+        ndim = rng.randint(1, 6)
+        big = rng.random() < 0.3
+        full = [rng.randint(1, 6 if ndim > 3 else (40 if not big else 300)) for _ in range(ndim)]
+        full[-1] = rng.choice([1, 2, 3, 7, 8, 16, 17, 33, 64, 100, 257, 1024, 1030]) if ndim < 4 else rng.randint(1, 40)
+        while np.prod(full) > 3_000_000:
+            k = rng.randrange(ndim)
+            full[k] = max(1, full[k] // 2)
+        g = torch.Generator().manual_seed(seed * 100000 + case)
+        src = torch.randint(0, 120, tuple(full), generator=g).to(dtype)
+        dstfull = [f + rng.choice([0, 0, 1, 3]) for f in full]
+        sd = src.to(dev)
+        out = torch.full(tuple(dstfull), 7, dtype=dtype, device=dev)
+        want = torch.full(tuple(dstfull), 7, dtype=dtype)
+        # dimension d is cut into slabs, so the boxes cannot overlap in the destination
+        d = rng.randrange(ndim)
+        cuts = sorted(set([0, full[d]] + [rng.randint(0, full[d]) for _ in range(rng.randint(0, 4))]))
+        boxes = []
+        for a, b in zip(cuts[:-1], cuts[1:]):
+            lo = [rng.randint(0, f - 1) for f in full]
+            hi = [rng.randint(l + 1, f) for l, f in zip(lo, full)]
+            lo[d], hi[d] = a, b
+            shape = [h - l for l, h in zip(lo, hi)]
+            dlo = [rng.randint(0, df - s) for df, s in zip(dstfull, shape)]
+            dlo[d] = a
+            sidx = tuple(slice(l, h) for l, h in zip(lo, hi))
+            didx = tuple(slice(l, l + s) for l, s in zip(dlo, shape))
+            want[didx] = src[sidx]
+            sview, dview = sd[sidx], out[didx]
+            boxes.append(abi.make_box(sview.data_ptr(), dview.data_ptr(), shape, list(sview.stride()),
+                                      list(dview.stride())))
+        abi.set_tuning("box_unroll", rng.choice([0, 0, 1, 2, 4, 8]))
+        abi.set_tuning("copy_unroll", rng.choice([0, 0, 1, 2, 4, 8]))
+        abi.set_tuning("copy_max_blocks", rng.choice([0, 0, 1, 9]))
+        abi.set_tuning("copy_wg_per_cu", rng.choice([0, 0, 2, 4, 9]))
+        rng.shuffle(boxes)
+        abi.copy_boxes(boxes, itemsize, st)
+        torch.cuda.synchronize()
+        assert torch.equal(out.cpu(), want), (seed, case, itemsize, full, dstfull, d, cuts)
