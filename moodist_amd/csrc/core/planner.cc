@@ -47,6 +47,15 @@ bool overlaps(const Dims& ao, const Dims& as, const Dims& bo, const Dims& bs) {
   return true;
 }
 
+bool inside(const Dims& ao, const Dims& as, const Dims& bo, const Dims& bs) {
+  for (size_t i = 0; i < ao.size(); ++i) {
+    if (ao[i] < bo[i] || ao[i] + as[i] > bo[i] + bs[i]) {
+      return false;
+    }
+  }
+  return true;
+}
+
 // a slab that spans every dimension but the first is one contiguous range (:2863-2870)
 bool whole_rows(const Dims& part, const Dims& whole) {
   for (size_t i = 1; i < part.size(); ++i) {
@@ -271,6 +280,17 @@ std::vector<RankPlan> plan_redistribution(int size, const Dims& shape, size_t it
               rows = rows && whole_rows(y.shape, staged[y.index].shape);
               if (!rows) {
                 break;
+              }
+            }
+            // The reference accepts the staged pieces when their element counts add up to the
+            // piece wanted (:2945-2946).  Staging can hold the same elements twice, and pieces of
+            // another tensor of this rank, so equal counts do not mean the piece is covered: the
+            // reference then reads one element twice and leaves another unwritten.  Here the
+            // pieces must also lie inside the piece wanted and not overlap each other.
+            for (size_t p = 0; rows && p < again.size(); ++p) {
+              rows = inside(again[p].offset, again[p].shape, x.offset, x.shape);
+              for (size_t q = 0; rows && q < p; ++q) {
+                rows = !overlaps(again[p].offset, again[p].shape, again[q].offset, again[q].shape);
               }
             }
             if (rows && n == dims_numel(x.shape)) {

@@ -120,19 +120,28 @@ def _descrs(args, size):
     return out, counter
 
 
-def plan(size, shape, itemsize, inputs_arg, outputs_arg):
+def plan(size, shape, itemsize, inputs_arg, outputs_arg, strict_reuse=True):
     """inputs_arg/outputs_arg: lists of (rank, offset, shape) in global coordinates.
 
     Returns one Descriptor per rank.  Reads arrive sender by sender in rank
     order (the reference's arrival order is unspecified).
+
+    strict_reuse=False is the reference to the letter: staged pieces found inside a
+    destination are reused when their element counts add up to the piece wanted
+    (core/processgroup.cc:2931-2962).  Staging can hold an element twice (and pieces of the
+    rank's other tensors), so the counts can match while one element is read twice and another
+    never: the plan then passes the coverage check (:3079-3081) and executes to a wrong
+    result (tests/test_oracle_copy.py holds such a case).  strict_reuse=True, the default and
+    what the product does, also requires the pieces to lie inside the piece wanted and to be
+    pairwise disjoint; plans are the same wherever the reference's are right.
     """
-    return _plan(size, shape, itemsize, inputs_arg, outputs_arg)[0]
+    return _plan(size, shape, itemsize, inputs_arg, outputs_arg, strict_reuse)[0]
 
 
 def wire(size, shape, itemsize, inputs_arg, outputs_arg):
     """wire[sender][receiver]: the bytes `sender` puts on `receiver`'s queue while compiling
     (core/processgroup.cc:3015-3033)."""
-    sent = _plan(size, shape, itemsize, inputs_arg, outputs_arg)[1]
+    sent = _plan(size, shape, itemsize, inputs_arg, outputs_arg, True)[1]
     return [[pack_messages(sent[s][r], len(shape)) for r in range(size)] for s in range(size)]
 
 
@@ -172,7 +181,12 @@ def unpack_messages(data, ndim):
     return out
 
 
-def _plan(size, shape, itemsize, inputs_arg, outputs_arg):
+def _inside(a, b):
+    return all(ao >= bo and ao + ash <= bo + bsh
+               for ao, ash, bo, bsh in zip(a["offset"], a["shape"], b["offset"], b["shape"]))
+
+
+def _plan(size, shape, itemsize, inputs_arg, outputs_arg, strict_reuse=True):
     ndim = len(shape)
     for _, off, shp in list(inputs_arg) + list(outputs_arg):
         assert len(off) == ndim and len(shp) == ndim
@@ -211,6 +225,12 @@ def _plan(size, shape, itemsize, inputs_arg, outputs_arg):
                             cc = cc and _contiguous(x2["shape"], copyInputs[x2["index"]]["shape"])
                             if not cc:
                                 break
+                        if strict_reuse:
+                            # deviation from the reference, see plan(): the pieces must lie inside
+                            # the piece wanted and be pairwise disjoint
+                            for p, y in enumerate(rr):
+                                cc = cc and _inside(y, x) and not any(
+                                    _intersecting(y["offset"], y["shape"], z["offset"], z["shape"]) for z in rr[:p])
                         if cc and n == _numel(x["shape"]):
                             for x2 in rr:
                                 ci = copyInputs[x2["index"]]

@@ -234,6 +234,26 @@ def test_cpp_planner_random_boxes_match_oracle():
             assert got["messages"] == wire[r], (trial, r)
 
 
+def test_cpp_planner_random_multi_slice_cases_match_oracle():
+    # several slices per rank, grids, overlapping outputs: the cases in which staging is reused
+    from test_oracle_copy import _random_redistribution
+
+    for seed in range(150):
+        rng = np.random.RandomState(seed)
+        size = int(rng.randint(1, 6))
+        shape, inputs, outputs = _random_redistribution(rng, size)
+        want = planner.plan(size, shape, 4, inputs, outputs)
+        wire = planner.wire(size, shape, 4, inputs, outputs)
+        world = moodist_amd.LocalWorld(size, 0)
+        for r, pg in enumerate(world):
+            got = pg.compile_op_full(shape, torch.int32, inputs, outputs).plan()
+            assert got["reads"] == [(x.rank, x.inputIndex, x.outputIndex, x.inputOffset, x.outputOffset, x.bytes)
+                                    for x in want[r].reads], (seed, r)
+            assert got["inputCopies"] == [(c.index, c.offset, c.shape) for c in want[r].inputCopies], (seed, r)
+            assert got["outputCopies"] == [(c.index, c.offset, c.shape) for c in want[r].outputCopies], (seed, r)
+            assert got["messages"] == wire[r], (seed, r)
+
+
 def test_plan_messages_hand_derived_bytes_and_deserializer_errors(core):
     from test_oracle_copy import WIRE_4X4_COL_TO_ROW_R0_TO_R1, WIRE_4X4_R0_TO_R1, WIRE_4X4_R1_TO_R0
 

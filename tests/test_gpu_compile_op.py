@@ -166,6 +166,45 @@ def test_overlapping_outputs_and_bystanders(world, dev):
         assert torch.equal(outs[r].cpu(), G[off[0]:off[0] + shp[0], off[1]:off[1] + shp[1]])
 
 
+@pytest.mark.parametrize("seed", [0, 1])
+def test_random_redistributions_match_numpy_slicing(world, dev, seed):
+    # inputs: one random dimension cut into slabs dealt to random ranks (some ranks hold several
+    # slabs, some none); outputs: a random box per rank, possibly overlapping each other.  Every
+    # output must equal the same slice of the global tensor.
+    rng = np.random.RandomState(seed)
+    for trial in range(25):
+        ndim = int(rng.randint(1, 5))
+        shape = [int(rng.randint(2, 20)) for _ in range(ndim)]
+        shape[-1] = int(rng.choice([3, 8, 16, 33, 64]))
+        dtype = [torch.float32, torch.bfloat16, torch.int64, torch.float64][trial % 4]
+        G = torch.from_numpy(rng.randint(-50, 50, shape)).to(dtype)
+        d = int(rng.randint(0, ndim))
+        cuts = sorted(set([0, shape[d]] + [int(x) for x in rng.randint(0, shape[d] + 1, 6)]))
+        ins = {r: [] for r in range(P)}
+        for a, b in zip(cuts[:-1], cuts[1:]):
+            off, shp = [0] * ndim, list(shape)
+            off[d], shp[d] = a, b - a
+            ins[int(rng.randint(0, P))].append((off, shp))
+        specs = {"shape": shape, "dtype": dtype}
+        tensors, outs, want = {}, {}, {}
+        for r in range(P):
+            ins[r].sort(key=lambda x: -int(np.prod(x[1])))  # a rank lists its slices largest first
+            lo = [int(rng.randint(0, n)) for n in shape]
+            hi = [int(rng.randint(l + 1, n + 1)) for l, n in zip(lo, shape)]
+            has_out = rng.rand() < 0.8
+            idx = tuple(slice(l, h) for l, h in zip(lo, hi))
+            outs[r] = torch.zeros([h - l for l, h in zip(lo, hi)], dtype=dtype, device=dev) if has_out else None
+            want[r] = G[idx] if has_out else None
+            specs[r] = ([{"offset": o, "shape": s} for o, s in ins[r]] or None,
+                        [{"offset": lo, "shape": [h - l for l, h in zip(lo, hi)]}] if has_out else None)
+            tensors[r] = ([G[tuple(slice(o_, o_ + s_) for o_, s_ in zip(o, s))].contiguous().to(dev) for o, s in ins[r]],
+                          [outs[r]] if has_out else [])
+        run(world, specs, tensors)
+        for r in range(P):
+            if outs[r] is not None:
+                assert torch.equal(outs[r].cpu(), want[r]), (seed, trial, r, shape, d, cuts)
+
+
 def test_future_before_every_rank_called(world, dev):
     ops = [compile_op(pg, shape=[4], dtype=torch.float32, inputs=[{"offset": [0], "shape": [4]}] if r == 0 else None,
                       outputs=[{"offset": [0], "shape": [4]}]) for r, pg in enumerate(world)]

@@ -185,6 +185,83 @@ def test_plan_wire_round_trip_and_record_length():
             planner.unpack_messages(data + b"\0", ndim)
 
 
+def _random_redistribution(rng, size):
+    """Non-overlapping inputs (slabs along one dimension or a grid over two) dealt to random ranks,
+    up to two random output boxes per rank; every rank lists its slices largest first."""
+    ndim = int(rng.randint(1, 5))
+    shape = [int(rng.randint(1, 12)) for _ in range(ndim)]
+    d1, d2 = int(rng.randint(0, ndim)), int(rng.randint(0, ndim))
+    c1 = sorted(set([0, shape[d1]] + [int(x) for x in rng.randint(0, shape[d1] + 1, 4)]))
+    c2 = sorted(set([0, shape[d2]] + [int(x) for x in rng.randint(0, shape[d2] + 1, 3)])) \
+        if d2 != d1 and rng.rand() < 0.5 else [0, shape[d2]]
+    inputs = []
+    for a, b in zip(c1[:-1], c1[1:]):
+        for c, e in zip(c2[:-1], c2[1:]):
+            off, shp = [0] * ndim, list(shape)
+            off[d1], shp[d1] = a, b - a
+            if len(c2) > 2:
+                off[d2], shp[d2] = c, e - c
+            inputs.append((int(rng.randint(0, size)), off, shp))
+    outputs = []
+    for r in range(size):
+        for _ in range(int(rng.randint(0, 3))):
+            lo = [int(rng.randint(0, n)) for n in shape]
+            hi = [int(rng.randint(l + 1, n + 1)) for l, n in zip(lo, shape)]
+            outputs.append((r, lo, [h - l for l, h in zip(lo, hi)]))
+    inputs.sort(key=lambda x: (x[0], -int(np.prod(x[2]))))
+    outputs.sort(key=lambda x: (x[0], -int(np.prod(x[2]))))
+    return shape, inputs, outputs
+
+
+def _executes_correctly(size, shape, inputs, outputs, G, **kw):
+    descs = planner.plan(size, shape, 4, inputs, outputs, **kw)
+    ins = [[_u8(G[tuple(slice(o, o + s) for o, s in zip(off, shp))]).copy() for r, off, shp in inputs if r == q]
+           for q in range(size)]
+    outs = [[np.zeros(n, dtype=np.uint8) for n in d.outputs] for d in descs]
+    planner.execute(descs, 4, ins, outs)
+    counter = {}
+    for r, off, shp in outputs:
+        i = counter.get(r, 0)
+        counter[r] = i + 1
+        if not np.array_equal(outs[r][i].view(np.int32).reshape(shp), G[tuple(slice(o, o + s) for o, s in zip(off, shp))]):
+            return False
+    return True
+
+
+def test_planner_random_redistributions_execute_to_numpy_slicing():
+    # pins the planner restatement (with the sound staging-reuse rule) on 600 random cases
+    for seed in range(600):
+        rng = np.random.RandomState(seed)
+        size = int(rng.randint(1, 6))
+        shape, inputs, outputs = _random_redistribution(rng, size)
+        G = rng.randint(-50, 50, shape).astype(np.int32)
+        assert _executes_correctly(size, shape, inputs, outputs, G), (seed, shape, inputs, outputs)
+
+
+def test_reference_staging_reuse_rule_can_leave_an_element_unwritten():
+    # core/processgroup.cc:2931-2962 reuses staged pieces when their element counts add up to the
+    # piece wanted.  Rank 1 holds rows 11-12 and row 9 of a [15, 3] tensor; earlier destinations
+    # make it stage element [9, 2] twice; rank 5 then wants [9, 1:3], finds the two staged copies
+    # of [9, 2] (1 + 1 = 2 elements) and reads [9, 2] twice instead of [9, 1] and [9, 2].  The
+    # plan passes the reference's coverage check (:3079-3081).  The sound rule gets it right.
+    shape = [15, 3]
+    inputs = [(1, [11, 0], [2, 3]), (1, [9, 0], [1, 3]), (3, [10, 0], [1, 3]), (6, [5, 0], [4, 3]),
+              (7, [0, 0], [5, 3]), (7, [13, 0], [2, 3])]
+    outputs = [(0, [4, 2], [8, 1]), (1, [10, 2], [5, 1]), (2, [13, 2], [2, 1]), (3, [11, 0], [3, 1]),
+               (4, [3, 2], [11, 1]), (5, [9, 1], [1, 2]), (6, [12, 1], [3, 2]), (7, [11, 2], [2, 1])]
+    G = np.arange(45, dtype=np.int32).reshape(15, 3)
+    assert not _executes_correctly(8, shape, inputs, outputs, G, strict_reuse=False)
+    assert _executes_correctly(8, shape, inputs, outputs, G)
+    # where the reference's plan is right the two rules give the same plan
+    for seed in range(200):
+        rng = np.random.RandomState(seed)
+        size = int(rng.randint(1, 6))
+        shp, ins, outs = _random_redistribution(rng, size)
+        Gr = rng.randint(-50, 50, shp).astype(np.int32)
+        if _executes_correctly(size, shp, ins, outs, Gr, strict_reuse=False):
+            assert planner.plan(size, shp, 4, ins, outs, strict_reuse=False) == planner.plan(size, shp, 4, ins, outs)
+
+
 def test_planner_column_to_row_uses_output_copies():
     inputs = [(0, [0, 0], [4, 2]), (1, [0, 2], [4, 2])]
     outputs = [(0, [0, 0], [2, 4]), (1, [2, 0], [2, 4])]
