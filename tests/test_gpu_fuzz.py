@@ -14,6 +14,9 @@ import numpy as np
 import pytest
 import torch
 
+import torch.distributed as dist
+
+import moodist_amd
 import oracle
 from moodist_amd import _abi as abi
 from util import ALL_DTYPES, TORCH_TO_CODE, bits, same_bits
@@ -129,3 +132,77 @@ def test_copy_random_boxes_match_torch_slicing(dev, knobs, seed):
         abi.copy_boxes(boxes, itemsize, st)
         torch.cuda.synchronize()
         assert torch.equal(out.cpu(), want), (seed, case, itemsize, full, dstfull, d, cuts)
+
+
+def test_process_group_random_sequences_match_the_oracle(dev):
+    # random worlds (1..16 ranks) running random sequences of reduce_scatter, all_gather (flat and
+    # list form) and allreduce (sizes that do and do not divide by the world) on random dtypes
+    rng = random.Random(5)
+    dts = [torch.float32, torch.float64, torch.int32, torch.int64, torch.bfloat16, torch.float16]
+    ops = {"SUM": (dist.ReduceOp.SUM, oracle.OP_SUM), "MIN": (dist.ReduceOp.MIN, oracle.OP_MIN),
+           "MAX": (dist.ReduceOp.MAX, oracle.OP_MAX), "AVG": (dist.ReduceOp.AVG, oracle.OP_AVG)}
+    for case in range(60):
+        P = rng.choice([1, 2, 3, 4, 5, 8, 16])
+        world = moodist_amd.LocalWorld(P, dev)
+        for step in range(rng.randint(1, 5)):
+            kind = rng.choice(["rs", "ag", "ar", "agl"])
+            dtype = rng.choice(dts)
+            n = rng.choice([1, 3, 16, 100, 1000, 4097, rng.randint(1, 50000)])
+            g = torch.Generator().manual_seed(case * 100 + step)
+
+            def rnd(m):
+                if dtype.is_floating_point:
+                    return (torch.randn(m, generator=g) * 3).to(dtype)
+                return torch.randint(-1000, 1000, (m,), generator=g).to(dtype)
+
+            what = (case, step, kind, P, dtype, n)
+            if kind == "rs":
+                name = rng.choice(list(ops))
+                if name == "AVG" and not dtype.is_floating_point:
+                    name = "SUM"
+                ins = [rnd(n * P) for _ in range(P)]
+                d_in = [t.to(dev) for t in ins]
+                outs = [torch.zeros(n, dtype=dtype, device=dev) for _ in range(P)]
+                opts = dist.ReduceScatterOptions()
+                opts.reduceOp = ops[name][0]
+                for w in [pg._reduce_scatter_base(outs[r], d_in[r], opts) for r, pg in enumerate(world)]:
+                    w.wait()
+                torch.cuda.synchronize()
+                scale = float(np.float32(1.0) / np.float32(P))
+                for r in range(P):
+                    want = oracle.reduce([bits(t[r * n:(r + 1) * n]) for t in ins], r, TORCH_TO_CODE[dtype],
+                                         ops[name][1], scale)
+                    assert same_bits(bits(outs[r]), want), what + (name, r)
+            elif kind in ("ag", "agl"):
+                ins = [rnd(n) for _ in range(P)]
+                d_in = [t.to(dev) for t in ins]
+                if kind == "ag":
+                    outs = [torch.zeros(n * P, dtype=dtype, device=dev) for _ in range(P)]
+                    works = [pg._allgather_base(outs[r], d_in[r]) for r, pg in enumerate(world)]
+                else:
+                    lists = [[torch.zeros(n, dtype=dtype, device=dev) for _ in range(P)] for _ in range(P)]
+                    works = [pg.allgather([lists[r]], [d_in[r]]) for r, pg in enumerate(world)]
+                for w in works:
+                    w.wait()
+                torch.cuda.synchronize()
+                want = bits(torch.cat(ins))
+                for r in range(P):
+                    got = outs[r] if kind == "ag" else torch.cat(lists[r])
+                    assert same_bits(bits(got), want), what + (r,)
+            else:
+                name = rng.choice(["SUM", "MAX", "MIN"])
+                ins = [rnd(n) for _ in range(P)]
+                ts = [t.to(dev) for t in ins]
+                opts = dist.AllreduceOptions()
+                opts.reduceOp = ops[name][0]
+                for w in [pg.allreduce([ts[r]], opts) for r, pg in enumerate(world)]:
+                    w.wait()
+                torch.cuda.synchronize()
+                # chunk q of the (padded) tensor is folded starting at rank q (core/processgroup.cc:1674-1722)
+                padded = (n + P - 1) // P * P
+                c = padded // P
+                pin = [torch.cat([t, torch.zeros(padded - n, dtype=dtype)]) for t in ins]
+                want = np.concatenate([oracle.reduce([bits(t[q * c:(q + 1) * c]) for t in pin], q,
+                                                     TORCH_TO_CODE[dtype], ops[name][1], 1.0) for q in range(P)])[:n]
+                for r in range(P):
+                    assert same_bits(bits(ts[r]), want), what + (name, r)
