@@ -134,6 +134,44 @@ def test_copy_random_boxes_match_torch_slicing(dev, knobs, seed):
         assert torch.equal(out.cpu(), want), (seed, case, itemsize, full, dstfull, d, cuts)
 
 
+@pytest.mark.parametrize("seed", [1, 2])
+def test_gather_random_shapes_match_numpy(dev, knobs, seed):
+    # 1..70 shards, 1..300 rows, widths with and without a 16-byte body, independent row pitches,
+    # byte misalignment of every shard and of the output, guard bytes between and after shards
+    st = torch.cuda.current_stream().cuda_stream
+    rng = random.Random(seed)
+    for case in range(200):
+        P = rng.choice([1, 2, 3, 8, 9, 33, 70])
+        rows = rng.choice([1, 1, 2, 5, 64, 300])
+        width = rng.choice([1, 3, 15, 16, 17, 100, 1000, 4096, 4100, rng.randint(1, 20000)])
+        if rows * width * P > 10_000_000:
+            rows = max(1, 10_000_000 // (width * P))
+        sp = width + rng.choice([0, 0, 1, 16, 100])
+        dp = width + rng.choice([0, 0, 3, 16, 128])
+        if rows == 1:
+            sp = dp = width
+        stride = rows * dp + rng.choice([0, 0, 5, 256])
+        soff = [rng.randrange(0, 17) for _ in range(P)]
+        doff = rng.randrange(0, 17)
+        g = torch.Generator().manual_seed(seed * 100000 + case)
+        shards = [torch.randint(0, 255, (rows * sp + 32,), generator=g, dtype=torch.uint8) for _ in range(P)]
+        d = [s.to(dev) for s in shards]
+        out = torch.full((P * stride + 64,), 7, dtype=torch.uint8, device=dev)
+        for k in ("copy_unroll", "box_unroll"):
+            abi.set_tuning(k, rng.choice([0, 0, 1, 2, 4, 8]))
+        abi.set_tuning("copy_max_blocks", rng.choice([0, 0, 1, 11]))
+        abi.set_tuning("copy_wg_per_cu", rng.choice([0, 0, 2, 5, 9]))
+        abi.gather([d[s].data_ptr() + soff[s] for s in range(P)], out.data_ptr() + doff, width, rows, sp, dp, stride, st)
+        torch.cuda.synchronize()
+        want = np.full(P * stride + 64, 7, dtype=np.uint8)
+        for s in range(P):
+            src = shards[s].numpy()[soff[s]:soff[s] + rows * sp]
+            for r in range(rows):
+                lo = doff + s * stride + r * dp
+                want[lo:lo + width] = src[r * sp:r * sp + width]
+        assert np.array_equal(out.cpu().numpy(), want), (seed, case, P, rows, width, sp, dp, stride, soff, doff)
+
+
 def test_process_group_random_sequences_match_the_oracle(dev):
     # random worlds (1..16 ranks) running random sequences of reduce_scatter, all_gather (flat and
     # list form) and allreduce (sizes that do and do not divide by the world) on random dtypes
