@@ -509,8 +509,26 @@ struct Launcher {
     }
   }
 
+  // A box the kernels cannot index (more than kMaxOuter strided extents, or more than 2^31
+  // rows) is cut into pieces on the host.  The number of pieces of one call is bounded, so that
+  // an absurd box is refused instead of occupying the host for hours.
+  static constexpr size_t kMaxPieces = (size_t)1 << 20;
+  size_t pieces = 0;
+
+  bool count_piece() {
+    if (++pieces > kMaxPieces) {
+      set_error("copy: the boxes of this call break into more than %zu pieces; split the call", kMaxPieces);
+      rc = MDH_EINVAL;
+      return false;
+    }
+    return true;
+  }
+
   // rows x run with <= kMaxOuter strided extents
   void emit(const HostBox& h) {
+    if (!count_piece()) {
+      return;
+    }
     const int vec = vec_width(h);
     int lg = 0;
     while ((1 << lg) < vec) {
@@ -583,7 +601,9 @@ struct Launcher {
         return;
       }
       if ((h.run & 15) == 0) {
-        flat.push_back(Segment{h.src, h.dst, (uint64_t)h.run});
+        if (count_piece()) {
+          flat.push_back(Segment{h.src, h.dst, (uint64_t)h.run});
+        }
         return;
       }
       emit(h);
@@ -602,7 +622,7 @@ struct Launcher {
         p.sstride[d] = h.sstride[d + 1];
         p.dstride[d] = h.dstride[d + 1];
       }
-      for (int64_t i = 0; i < h.shape[0]; ++i) {
+      for (int64_t i = 0; i < h.shape[0] && rc == MDH_OK; ++i) {
         p.src = h.src + i * h.sstride[0];
         p.dst = h.dst + i * h.dstride[0];
         add(p);
@@ -708,6 +728,17 @@ extern "C" int mdh_copy_boxes(const mdh_box* boxes, int nboxes, int itemsize, vo
     }
     if (numel == 0) {
       continue;
+    }
+    // the bytes a side spans must be a plausible device size too (keeps every later offset
+    // computation inside 64 bits)
+    unsigned __int128 sspan = 0, dspan = 0;
+    for (int d = 0; d < b.ndim; ++d) {
+      sspan += (unsigned __int128)(b.shape[d] - 1) * (unsigned __int128)b.src_strides[d];
+      dspan += (unsigned __int128)(b.shape[d] - 1) * (unsigned __int128)b.dst_strides[d];
+    }
+    if (sspan > ((unsigned __int128)1 << 48) || dspan > ((unsigned __int128)1 << 48)) {
+      set_error("mdh_copy_boxes: box %d spans more than a plausible device size", i);
+      return MDH_EINVAL;
     }
     if (!b.src || !b.dst) {
       set_error("mdh_copy_boxes: box %d has a null pointer", i);

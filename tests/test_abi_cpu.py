@@ -58,6 +58,12 @@ def test_box_struct_layout_matches_header():
     (lambda: abi.copy_boxes([abi.make_box(0, 32, [4], [1], [1])], 4), "null pointer"),
     (lambda: abi.copy_boxes([abi.make_box(16, 32, [4], [-1], [1])], 4), "negative extent or stride"),
     (lambda: abi.copy_boxes([abi.make_box(18, 32, [4], [1], [1])], 4), "not aligned to its element size"),
+    (lambda: abi.copy_boxes([abi.make_box(16, 32, [4, 4], [2 ** 50, 1], [4, 1])], 4), "spans more than a plausible device size"),
+    # five strided extents that cannot merge, the slowest ones huge: the host would have to cut
+    # the box into 2^24 pieces
+    (lambda: abi.copy_boxes([abi.make_box(16, 1 << 40, [4096, 4096, 2, 2, 2, 1], [2 ** 22, 2 ** 10, 64, 16, 4, 1],
+                                          [2 ** 24, 2 ** 11, 128, 32, 8, 1])], 1), "more than 1048576 pieces"),
+    (lambda: abi.set_tuning("reduce_wg_per_cu", 10), "does not take 10"),
     (lambda: abi.set_tuning("no_such_knob", 1), "unknown knob"),
     (lambda: abi.set_tuning("reduce_unroll", 3), "does not take 3"),
 ])
