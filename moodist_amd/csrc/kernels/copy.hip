@@ -777,13 +777,15 @@ extern "C" int mdh_gather(const void* const* srcs, int nsrc, void* dst, size_t w
     set_error("mdh_gather: a row pitch is smaller than the row width");
     return MDH_EINVAL;
   }
+  const unsigned __int128 limit = (unsigned __int128)1 << 48;
+  if (width > limit || rows > ((size_t)1 << 40) || (unsigned __int128)rows * src_pitch > limit ||
+      (unsigned __int128)rows * dst_pitch > limit || (unsigned __int128)nsrc * dst_shard_stride > limit) {
+    set_error("mdh_gather: not a plausible device size");
+    return MDH_EINVAL;
+  }
   const size_t extent = (rows - 1) * dst_pitch + width;
   if (nsrc > 1 && dst_shard_stride < extent) {
     set_error("mdh_gather: shards would overlap in the destination");
-    return MDH_EINVAL;
-  }
-  if (width > ((size_t)1 << 48) || rows > ((size_t)1 << 40)) {
-    set_error("mdh_gather: not a plausible device size");
     return MDH_EINVAL;
   }
   Launcher L;

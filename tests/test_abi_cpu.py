@@ -54,6 +54,8 @@ def test_box_struct_layout_matches_header():
     (lambda: abi.gather([16], 1024, 8, 2, 4, 8, 64), "row pitch is smaller"),
     (lambda: abi.gather([16, 32], 1024, 8, 2, 8, 8, 8), "shards would overlap"),
     (lambda: abi.gather([0], 1024, 8, 1, 8, 8, 8), "source 0 is null"),
+    (lambda: abi.gather([16], 1024, 8, 2 ** 30, 2 ** 40, 8, 8), "not a plausible device size"),
+    (lambda: abi.gather([16, 32], 1024, 8, 1, 8, 8, 2 ** 60), "not a plausible device size"),
     (lambda: abi.copy_boxes([abi.make_box(16, 32, [4], [1], [1])], 3), "itemsize 3"),
     (lambda: abi.copy_boxes([abi.make_box(0, 32, [4], [1], [1])], 4), "null pointer"),
     (lambda: abi.copy_boxes([abi.make_box(16, 32, [4], [-1], [1])], 4), "negative extent or stride"),
