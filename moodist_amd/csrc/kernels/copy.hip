@@ -42,6 +42,7 @@ struct CopyArgs {
   uint32_t tile_end[kMaxBoxes]; // tiles of boxes 0..k, cumulative; unused entries are ~0
   uint32_t nboxes;
   uint32_t total_tiles;
+  uint32_t tiles_per_box; // non-zero when every box has the same tile count
 };
 static_assert(sizeof(CopyArgs) <= 4096, "kernel arguments are limited to 4 KiB");
 
@@ -146,13 +147,18 @@ __global__ __launch_bounds__(kBlock) void copy_boxes16_kernel(CopyArgs a) {
   constexpr uint32_t log2slots = ilog2(kBlock * U);
   for (uint32_t tile = blockIdx.x; tile < a.total_tiles; tile += gridDim.x) {
     uint32_t b = 0, start = 0;
+    if (a.tiles_per_box) {
+      b = tile / a.tiles_per_box; // equal boxes (the shards of a gather or of a redistribution)
+      start = b * a.tiles_per_box;
+    } else {
 #pragma unroll
-    for (int k = 0; k < kMaxBoxes - 1; ++k) {
-      const uint32_t e = a.tile_end[k];
-      // ends ascend, so the last one at or below the tile names the box; written as selects
-      // of scalars so that the whole scan stays on the scalar unit
-      b = tile >= e ? (uint32_t)(k + 1) : b;
-      start = tile >= e ? e : start;
+      for (int k = 0; k < kMaxBoxes - 1; ++k) {
+        const uint32_t e = a.tile_end[k];
+        // ends ascend, so the last one at or below the tile names the box; written as selects
+        // of scalars so that the whole scan stays on the scalar unit
+        b = tile >= e ? (uint32_t)(k + 1) : b;
+        start = tile >= e ? e : start;
+      }
     }
     const BoxDesc& B = a.box[b];
     const uint32_t local = tile - start;
@@ -448,6 +454,8 @@ struct Launcher {
       CopyArgs a{};
       a.nboxes = 0;
       uint64_t tiles = 0;
+      uint64_t first_n = 0;
+      bool equal = true;
       while (i < list.size() && a.nboxes < (uint32_t)kMaxBoxes) {
         BoxDesc d = list[i];
         uint32_t tc = 1, log2tc = 0;
@@ -466,11 +474,16 @@ struct Launcher {
           }
           break;
         }
+        if (a.nboxes == 0) {
+          first_n = n;
+        }
+        equal = equal && n == first_n;
         tiles += n;
         a.tile_end[a.nboxes] = (uint32_t)tiles;
         a.box[a.nboxes++] = d;
         ++i;
       }
+      a.tiles_per_box = equal ? (uint32_t)first_n : 0;
       for (uint32_t k = a.nboxes; k < (uint32_t)kMaxBoxes; ++k) {
         a.tile_end[k] = 0xffffffffu;
       }
