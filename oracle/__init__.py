@@ -59,7 +59,8 @@ def lib():
         L.orc_copy_box.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, i64p, i64p, i64p, ctypes.c_int]
         L.orc_copy_box.restype = ctypes.c_int
         L.orc_cpu_reduce_scatter_ranks.argtypes = [vpp, vpp, ctypes.c_int, ctypes.c_int, ctypes.c_size_t,
-                                                   ctypes.c_int, ctypes.c_int, ctypes.c_int]
+                                                   ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                                   ctypes.POINTER(ctypes.c_double)]
         L.orc_cpu_reduce_scatter_ranks.restype = ctypes.c_double
         L.orc_f32_to_bf16.argtypes = [ctypes.c_float]
         L.orc_f32_to_bf16.restype = ctypes.c_uint16
@@ -124,9 +125,11 @@ def copy_box(src, src_off, dst, dst_off, shape, src_strides, dst_strides, itemsi
 
 
 def cpu_reduce_scatter_seconds(inputs, outputs, nthreads, numel, dtype, op=OP_SUM, reps=3):
-    """Time the restated CPU reduce-scatter with `nthreads` rank-threads; see oracle.c."""
+    """Time the restated CPU reduce-scatter with `nthreads` rank-threads that live through all
+    `reps` repetitions; returns (median seconds, best seconds) per repetition; see oracle.c."""
+    best = ctypes.c_double()
     t = lib().orc_cpu_reduce_scatter_ranks(_ptr_table(inputs), _ptr_table(outputs), len(inputs), nthreads, numel,
-                                           dtype, op, reps)
+                                           dtype, op, reps, ctypes.byref(best))
     if t < 0:
         raise ValueError("orc_cpu_reduce_scatter_ranks rejected its arguments")
-    return t
+    return t, best.value

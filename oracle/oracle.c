@@ -336,18 +336,19 @@ int orc_copy_box(const void* src, void* dst, int ndim, const int64_t* shape, con
  * core/cputhread.cc:3589-3603) followed by the scalar fold loop (:3581-3585).
  *
  * inputs[p] is rank p's full input of nranks*numel elements; outputs[r] gets
- * numel elements.  Ranks 0..nthreads-1 run concurrently.  Returns wall seconds
- * for the slowest thread of the best of `reps` repetitions (<0 on error).
+ * numel elements.  Ranks 0..nthreads-1 run concurrently and stay alive, with their
+ * temporaries, over all `reps` repetitions (a barrier starts each one).  Returns the
+ * median over the repetitions of the wall seconds of the slowest thread (<0 on error).
  * ---------------------------------------------------------------------- */
 
 typedef struct {
   const void* const* inputs;
   void* output;
   void* tmp;
-  int rank, nranks, dtype, op;
+  int rank, nranks, dtype, op, reps;
   size_t numel;
   pthread_barrier_t* bar;
-  double seconds;
+  double* seconds; /* one per repetition */
 } rank_job;
 
 static double now_s(void) {
@@ -356,68 +357,91 @@ static double now_s(void) {
   return (double)ts.tv_sec + 1e-9 * (double)ts.tv_nsec;
 }
 
+/* One rank's service thread: it lives for all repetitions, as the reference's does for the life
+ * of the process (core/cputhread.cc:6415-6433), and keeps its temporary. */
 static void* rank_thread(void* p) {
   rank_job* j = (rank_job*)p;
   size_t isz = item_size(j->dtype);
   size_t bytes = j->numel * isz;
-  pthread_barrier_wait(j->bar);
-  double t0 = now_s();
-  memcpy(j->output, (const char*)j->inputs[j->rank] + bytes * (size_t)j->rank, bytes);
-  for (int k = 1; k < j->nranks; ++k) {
-    int peer = (j->rank + k) % j->nranks;
-    memcpy(j->tmp, (const char*)j->inputs[peer] + bytes * (size_t)j->rank, bytes);
-    if (j->dtype == DT_F32) {
-      fold_f32((float*)j->output, (const float*)j->tmp, j->numel, j->op);
-    } else if (j->dtype == DT_F64) {
-      fold_f64((double*)j->output, (const double*)j->tmp, j->numel, j->op);
-    } else if (j->dtype == DT_I32) {
-      fold_i32((int32_t*)j->output, (const int32_t*)j->tmp, j->numel, j->op);
-    } else {
-      fold_i64((int64_t*)j->output, (const int64_t*)j->tmp, j->numel, j->op);
+  for (int rep = 0; rep < j->reps; ++rep) {
+    pthread_barrier_wait(j->bar);
+    double t0 = now_s();
+    memcpy(j->output, (const char*)j->inputs[j->rank] + bytes * (size_t)j->rank, bytes);
+    for (int k = 1; k < j->nranks; ++k) {
+      int peer = (j->rank + k) % j->nranks;
+      memcpy(j->tmp, (const char*)j->inputs[peer] + bytes * (size_t)j->rank, bytes);
+      if (j->dtype == DT_F32) {
+        fold_f32((float*)j->output, (const float*)j->tmp, j->numel, j->op);
+      } else if (j->dtype == DT_F64) {
+        fold_f64((double*)j->output, (const double*)j->tmp, j->numel, j->op);
+      } else if (j->dtype == DT_I32) {
+        fold_i32((int32_t*)j->output, (const int32_t*)j->tmp, j->numel, j->op);
+      } else {
+        fold_i64((int64_t*)j->output, (const int64_t*)j->tmp, j->numel, j->op);
+      }
     }
+    j->seconds[rep] = now_s() - t0;
   }
-  j->seconds = now_s() - t0;
   return NULL;
 }
 
+static int cmp_double(const void* a, const void* b) {
+  double x = *(const double*)a, y = *(const double*)b;
+  return (x > y) - (x < y);
+}
+
+/* Returns the median over `reps` repetitions of the time of the slowest rank-thread; *best_out
+ * (may be NULL) receives the fastest repetition. */
 double orc_cpu_reduce_scatter_ranks(const void* const* inputs, void* const* outputs, int nranks, int nthreads,
-    size_t numel, int dtype, int op, int reps) {
+    size_t numel, int dtype, int op, int reps, double* best_out) {
   size_t isz = item_size(dtype);
   if (!(dtype == DT_F32 || dtype == DT_F64 || dtype == DT_I32 || dtype == DT_I64)) return -1.0;
   if (op != OP_SUM && op != OP_MIN && op != OP_MAX) return -1.0;
-  if (nthreads < 1 || nthreads > nranks || nthreads > 256 || reps < 1) return -1.0;
+  if (nthreads < 1 || nthreads > nranks || nthreads > 256 || reps < 1 || reps > 4096) return -1.0;
   pthread_t th[256];
   rank_job jobs[256];
   pthread_barrier_t bar;
-  double best = -1.0;
+  double* times = (double*)calloc((size_t)nthreads * (size_t)reps, sizeof(double));
+  if (!times) return -1.0;
   for (int t = 0; t < nthreads; ++t) {
     jobs[t].tmp = malloc(numel * isz + 1);
     if (!jobs[t].tmp) return -1.0;
+    /* the reference keeps its temporary across calls: take the page faults before the clock starts */
+    memset(jobs[t].tmp, 0, numel * isz + 1);
   }
+  pthread_barrier_init(&bar, NULL, (unsigned)nthreads);
+  for (int t = 0; t < nthreads; ++t) {
+    jobs[t].inputs = inputs;
+    jobs[t].output = outputs[t];
+    jobs[t].rank = t;
+    jobs[t].nranks = nranks;
+    jobs[t].dtype = dtype;
+    jobs[t].op = op;
+    jobs[t].reps = reps;
+    jobs[t].numel = numel;
+    jobs[t].bar = &bar;
+    jobs[t].seconds = times + (size_t)t * (size_t)reps;
+    pthread_create(&th[t], NULL, rank_thread, &jobs[t]);
+  }
+  for (int t = 0; t < nthreads; ++t) {
+    pthread_join(th[t], NULL);
+  }
+  pthread_barrier_destroy(&bar);
+  /* per repetition: the slowest thread */
   for (int rep = 0; rep < reps; ++rep) {
-    pthread_barrier_init(&bar, NULL, (unsigned)nthreads);
-    for (int t = 0; t < nthreads; ++t) {
-      jobs[t].inputs = inputs;
-      jobs[t].output = outputs[t];
-      jobs[t].rank = t;
-      jobs[t].nranks = nranks;
-      jobs[t].dtype = dtype;
-      jobs[t].op = op;
-      jobs[t].numel = numel;
-      jobs[t].bar = &bar;
-      jobs[t].seconds = 0.0;
-      pthread_create(&th[t], NULL, rank_thread, &jobs[t]);
-    }
     double worst = 0.0;
     for (int t = 0; t < nthreads; ++t) {
-      pthread_join(th[t], NULL);
-      if (jobs[t].seconds > worst) worst = jobs[t].seconds;
+      double s = times[(size_t)t * (size_t)reps + (size_t)rep];
+      if (s > worst) worst = s;
     }
-    pthread_barrier_destroy(&bar);
-    if (best < 0.0 || worst < best) best = worst;
+    times[rep] = worst; /* row 0 is overwritten only after its own entry was read */
   }
+  qsort(times, (size_t)reps, sizeof(double), cmp_double);
+  double median = times[reps / 2];
+  if (best_out) *best_out = times[0];
   for (int t = 0; t < nthreads; ++t) free(jobs[t].tmp);
-  return best;
+  free(times);
+  return median;
 }
 
 /* Exposed so the tests can pin the 16-bit conversions against torch's. */
