@@ -19,6 +19,8 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+CLOCK_WARMUP_S = 0.3   # untimed launches before the first timed window
+TIMED_WINDOWS = 11     # windows of `steps` launches; the median window is reported
 INFINITY_CACHE_BYTES = 256 << 20
 # (65568.73 KiB x 1.99971 fetched + 16384.00 KiB x 1.00000 written) per launch of the fp32 P=8 reduction
 MEASURED_TRAFFIC_BYTES = {"reduce_fp32_p8": 151031143}
@@ -120,7 +122,7 @@ def build_workload(name, torch, abi, dev):
 
         desc = {"workload": name, "op": "all_gather_into_tensor chunk assembly", "sources": P, "numel": n,
                 "dtype": "bfloat16", "buffer_sets": nsets}
-        return desc, set_bytes, launch, check, "copy_boxes_kernel"
+        return desc, set_bytes, launch, check, "copy_boxes16_kernel" if pad else "copy_flat_kernel"
 
     if name.startswith("redistribute"):
         # redistribute_fp32_8192, redistribute_bf16_8192, redistribute_bf16_3d
@@ -167,7 +169,7 @@ def build_workload(name, torch, abi, dev):
 
         desc = {"workload": name, "op": "compile_op redistribution copies", "sources": P,
                 "global_shape": list(shape), "dtype": str(tdt).replace("torch.", ""), "buffer_sets": nsets}
-        return desc, set_bytes, launch, check, "copy_boxes_kernel"
+        return desc, set_bytes, launch, check, "copy_boxes16_kernel"
 
     raise SystemExit("bench: unknown workload %r" % name)
 
@@ -204,7 +206,8 @@ def cpu_baseline(seconds_budget=12.0):
     return {
         "value": round(alg_bytes / median / 1e9, 2),
         "unit": "GB/s",
-        "cores": threads,
+        "cores": threads,  # threads used (one per emulated rank)
+        "host_cores": os.cpu_count(),
         "kind": "port",
         "sample": "full workload (8 ranks x 8 chunks of 4,194,304 fp32), %d rank-threads at once, median over %d "
                   "repetitions in batches of 20 (best %.2f GB/s); one rank-thread alone: %.2f GB/s"
@@ -238,18 +241,46 @@ def main():
     for i in range(args.warmup):
         launch(i)
     torch.cuda.synchronize()
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()  # on torch's current stream, the stream every launch above and below uses
-    for i in range(args.steps):
-        launch(i)
-    enqueue_ms = (time.perf_counter() - t0) * 1e3
-    e1.record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3
-    ms = e0.elapsed_time(e1)
+    # Clock warm-up: a fresh box takes a few hundred milliseconds of work to reach its steady
+    # clocks, far longer than `warmup` launches of 25 us; keep launching until CLOCK_WARMUP_S of
+    # wall time have passed.  These launches are not timed.
+    clock_launches = 0
+    t_warm = time.perf_counter()
+    while time.perf_counter() - t_warm < CLOCK_WARMUP_S:
+        for i in range(50):
+            launch(clock_launches + i)
+        clock_launches += 50
+        torch.cuda.synchronize()
+    # TIMED_WINDOWS windows of exactly `steps` launches each, every one bracketed by a
+    # synchronize on both sides and by two HIP events on the launch stream; the reported step
+    # time is the median window's (one window of 20 launches is 0.5 ms: a single one is noise).
+    window_ms, enqueue_ms, wall_ms = [], [], []
+    done = 0
+    for w in range(TIMED_WINDOWS):
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()  # on torch's current stream, the stream every launch above and below uses
+        for i in range(args.steps):
+            launch(done + i)
+        enqueue_ms.append((time.perf_counter() - t0) * 1e3)
+        e1.record()
+        torch.cuda.synchronize()
+        wall_ms.append((time.perf_counter() - t0) * 1e3)
+        window_ms.append(e0.elapsed_time(e1))
+        done += args.steps
+
+    def median(v):
+        v = sorted(v)
+        return v[len(v) // 2]
+
+    ms = median(window_ms)
+    enqueue_ms, wall_ms = median(enqueue_ms), median(wall_ms)
     ms_per_step = ms / args.steps
+    desc["timed_windows"] = TIMED_WINDOWS
+    desc["window_ms_min_median_max"] = [round(min(window_ms), 5), round(ms, 5), round(max(window_ms), 5)]
+    desc["clock_warmup_launches"] = clock_launches
     if not args.no_check:
         check()
     gbs = alg_bytes / (ms_per_step * 1e-3) / 1e9

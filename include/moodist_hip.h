@@ -16,8 +16,8 @@
  *     for the calling thread;
  *   - allocates nothing, frees nothing, never synchronises: work is enqueued
  *     on `stream` (a hipStream_t; NULL is the default stream) and the caller
- *     owns every buffer until that work has finished.  Long launches ask for
- *     40-64 KiB of dynamic LDS per workgroup that the kernels never touch: it
+ *     owns every buffer until that work has finished.  Long copies ask for
+ *     40 KiB of dynamic LDS per workgroup that the kernels never touch: it
  *     limits how many workgroups a CU holds at once;
  *   - all data pointers are device pointers on the current device; pointer
  *     TABLES (srcs, boxes) are host memory and are consumed before return;
@@ -151,8 +151,10 @@ int mdh_copy_boxes(const mdh_box* boxes, int nboxes, int itemsize, void* stream)
 
 /*
  * Launch-shape knobs, for measurement; 0 (the default) lets the library choose
- * by size.  Names: "reduce_unroll" (sub-tiles per lane: 1, 2, 4; 8 is taken as 4),
- * "reduce_max_blocks" (0 = one tile per workgroup), "reduce_wg_per_cu" (1..8
+ * by size.  Names: "reduce_unroll" (KiB of every source per tile: 1, 2, 4, 8, 16),
+ * "reduce_chunk" (sources whose loads are in flight together: 1, 2, 4, 8; the pairs
+ * compiled are 16x1, 16x2, 8x2, 4x4, 2x8, 1x8 and a call that forces another pair fails),
+ * "reduce_max_blocks" (waves of the grid; 0 = chosen by size), "reduce_wg_per_cu" (2..8
  * caps the workgroups resident on a CU, 9 = never cap), "copy_unroll" (1, 2,
  * 4, 8; contiguous segments), "box_unroll" (1, 2, 4, 8; strided boxes),
  * "copy_max_blocks", "copy_wg_per_cu" (2..8, 9 = never cap).  Returns MDH_EINVAL for an unknown name or value.

@@ -68,6 +68,9 @@ int* knob(const char* name) {
   if (!std::strcmp(name, "reduce_unroll")) {
     return &t.reduce_unroll;
   }
+  if (!std::strcmp(name, "reduce_chunk")) {
+    return &t.reduce_chunk;
+  }
   if (!std::strcmp(name, "reduce_max_blocks")) {
     return &t.reduce_max_blocks;
   }
@@ -96,9 +99,10 @@ extern "C" int mdh_set_tuning(const char* name, int value) {
     mdh::set_error("mdh_set_tuning: unknown knob");
     return MDH_EINVAL;
   }
-  const bool unroll = std::strstr(name, "unroll") != nullptr;
+  const bool unroll = std::strstr(name, "unroll") != nullptr || !std::strcmp(name, "reduce_chunk");
   if (unroll) {
-    if (!(value == 0 || value == 1 || value == 2 || value == 4 || value == 8)) {
+    const bool sixteen = value == 16 && !std::strcmp(name, "reduce_unroll");
+    if (!(value == 0 || value == 1 || value == 2 || value == 4 || value == 8 || sixteen)) {
       mdh::set_error("mdh_set_tuning: %s does not take %d", name, value);
       return MDH_EINVAL;
     }

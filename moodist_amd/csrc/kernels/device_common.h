@@ -80,7 +80,8 @@ int check_launch(const char* what);
 
 // 0 = choose by size (the default); any other value is taken as given.
 struct Tuning {
-  int reduce_unroll = 0;
+  int reduce_unroll = 0; // KiB of each source per tile: 1, 2, 4, 8, 16
+  int reduce_chunk = 0;  // sources in flight together: 1, 2, 4, 8
   int reduce_max_blocks = 0;
   int reduce_wg_per_cu = 0; // cap on resident workgroups per CU (1..8; 9 = none), through an unused LDS allocation
   int copy_unroll = 0; // contiguous segments

@@ -3,10 +3,10 @@
 //
 // What the reference does in K-1 two-source passes over the destination
 // (core/reduce_scatter.cc:104-142 emitting reduce_n2 calls,
-// core/kernels.cc:171-413) is done here in one pass: every lane issues one
-// 16-byte load per source (up to 8 sources x U tiles in flight), folds the
-// values in the reference's order in registers and writes 16 bytes once.
-// HBM traffic is (K+1) x bytes instead of (3K-3) x bytes.
+// core/kernels.cc:171-413) is done here in one pass: a wave takes a tile of up
+// to 16 KiB, reads it from every source in the reference's order (one, two,
+// four or eight sources' loads in flight at a time), folds in registers and
+// writes the tile once.  HBM traffic is (K+1) x bytes instead of (3K-3) x bytes.
 //
 // Fold order, element ops and the AVG / PREMUL_SUM rules are those of the
 // reference's CPU path (core/cputhread.cc:125-148, :3571-3587, :3680-3686;
@@ -156,12 +156,16 @@ constexpr int per_vec() {
   return 16 / (int)sizeof(typename Traits<T>::elem_t);
 }
 
+// A workgroup of the reduction is one wave: every wave is placed, runs and retires on its own,
+// and a launch aims at about one wave per SIMD (1024 on the chip).
+constexpr int kWave = 64;
+
 // Loads CNT sources' vectors for U sub-tiles (CNT*U loads in flight), then
 // folds them into acc in source order.  Each source is addressed through a
 // buffer descriptor whose base is the tile's first byte (wave-uniform, in
 // SGPRs) and whose size is the bytes left in the tile: the lane offset is one
 // VGPR, and vectors past the end read as zero instead of needing a predicate.
-template<typename T, int F, int CNT, int U, int MODE>
+template<typename T, int F, int CNT, int U, int MODE, bool FIRST>
 __device__ __forceinline__ void fold_chunk(const ReduceArgs& a, int j0, uint64_t tile_byte, uint32_t tile_bytes,
     uint32_t lane_byte, typename Traits<T>::acc_t (&acc)[U][per_vec<T>()]) {
   using Tr = Traits<T>;
@@ -174,13 +178,11 @@ __device__ __forceinline__ void fold_chunk(const ReduceArgs& a, int j0, uint64_t
     const __amdgpu_buffer_rsrc_t rs = tile_rsrc((const char*)a.src[j0 + k] + tile_byte, tile_bytes);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      v[k][u] = tile_load(rs, lane_byte + (uint32_t)u * (kBlock * 16));
+      v[k][u] = tile_load(rs, lane_byte + (uint32_t)u * (kWave * 16));
     }
   }
-  // Every load of the chunk is issued before the first add.  Without this fence the
-  // instruction scheduler interleaves loads with arithmetic to save registers (about a dozen
-  // loads in flight per lane instead of 8*U); on the eight-source workload both orders time the
-  // same, the fence just makes the number in flight independent of scheduler heuristics.
+  // Every load of the chunk is issued before the first add: the number in flight is then
+  // CNT*U whatever the instruction scheduler would have preferred.
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int k = 0; k < CNT; ++k) {
@@ -194,8 +196,8 @@ __device__ __forceinline__ void fold_chunk(const ReduceArgs& a, int j0, uint64_t
         if constexpr (MODE == kPremul) {
           x = Tr::premul(x, a.scale);
         }
-        if (k == 0 && j0 == 0) {
-          acc[u][i] = x;
+        if (FIRST && k == 0) {
+          acc[u][i] = x; // the first source initialises the accumulator (the reference's memcpy)
         } else {
           acc[u][i] = fold<F>(acc[u][i], x);
         }
@@ -228,72 +230,82 @@ __device__ __forceinline__ void reduce_one_elem(const ReduceArgs& a, int nsrc, u
   ((elem_t*)a.dst)[i] = Tr::template finish<F>(acc, a.mode, a.scale);
 }
 
-template<typename T, int F, int U, int MODE>
+// The sources left over when the count is not a multiple of CH (1 .. CH-1 of them).
+template<typename T, int F, int U, int CH, int MODE, bool FIRST, int R = CH - 1>
+__device__ __forceinline__ void fold_rest(const ReduceArgs& a, int rest, int j0, uint64_t tile_byte,
+    uint32_t tile_bytes, uint32_t lane_byte, typename Traits<T>::acc_t (&acc)[U][per_vec<T>()]) {
+  if constexpr (R >= 1) {
+    if (rest == R) {
+      fold_chunk<T, F, R, U, MODE, FIRST>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
+    } else {
+      fold_rest<T, F, U, CH, MODE, FIRST, R - 1>(a, rest, j0, tile_byte, tile_bytes, lane_byte, acc);
+    }
+  }
+}
+
+// One tile: U KiB of every source (U sub-tiles of one wave-wide 16-byte load each), consumed CH
+// sources at a time in order, so the fold stays a left fold and CH*U loads are in flight.
+template<typename T, int F, int U, int CH, int MODE>
 __device__ __forceinline__ void reduce_tile(const ReduceArgs& a, int nsrc, uint64_t tile_byte, uint32_t tile_bytes) {
   using Tr = Traits<T>;
   using elem_t = typename Tr::elem_t;
   using acc_t = typename Tr::acc_t;
   constexpr int N = per_vec<T>();
-  constexpr int CH = 8;
   const uint32_t lane_byte = threadIdx.x * 16;
   acc_t acc[U][N];
-  int j0 = 0;
-  for (; nsrc - j0 >= CH; j0 += CH) {
-    fold_chunk<T, F, CH, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
-  }
-  switch (nsrc - j0) {
-  case 1:
-    fold_chunk<T, F, 1, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
-    break;
-  case 2:
-    fold_chunk<T, F, 2, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
-    break;
-  case 3:
-    fold_chunk<T, F, 3, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
-    break;
-  case 4:
-    fold_chunk<T, F, 4, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
-    break;
-  case 5:
-    fold_chunk<T, F, 5, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
-    break;
-  case 6:
-    fold_chunk<T, F, 6, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
-    break;
-  case 7:
-    fold_chunk<T, F, 7, U, MODE>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
-    break;
-  default:
-    break;
+  // the first group is peeled so that "initialise or fold" is decided at compile time
+  if (nsrc >= CH) {
+    fold_chunk<T, F, CH, U, MODE, true>(a, 0, tile_byte, tile_bytes, lane_byte, acc);
+    int j0 = CH;
+    for (; nsrc - j0 >= CH; j0 += CH) {
+      fold_chunk<T, F, CH, U, MODE, false>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
+    }
+    fold_rest<T, F, U, CH, MODE, false>(a, nsrc - j0, j0, tile_byte, tile_bytes, lane_byte, acc);
+  } else {
+    fold_rest<T, F, U, CH, MODE, true>(a, nsrc, 0, tile_byte, tile_bytes, lane_byte, acc);
   }
   const __amdgpu_buffer_rsrc_t rd = tile_rsrc((const char*)a.dst + tile_byte, tile_bytes);
   u32x4 out[U];
+  // AVG's extra multiply is decided once per tile (wave-uniform), not per element
+  const int mode = MODE == kPremul ? (int)kPremul : a.mode;
+  if (mode == kAvg) {
 #pragma unroll
-  for (int u = 0; u < U; ++u) {
-    elem_t e[N];
+    for (int u = 0; u < U; ++u) {
+      elem_t e[N];
 #pragma unroll
-    for (int i = 0; i < N; ++i) {
-      e[i] = Tr::template finish<F>(acc[u][i], MODE == kPremul ? (int)kPremul : a.mode, a.scale);
+      for (int i = 0; i < N; ++i) {
+        e[i] = Tr::template finish<F>(acc[u][i], kAvg, a.scale);
+      }
+      __builtin_memcpy(&out[u], e, 16);
     }
-    __builtin_memcpy(&out[u], e, 16);
+  } else {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      elem_t e[N];
+#pragma unroll
+      for (int i = 0; i < N; ++i) {
+        e[i] = Tr::template finish<F>(acc[u][i], kPlain, a.scale);
+      }
+      __builtin_memcpy(&out[u], e, 16);
+    }
   }
   // results in registers of their own, then the stores back to back (a shared data register
   // would make each store wait for the one before it)
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int u = 0; u < U; ++u) {
-    tile_store(rd, lane_byte + (uint32_t)u * (kBlock * 16), out[u]); // dropped by the hardware past the end
+    tile_store(rd, lane_byte + (uint32_t)u * (kWave * 16), out[u]); // dropped by the hardware past the end
   }
 }
 
-// A tile is kBlock*U consecutive 16-byte vectors; tiles are dealt to
-// workgroups round-robin.  Pointers need only element alignment: gfx950's
+// A tile is kWave*U consecutive 16-byte vectors (U KiB); tiles are dealt to
+// waves round-robin.  Pointers need only element alignment: gfx950's
 // 16-byte buffer accesses take any byte address.  Elements past the last whole
 // vector (fewer than 16 bytes) are folded by workgroup 0.
-template<typename T, int F, int U, bool PREMUL>
-__global__ __launch_bounds__(kBlock) void reduce_vec_kernel(ReduceArgs a) {
+template<typename T, int F, int U, int CH, bool PREMUL>
+__global__ __launch_bounds__(kWave) void reduce_vec_kernel(ReduceArgs a) {
   const int nsrc = a.nsrc;
-  constexpr uint64_t tile_bytes = (uint64_t)kBlock * U * 16;
+  constexpr uint64_t tile_bytes = (uint64_t)kWave * U * 16;
   const uint64_t body_bytes = a.nvec * 16;
   const uint64_t ntiles = (body_bytes + tile_bytes - 1) / tile_bytes;
   for (uint64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
@@ -304,7 +316,7 @@ __global__ __launch_bounds__(kBlock) void reduce_vec_kernel(ReduceArgs a) {
     // element type after the multiply, which takes several times the registers of the plain
     // fold, and a kernel's register budget is that of its hungriest path.  AVG is the plain
     // fold with one more multiply when the result is written (a wave-uniform test there).
-    reduce_tile<T, F, U, PREMUL ? kPremul : kPlain>(a, nsrc, tile_byte, n);
+    reduce_tile<T, F, U, CH, PREMUL ? kPremul : kPlain>(a, nsrc, tile_byte, n);
   }
   if (blockIdx.x == 0) {
     const uint64_t i = a.nvec * per_vec<T>() + threadIdx.x;
@@ -315,41 +327,63 @@ __global__ __launch_bounds__(kBlock) void reduce_vec_kernel(ReduceArgs a) {
 }
 
 struct LaunchShape {
-  int unroll;    // sub-tiles per lane: 1, 2 or 4
-  int wg_per_cu; // 0 = as many as the registers allow
+  int unroll;     // sub-tiles (KiB of each source) per tile: 1, 2, 4, 8 or 16
+  int chunk;      // sources whose loads are in flight together: 1, 2, 4 or 8
+  uint64_t waves; // grid size
 };
 
-// Chosen by measurement on MI355X (TB/s of algorithmic bytes on one box; sub-tiles/workgroups
-// per CU, "-" = no cap):
-//   fp32  8 x 16 MiB   4/-: 6.34   2/-: 5.26   1/2: 5.36   2/2: 5.56
-//   fp32  8 x 32 MiB   4/-: 6.40   1/2: 6.08        8 x 48 MiB   4/-: 6.37   1/2: 6.52
-//   fp32  8 x 64 MiB   4/-: 6.34   1/2: 6.56        8 x 128 MiB  4/-: 6.30   1/2: 6.68
-//   fp32 16 x 32 MiB   4/-: 6.40   1/2: 6.23       16 x 48 MiB   4/-: 6.30   1/2: 6.69
-//   fp32 32 x 64 MiB   4/-: 5.97   1/2: 6.53       64 x 64 MiB   4/-: 6.42   1/2: 6.55
-//   bf16 16 x 16 MiB   4/-: 6.27   1/2: 5.35       16 x 64 MiB   4/-: 6.13   1/2: 6.64
-//   bf16  8 x 16 MiB   4/-: 6.10   2/2: 5.54        8 x 64 MiB   4/-: 6.32   2/2: 6.61   1/2: 6.08
-//   fp16  8 x 64 MiB   4/-: 6.30   1/2: 6.47   2/2: 5.96
-//   fp32  4 x 32 MiB   4/-: 6.48   1/2: 5.21   (few sources: a cap starves the CU)
-// Four sub-tiles and no cap is best or equal below about 48 MiB per source and with fewer
-// than eight sources.  Above that a launch spends most of its time in a steady state in
-// which reads and writes interleave at the DRAM, and two workgroups per CU with eight loads
-// in flight per lane do better (bf16 with eight or nine sources: sixteen).
+// Chosen by measurement on MI355X (percent of 8 TB/s, algorithmic bytes; one-wave workgroups;
+// tile KiB x sources in flight @ waves):
+//   fp32  8 x 16 MiB   16x1@1024: 84.4   16x1@512: 80.4   16x2@1024: 83.3   8x2@2048: 77.9   4x8@1024: 72.8
+//   fp32  8 x 64 MiB   16x1@512: 84.8    16x1@1024: 81.6  16x1@4096: 82.8   16x2@1024: 84.8  8x2@512: 83.8
+//   fp32 16 x 32 MiB   16x1@512: 86.8    16x1@1024: 85.2  16x2@1024: 86.3   8x1@1024: 84.2
+//   fp32 64 x 4 MiB    8x2@512: 87.0     16x1@256: 64.4   16x2@256: 78.1    4x4@1024: 80.0   4x2@1024: 85.9
+//   fp32 16 x 8 MiB    16x1@512: 83.1    8x1@1024: 83.9   8x2@1024: 80.0
+//   fp32  2 x 64 MiB   16x1@512: 84.3    8x2@512: 84.5    16x2@1024: 77.7
+//   fp32  8 x 4 MiB    4x8@1024: 63.7    8x2@512: 60.3    16x1@256: 52.6
+//   fp32  8 x 1 MiB    2x8@512: 31.3     4x8@256: 30.5    16x1@64: 16.1
+//   bf16 16 x 64 MiB   16x1@4096: 84.0   16x1@1024: 82.5  16x1@512: 78.6    8x2@512: 80.8    16x2@1024: 82.5
+//   bf16  8 x 16 MiB   16x1@1024: 79.4   16x1@512: 65.1   8x2@1024: 73.6    4x4@4096: 75.0
+// against 79.4 / 80.1 / 78.6 / 82.3 / 77.8 / 72.2 / 63.0 / 24.2 (fp32) for 256-lane workgroups that keep
+// eight sources x 4 KiB in flight per lane.  What the good shapes share: the longest tile that
+// still leaves about 512 tiles, sixteen loads in flight per lane, one source (or two) at a time,
+// and no more than about one wave per SIMD -- the chip then sweeps one source after the other
+// and the writes come in a burst of their own, instead of nine streams interleaving at the DRAM.
 template<typename T, bool PREMUL>
 LaunchShape choose_shape(const ReduceArgs& a) {
   const Tuning& t = tuning();
   constexpr bool half = sizeof(typename Traits<T>::elem_t) == 2;
-  LaunchShape s{auto_unroll(a.nvec, 4), 0};
-  if (PREMUL && half) {
-    s.unroll = 1; // the per-element rounding of PREMUL_SUM fills the register file on its own
-  } else if (!PREMUL && a.nvec >= ((uint64_t)48 << 20) / 16 && a.nsrc >= 8) {
-    s.unroll = (std::is_same_v<T, bf16_t> && a.nsrc < 10) ? 2 : 1;
-    s.wg_per_cu = 2;
+  int u = 16;
+  while (u > 1 && a.nvec / ((uint64_t)kWave * u) < 512) {
+    u >>= 1;
   }
+  if (PREMUL && half && u > 4) {
+    u = 4; // the per-element rounding of PREMUL_SUM needs several registers per element
+  }
+  int ch = u >= 16 ? 1 : 16 / u > 8 ? 8 : 16 / u;
   if (t.reduce_unroll) {
-    s.unroll = t.reduce_unroll > 4 ? 4 : t.reduce_unroll;
+    u = t.reduce_unroll;
+    ch = u >= 16 ? 1 : 16 / u > 8 ? 8 : 16 / u;
   }
-  if (t.reduce_wg_per_cu) {
-    s.wg_per_cu = t.reduce_wg_per_cu > 8 ? 0 : t.reduce_wg_per_cu; // 9 = no cap
+  if (t.reduce_chunk) {
+    ch = t.reduce_chunk;
+    if (!t.reduce_unroll) {
+      u = ch == 1 ? 16 : ch == 2 ? (u >= 16 ? 16 : 8) : ch == 4 ? 4 : u > 2 ? 2 : u;
+    }
+  }
+  LaunchShape s{u, ch, 0};
+  const uint64_t tile_vecs = (uint64_t)kWave * u;
+  uint64_t ntiles = (a.nvec + tile_vecs - 1) / tile_vecs;
+  if (ntiles == 0) {
+    ntiles = 1; // tail only
+  }
+  // From two tiles per SIMD on, 512 waves that walk the tiles keep fewer streams open (fp32
+  // 8 x 64 MiB: 84.8 % against 82.8 % with a wave per tile).  16-bit types spend three to four
+  // times the arithmetic per byte (widening), which a lone wave on a SIMD cannot overlap with its
+  // own loads: they keep a wave per tile (bf16 16 x 64 MiB: 84.0 % against 78.6 % with 512 waves).
+  s.waves = (ntiles >= 2048 && !half) ? 512 : ntiles;
+  if (t.reduce_max_blocks > 0) {
+    s.waves = ntiles < (uint64_t)t.reduce_max_blocks ? ntiles : (uint64_t)t.reduce_max_blocks;
   }
   return s;
 }
@@ -358,47 +392,25 @@ template<typename T, int F, bool PREMUL = false>
 int launch_vec(const ReduceArgs& a, hipStream_t stream) {
   const Tuning& t = tuning();
   const LaunchShape shape = choose_shape<T, PREMUL>(a);
-  const int U = shape.unroll;
-  const uint64_t tile_vecs = (uint64_t)kBlock * U;
-  uint64_t ntiles = (a.nvec + tile_vecs - 1) / tile_vecs;
-  if (ntiles == 0) {
-    ntiles = 1; // tail only
+  dim3 g((unsigned)shape.waves), b(kWave);
+  // reduce_wg_per_cu (measurement only): an unused LDS allocation caps the waves resident on a CU
+  const int cap = t.reduce_wg_per_cu >= 2 && t.reduce_wg_per_cu <= 8 ? t.reduce_wg_per_cu : 0;
+  const size_t lds = kLdsForCap[cap];
+#define MDH_LAUNCH_REDUCE(UU, CC)                                                  \
+  if (shape.unroll == UU && shape.chunk == CC) {                                   \
+    hipLaunchKernelGGL((reduce_vec_kernel<T, F, UU, CC, PREMUL>), g, b, lds, stream, a); \
+    return check_launch("reduce_vec_kernel");                                      \
   }
-  uint64_t grid = ntiles;
-  if (t.reduce_max_blocks > 0 && grid > (uint64_t)t.reduce_max_blocks) {
-    grid = t.reduce_max_blocks;
-  }
-  if (grid > 0x7fffffffull) {
-    grid = 0x7fffffffull;
-  }
-  dim3 g((unsigned)grid), b(kBlock);
-  const size_t lds = kLdsForCap[shape.wg_per_cu];
-#define MDH_LAUNCH_REDUCE(UU)                                                                            \
-  do {                                                                                                   \
-    auto* fn = reduce_vec_kernel<T, F, UU, PREMUL>;                                                      \
-    if (lds > 65536) {                                                                                   \
-      /* more than 64 KiB of dynamic LDS has to be allowed once per kernel */                            \
-      static bool raised = false;                                                                        \
-      if (!raised) {                                                                                     \
-        if (hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) { \
-          (void)hipGetLastError();                                                                       \
-          set_error("reduce_vec_kernel: the device refused %zu bytes of dynamic LDS", lds);              \
-          return MDH_ELAUNCH;                                                                            \
-        }                                                                                                \
-        raised = true;                                                                                   \
-      }                                                                                                  \
-    }                                                                                                    \
-    hipLaunchKernelGGL(fn, g, b, lds, stream, a);                                                        \
-  } while (0)
-  if (U == 1) {
-    MDH_LAUNCH_REDUCE(1);
-  } else if (U == 2) {
-    MDH_LAUNCH_REDUCE(2);
-  } else {
-    MDH_LAUNCH_REDUCE(4);
-  }
+  MDH_LAUNCH_REDUCE(16, 1)
+  MDH_LAUNCH_REDUCE(16, 2)
+  MDH_LAUNCH_REDUCE(8, 2)
+  MDH_LAUNCH_REDUCE(4, 4)
+  MDH_LAUNCH_REDUCE(2, 8)
+  MDH_LAUNCH_REDUCE(1, 8)
 #undef MDH_LAUNCH_REDUCE
-  return check_launch("reduce_vec_kernel");
+  set_error("reduce: no kernel for %d sub-tiles x %d sources in flight (compiled: 16x1, 16x2, 8x2, 4x4, 2x8, 1x8)",
+      shape.unroll, shape.chunk);
+  return MDH_EINVAL;
 }
 
 template<typename T, int F>
