@@ -77,7 +77,8 @@ int moodist_pg_rank(moodist_pg* pg);
 int moodist_pg_size(moodist_pg* pg);
 /* processGroupGetOption / processGroupSetOption (api/processgroup_api.h:39-40).
  * Names as in the reference (core/processgroup.cc:2455-2488): prefer_kernel_less,
- * force_kernel_less, num_chunks, chunk_size, method.  Unknown name -> error. */
+ * force_kernel_less, num_chunks, chunk_size, method; and snapshot_inputs (not in the
+ * reference; needs a core loaded through moodistGetApi).  Unknown name -> error. */
 int moodist_pg_get_option(moodist_pg* pg, const char* name, int64_t* value);
 int moodist_pg_set_option(moodist_pg* pg, const char* name, int64_t value);
 
@@ -106,6 +107,20 @@ int moodist_pg_allreduce(moodist_pg* pg, const moodist_tensor* tensor, const moo
  * for an output.  kind: 0 = all_gather, 1 = reduce_scatter. */
 int moodist_pg_stage_input(moodist_pg* pg, int kind, const moodist_tensor* input, int reduce_op, void* stream,
     float premul_value, moodist_work** work);
+
+/* The work of the collective this rank posted most recently (a new reference; NULL into *work
+ * if it has posted none).  For callers of the CoreApi table, whose collectives return nothing
+ * (api/processgroup_api.h:43-49) -- there a call has done its part when it returns, here the
+ * launch may still be waiting for other ranks.  No counterpart in the reference. */
+int moodist_pg_last_work(moodist_pg* pg, moodist_work** work);
+
+/* Ties `ctx` to the collective this rank posted most recently: release(ctx) is called exactly
+ * once, when that collective's launches have been enqueued (at once if they already have, or
+ * if the rank has posted nothing).  For the buffers of the calls above, which the core reads
+ * when the LAST rank posts: the caller keeps them alive at least that long.  The reference
+ * holds tensor references inside the operation instead (core/processgroup.cc:3239-3245), as
+ * the CoreApi table of moodist_plugin.h does here. */
+int moodist_pg_keep_alive(moodist_pg* pg, void* ctx, void (*release)(void* ctx));
 
 /* Work: wait() fails if not every rank has posted yet (the launch has not happened). */
 int moodist_work_is_completed(moodist_work* work);

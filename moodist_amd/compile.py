@@ -8,6 +8,8 @@ ranks of a LocalWorld share a process, so the gathering is a list on the world, 
 operation a rank gets back becomes callable once the last rank has called compile_op.
 """
 
+import weakref
+
 import torch
 
 
@@ -89,12 +91,18 @@ def _check(specs, ndim):
 class _Round:
     """One collective compile_op call: what every rank of the world has said so far."""
 
-    def __init__(self, size):
+    def __init__(self, size, first_group):
         self.size = size
         self.info = {}
+        # the group that opened the round: once it is gone the round is stale (the store's id may
+        # by then name another object)
+        self.first = weakref.ref(first_group)
 
     def complete(self):
         return len(self.info) == self.size
+
+
+_rounds = {}  # id(store) -> the round the ranks of that store's world are filling
 
 
 class CompiledOp:
@@ -158,9 +166,10 @@ def compile_op(group, shape=None, dtype=None, inputs=None, outputs=None):
     if outputs is not None:
         outputs = _check(outputs, len(shape))
 
-    world = group.world
-    rnd = world._compile_round
-    if rnd is None or rnd.complete() or group.rank() in rnd.info:
-        rnd = world._compile_round = _Round(world.size)
+    # the ranks of a world share a store object: its identity names the round being gathered
+    key = id(group._store)
+    rnd = _rounds.get(key)
+    if rnd is None or rnd.first() is None or rnd.complete() or group.rank() in rnd.info:
+        rnd = _rounds[key] = _Round(group.size(), group)
     rnd.info[group.rank()] = (shape, dtype, inputs, outputs)
     return CompiledOp(group, rnd)

@@ -8,10 +8,10 @@ here="$(cd "$(dirname "$0")" && pwd)"
 root="$(cd "$here/../.." && pwd)"
 pkg="$here/.."
 cxx="${CXX:-g++}"
-common=(-O2 -std=c++17 -fPIC -Wall -Wextra -fvisibility=hidden -I"$root/include" -I"$here/core")
+common=(-O2 -std=c++20 -fPIC -Wall -Wextra -fvisibility=hidden -I"$root/include" -I"$here/core")
 mkdir -p "$here/build"
 objs=()
-for f in hip_loader planner processgroup c_api; do
+for f in hip_loader planner processgroup c_api plugin; do
   o="$here/build/core_$f.o"
   "$cxx" "${common[@]}" -c "$here/core/$f.cc" -o "$o" &
   objs+=("$o")

@@ -6,25 +6,12 @@
 #include <string>
 #include <vector>
 
+#include "c_handles.h"
 #include "hip_loader.h"
 #include "moodist_core.h"
 #include "processgroup.h"
 
 using namespace moodist;
-
-struct moodist_world {
-  std::unique_ptr<World> impl;
-};
-struct moodist_work {
-  std::shared_ptr<Collective> c;
-};
-struct moodist_op {
-  ProcessGroup* pg;
-  std::shared_ptr<CompiledOp> op;
-};
-struct moodist_future {
-  std::shared_ptr<Collective> c;
-};
 
 namespace {
 
@@ -96,7 +83,7 @@ int moodist_world_create(int size, int device, moodist_world** world) {
     if (!world) {
       throw std::runtime_error("moodist: null out pointer");
     }
-    *world = new moodist_world{std::make_unique<World>(size, device)};
+    *world = new moodist_world{std::make_shared<World>(size, device)};
   });
 }
 
@@ -180,6 +167,29 @@ int moodist_pg_stage_input(moodist_pg* pg, int kind, const moodist_tensor* input
       give(work, as_pg(pg)->reduce_scatter(nullptr, *input, reduce_op, stream, premul_value));
     } else {
       throw std::runtime_error("moodist: stage_input kind must be 0 (all_gather) or 1 (reduce_scatter)");
+    }
+  });
+}
+
+int moodist_pg_last_work(moodist_pg* pg, moodist_work** work) {
+  return guarded([&] {
+    if (!work) {
+      throw std::runtime_error("moodist: null out pointer");
+    }
+    std::shared_ptr<Collective> c = as_pg(pg)->last;
+    *work = c ? new moodist_work{std::move(c)} : nullptr;
+  });
+}
+
+int moodist_pg_keep_alive(moodist_pg* pg, void* ctx, void (*release)(void* ctx)) {
+  return guarded([&] {
+    if (!release) {
+      throw std::runtime_error("moodist: null release function");
+    }
+    std::shared_ptr<void> held(ctx, release); // from here on `ctx` is released exactly once
+    ProcessGroup* g = as_pg(pg);
+    if (g->last) {
+      g->world->attach(*g->last, g->rank, std::move(held));
     }
   });
 }

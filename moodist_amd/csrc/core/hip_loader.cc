@@ -35,11 +35,20 @@ std::string sibling_kernel_library() {
 HipRuntime load() {
   HipRuntime r{};
   void* rt = nullptr;
-  for (const char* name : {"libamdhip64.so", "libamdhip64.so.7", "libamdhip64.so.6", "/opt/rocm/lib/libamdhip64.so"}) {
-    rt = dlopen(name, RTLD_NOW | RTLD_GLOBAL);
+  const char* const names[] = {"libamdhip64.so.7", "libamdhip64.so.6", "libamdhip64.so", "/opt/rocm/lib/libamdhip64.so"};
+  // a runtime the process has already mapped (torch's) is the one to use: a second copy would
+  // have its own device state
+  for (const char* name : names) {
+    rt = dlopen(name, RTLD_NOW | RTLD_GLOBAL | RTLD_NOLOAD);
     if (rt) {
       break;
     }
+  }
+  for (const char* name : names) {
+    if (rt) {
+      break;
+    }
+    rt = dlopen(name, RTLD_NOW | RTLD_GLOBAL);
   }
   if (!rt) {
     throw std::runtime_error(std::string("moodist: cannot load the HIP runtime (libamdhip64.so): ") + dlerror());

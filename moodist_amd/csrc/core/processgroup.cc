@@ -152,6 +152,8 @@ int64_t ProcessGroup::get_option(const std::string& name) const {
     return options.chunkSize;
   } else if (name == "method") {
     return options.method;
+  } else if (name == "snapshot_inputs") {
+    return options.snapshotInputs ? 1 : 0;
   }
   throw std::runtime_error("Unknown option: " + name);
 }
@@ -167,24 +169,48 @@ void ProcessGroup::set_option(const std::string& name, int64_t value) {
     options.chunkSize = value;
   } else if (name == "method") {
     options.method = value;
+  } else if (name == "snapshot_inputs") {
+    if (value != 0 && !world->allocator.alloc) {
+      throw std::runtime_error("moodist: snapshot_inputs needs a device allocator, which only a core loaded through "
+                               "moodistGetApi has (the wrapper's caching allocator)");
+    }
+    options.snapshotInputs = value != 0;
   } else {
     throw std::runtime_error("Unknown option: " + name);
   }
 }
 
+void ProcessGroup::snapshot(moodist_tensor& input, void* stream, Keep& keep) {
+  const size_t bytes = bytes_of(input);
+  if (!options.snapshotInputs || internal_input || bytes == 0) {
+    return;
+  }
+  void* cleanup = nullptr;
+  void* copy = world->allocator.alloc(bytes, &cleanup, stream, world->device);
+  if (!copy) {
+    throw std::runtime_error("moodist: could not allocate " + std::to_string(bytes) + " bytes for an input snapshot");
+  }
+  auto release = world->allocator.free;
+  keep.push_back(std::shared_ptr<void>(cleanup, [release](void* c) { release(c); }));
+  check_hip(hip().MemcpyAsync(copy, input.data, bytes, kHipMemcpyDeviceToDevice, stream), "hipMemcpyAsync");
+  input.data = copy;
+}
+
 std::shared_ptr<Collective> ProcessGroup::all_gather(const moodist_tensor* output, const moodist_tensor& input,
-    void* stream) {
-  return all_gather_impl(output, input, stream, nullptr);
+    void* stream, Keep keep) {
+  return all_gather_impl(output, input, stream, nullptr, std::move(keep));
 }
 
 std::shared_ptr<Collective> ProcessGroup::all_gather_impl(const moodist_tensor* output, const moodist_tensor& input,
-    void* stream, const moodist_tensor* copy_back) {
+    void* stream, const moodist_tensor* copy_back, Keep keep) {
   Busy guard(*this);
   check_device_tensor(input, world->device, "all_gather input");
   const size_t bytes = bytes_of(input);
   MD_CHECK(bytes > 0); // core/processgroup.cc:1078
   Posting p;
   p.input = input;
+  snapshot(p.input, stream, keep);
+  p.keep = std::move(keep);
   p.stream = stream;
   if (output) {
     check_device_tensor(*output, world->device, "all_gather output");
@@ -197,14 +223,14 @@ std::shared_ptr<Collective> ProcessGroup::all_gather_impl(const moodist_tensor* 
     }
   }
   p.kernel_less = options.forceKernelLess || options.preferKernelLess;
-  return world->post(Kind::all_gather, next_seq++, rank, std::move(p), 0, 1.0f, bytes, input.dtype, 0, nullptr);
+  return last = world->post(Kind::all_gather, next_seq++, rank, std::move(p), 0, 1.0f, bytes, input.dtype, 0, nullptr);
 }
 
 // The list form of all_gather (wrapper/processgroup_wrapper.cc:112-129).  The reference gathers
 // into a flat temporary and copies each row out; here every source is copied straight into its
 // destination tensor, so no temporary exists.
 std::shared_ptr<Collective> ProcessGroup::all_gather_list(const moodist_tensor* outputs, size_t n_outputs,
-    const moodist_tensor& input, void* stream) {
+    const moodist_tensor& input, void* stream, Keep keep) {
   Busy guard(*this);
   check_device_tensor(input, world->device, "all_gather input");
   const size_t bytes = bytes_of(input);
@@ -215,6 +241,8 @@ std::shared_ptr<Collective> ProcessGroup::all_gather_list(const moodist_tensor* 
   }
   Posting p;
   p.input = input;
+  snapshot(p.input, stream, keep);
+  p.keep = std::move(keep);
   p.stream = stream;
   p.wants_output = true;
   for (size_t i = 0; i < n_outputs; ++i) {
@@ -224,11 +252,11 @@ std::shared_ptr<Collective> ProcessGroup::all_gather_list(const moodist_tensor* 
     p.outputs.push_back(outputs[i]);
   }
   p.kernel_less = options.forceKernelLess || options.preferKernelLess;
-  return world->post(Kind::all_gather, next_seq++, rank, std::move(p), 0, 1.0f, bytes, input.dtype, 0, nullptr);
+  return last = world->post(Kind::all_gather, next_seq++, rank, std::move(p), 0, 1.0f, bytes, input.dtype, 0, nullptr);
 }
 
 std::shared_ptr<Collective> ProcessGroup::reduce_scatter(const moodist_tensor* output, const moodist_tensor& input,
-    int reduce_op, void* stream, float premul) {
+    int reduce_op, void* stream, float premul, Keep keep) {
   Busy guard(*this);
   check_device_tensor(input, world->device, "reduce_scatter input");
   check_reduce_dtype(input.dtype);
@@ -244,6 +272,8 @@ std::shared_ptr<Collective> ProcessGroup::reduce_scatter(const moodist_tensor* o
   MD_CHECK(bytes % (size_t)input.itemsize == 0);
   Posting p;
   p.input = input;
+  snapshot(p.input, stream, keep);
+  p.keep = std::move(keep);
   p.stream = stream;
   if (output) {
     check_device_tensor(*output, world->device, "reduce_scatter output");
@@ -252,12 +282,12 @@ std::shared_ptr<Collective> ProcessGroup::reduce_scatter(const moodist_tensor* o
     p.output = *output;
     p.wants_output = true;
   }
-  return world->post(Kind::reduce_scatter, next_seq++, rank, std::move(p), reduce_op, premul, bytes, input.dtype, 0,
-      nullptr);
+  return last = world->post(Kind::reduce_scatter, next_seq++, rank, std::move(p), reduce_op, premul, bytes,
+             input.dtype, 0, nullptr);
 }
 
 std::shared_ptr<Collective> ProcessGroup::allreduce(const moodist_tensor& tensor, const moodist_tensor* scratch,
-    int reduce_op, void* stream, float premul) {
+    int reduce_op, void* stream, float premul, Keep keep) {
   check_device_tensor(tensor, world->device, "allreduce tensor");
   MD_CHECK(tensor.numel > 0); // core/processgroup.cc:1678
   const int64_t n = tensor.numel;
@@ -268,8 +298,16 @@ std::shared_ptr<Collective> ProcessGroup::allreduce(const moodist_tensor& tensor
     chunk.data = (char*)tensor.data + (size_t)rank * (size_t)chunk.numel * (size_t)tensor.itemsize;
     chunk.ndim = 1;
     chunk.shape[0] = chunk.numel;
-    reduce_scatter(&chunk, tensor, reduce_op, stream, premul);
-    return all_gather(&tensor, chunk, stream);
+    reduce_scatter(&chunk, tensor, reduce_op, stream, premul, keep); // both halves hold the tensor
+    // the gather's input is what the reduction will have written by then: never a snapshot
+    internal_input = true;
+    struct Reset {
+      bool& flag;
+      ~Reset() {
+        flag = false;
+      }
+    } reset{internal_input};
+    return all_gather(&tensor, chunk, stream, std::move(keep));
   }
   // padded temporary (:1694-1720)
   const int64_t padded = (n + size - 1) / size * size;
@@ -289,9 +327,17 @@ std::shared_ptr<Collective> ProcessGroup::allreduce(const moodist_tensor& tensor
   chunk.numel = padded / size;
   chunk.data = (char*)whole.data + (size_t)rank * (size_t)chunk.numel * (size_t)tensor.itemsize;
   chunk.shape[0] = chunk.numel;
-  reduce_scatter(&chunk, whole, reduce_op, stream, premul);
+  // `whole` already is a copy made at the call's position in the stream: no second snapshot
+  internal_input = true;
+  struct Reset {
+    bool& flag;
+    ~Reset() {
+      flag = false;
+    }
+  } reset{internal_input};
+  reduce_scatter(&chunk, whole, reduce_op, stream, premul, keep);
   // the copy back into `tensor` follows this rank's gather, wherever that gets launched
-  return all_gather_impl(&whole, chunk, stream, &tensor);
+  return all_gather_impl(&whole, chunk, stream, &tensor, std::move(keep));
 }
 
 std::shared_ptr<CompiledOp> ProcessGroup::compile_op_full(const Dims& shape, int dtype,
@@ -326,7 +372,8 @@ std::shared_ptr<CompiledOp> ProcessGroup::compile_op_full(const Dims& shape, int
 }
 
 std::shared_ptr<Collective> ProcessGroup::custom_op(const std::shared_ptr<CompiledOp>& op,
-    const moodist_tensor* inputs, size_t n_inputs, const moodist_tensor* outputs, size_t n_outputs, void* stream) {
+    const moodist_tensor* inputs, size_t n_inputs, const moodist_tensor* outputs, size_t n_outputs, void* stream,
+    Keep keep) {
   Busy guard(*this);
   const RankPlan& plan = op->plans[(size_t)rank];
   // core/processgroup.cc:3180-3185, :3205-3216
@@ -337,6 +384,7 @@ std::shared_ptr<Collective> ProcessGroup::custom_op(const std::shared_ptr<Compil
     throw std::runtime_error("moodist: custom op expected different number of outputs");
   }
   Posting p;
+  p.keep = std::move(keep);
   p.stream = stream;
   p.wants_output = n_outputs > 0;
   for (size_t i = 0; i < n_inputs; ++i) {
@@ -359,7 +407,7 @@ std::shared_ptr<Collective> ProcessGroup::custom_op(const std::shared_ptr<Compil
     check_device_tensor(outputs[i], world->device, "custom op output");
     p.outputs.push_back(outputs[i]);
   }
-  return world->post(Kind::custom, next_seq++, rank, std::move(p), 0, 1.0f, 0, op->dtype, op->id, op);
+  return last = world->post(Kind::custom, next_seq++, rank, std::move(p), 0, 1.0f, 0, op->dtype, op->id, op);
 }
 
 // ---------------------------------------------------------------- World
@@ -412,6 +460,16 @@ std::shared_ptr<Collective> World::post(Kind kind, uint64_t seq, int rank, Posti
   ++c->arrived;
   if (c->arrived == size) {
     pending.erase(seq);
+    // what the ranks asked to keep alive is let go once the launches are enqueued (or have
+    // failed): from then on stream order protects the buffers
+    struct Release {
+      Collective& c;
+      ~Release() {
+        for (Posting& q : c.post) {
+          q.keep.clear();
+        }
+      }
+    } release{*c};
     try {
       launch(*c, op);
     } catch (const std::exception& e) {
@@ -422,6 +480,13 @@ std::shared_ptr<Collective> World::post(Kind kind, uint64_t seq, int rank, Posti
     c->launched = true;
   }
   return c;
+}
+
+void World::attach(Collective& c, int rank, std::shared_ptr<void> held) {
+  std::lock_guard<std::mutex> l(mutex);
+  if (!c.launched && rank >= 0 && rank < size) {
+    c.post[(size_t)rank].keep.push_back(std::move(held));
+  }
 }
 
 // A rank's launch reads buffers that other ranks' streams may still be producing, and later

@@ -35,6 +35,19 @@ struct Posting {
   bool has_copy_back = false; // allreduce through a padded temporary
   moodist_tensor copy_back{};
   void* stream = nullptr;
+  // Whatever must stay alive until this rank's buffers have been read by the launches of the
+  // collective (tensor references, snapshot buffers); dropped right after the launches are
+  // enqueued, as the reference ties lifetime to the operation (core/processgroup.cc:3239-3245).
+  std::vector<std::shared_ptr<void>> keep;
+};
+
+using Keep = std::vector<std::shared_ptr<void>>;
+
+// Device memory for snapshots, supplied by whoever loaded the core (the reference's core
+// allocates through the wrapper's caching allocator the same way, api/moodist_api.h:71-74).
+struct DeviceAllocator {
+  void* (*alloc)(size_t bytes, void** cleanup, void* stream, int device) = nullptr;
+  void (*free)(void* cleanup) = nullptr;
 };
 
 struct Collective {
@@ -57,6 +70,9 @@ struct Options { // core/processgroup.cc:334-340
   int64_t numChunks = -1;
   int64_t chunkSize = -1;
   int64_t method = -1;
+  // Not in the reference: copy every posted input at the call's position in the rank's stream,
+  // so that the collective reads the values of call time even though it is launched later.
+  bool snapshotInputs = false;
 };
 
 struct CompiledOp {
@@ -72,17 +88,19 @@ class ProcessGroup {
 public:
   ProcessGroup(World* world, int rank, int size) : world(world), rank(rank), size(size) {}
 
-  std::shared_ptr<Collective> all_gather(const moodist_tensor* output, const moodist_tensor& input, void* stream);
+  // `keep` rides with the posting and is released once the collective's launches are enqueued.
+  std::shared_ptr<Collective> all_gather(const moodist_tensor* output, const moodist_tensor& input, void* stream,
+      Keep keep = {});
   std::shared_ptr<Collective> all_gather_list(const moodist_tensor* outputs, size_t n_outputs,
-      const moodist_tensor& input, void* stream);
+      const moodist_tensor& input, void* stream, Keep keep = {});
   std::shared_ptr<Collective> reduce_scatter(const moodist_tensor* output, const moodist_tensor& input, int reduce_op,
-      void* stream, float premul);
+      void* stream, float premul, Keep keep = {});
   std::shared_ptr<Collective> allreduce(const moodist_tensor& tensor, const moodist_tensor* scratch, int reduce_op,
-      void* stream, float premul);
+      void* stream, float premul, Keep keep = {});
   std::shared_ptr<CompiledOp> compile_op_full(const Dims& shape, int dtype, const std::vector<SliceSpec>& inputs,
       const std::vector<SliceSpec>& outputs);
   std::shared_ptr<Collective> custom_op(const std::shared_ptr<CompiledOp>& op, const moodist_tensor* inputs,
-      size_t n_inputs, const moodist_tensor* outputs, size_t n_outputs, void* stream);
+      size_t n_inputs, const moodist_tensor* outputs, size_t n_outputs, void* stream, Keep keep = {});
 
   int64_t get_option(const std::string& name) const;
   void set_option(const std::string& name, int64_t value);
@@ -91,10 +109,14 @@ public:
   const int rank;
   const int size;
   Options options;
+  std::shared_ptr<Collective> last; // the collective this rank posted most recently
 
 private:
   std::shared_ptr<Collective> all_gather_impl(const moodist_tensor* output, const moodist_tensor& input, void* stream,
-      const moodist_tensor* copy_back);
+      const moodist_tensor* copy_back, Keep keep);
+  // snapshot_inputs: replaces input.data by a copy made now on `stream`; the copy joins `keep`
+  void snapshot(moodist_tensor& input, void* stream, Keep& keep);
+  bool internal_input = false; // the second half of an allreduce: its input does not exist yet
 
   // "Concurrent use of process group detected" guard (core/processgroup.cc:172-183)
   struct Busy {
@@ -123,8 +145,13 @@ public:
   std::shared_ptr<Collective> post(Kind kind, uint64_t seq, int rank, Posting p, int reduce_op, float premul,
       size_t bytes, int dtype, uint32_t op_id, const std::shared_ptr<CompiledOp>& op);
 
+  // Adds `held` to what rank `rank` keeps alive for collective `c`; if the collective has
+  // launched already, `held` is simply dropped.
+  void attach(Collective& c, int rank, std::shared_ptr<void> held);
+
   const int size;
   const int device;
+  DeviceAllocator allocator; // empty unless the loader supplied one
 
 private:
   void launch(Collective& c, const std::shared_ptr<CompiledOp>& op);

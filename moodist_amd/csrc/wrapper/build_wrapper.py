@@ -21,7 +21,7 @@ out = os.path.join(pkg, "_C" + sysconfig.get_config_var("EXT_SUFFIX"))
 inc = cpp_extension.include_paths() + [sysconfig.get_paths()["include"], os.path.join(root, "include"),
                                        "/opt/rocm/include"]
 libdir = os.path.join(os.path.dirname(torch.__file__), "lib")
-cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
+cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++20", "-fPIC", "-shared", "-fvisibility=hidden",
        "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI), "-D__HIP_PLATFORM_AMD__=1",
        "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=_C", "-Wno-deprecated-declarations"]
 cmd += ["-I" + p for p in inc]

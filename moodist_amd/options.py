@@ -2,10 +2,13 @@
 
 Same surface as the reference's py/moodist/options.py:55-113: ``pg.options().name`` reads,
 ``pg.options().name = v`` writes, ``with pg.options(name=v):`` overrides for a block.  Booleans
-travel as 0/1 and "auto" as -1 (api/processgroup_api.h:35-40).
+travel as 0/1 and "auto" as -1 (api/processgroup_api.h:35-40).  ``snapshot_inputs`` is this
+build's addition.
 """
 
-_BOOL = ("prefer_kernel_less", "force_kernel_less")
+import contextlib
+
+_BOOL = ("prefer_kernel_less", "force_kernel_less", "snapshot_inputs")
 _INT = ("num_chunks", "chunk_size", "method")
 
 
@@ -23,22 +26,22 @@ def _decode(name, raw):
     return None if raw == -1 else raw
 
 
-class MoodistOptionsContext:
-    def __init__(self, pg, overrides):
-        self._pg = pg
-        self._overrides = overrides
-        self._saved = {}
+@contextlib.contextmanager
+def _override(pg, raw_values):
+    """Applies the raw values for the duration of a with-block, then puts back what was there
+    before, last change first."""
+    undo = contextlib.ExitStack()
+    with undo:
+        for name, raw in raw_values:
+            undo.callback(pg._set_option, name, pg._get_option(name))
+            pg._set_option(name, raw)
+        yield pg
 
-    def __enter__(self):
-        for name, raw in self._overrides.items():
-            self._saved[name] = self._pg._get_option(name)
-            self._pg._set_option(name, raw)
-        return self._pg
 
-    def __exit__(self, *exc):
-        for name, raw in self._saved.items():
-            self._pg._set_option(name, raw)
-        return False
+def MoodistOptionsContext(pg, overrides):
+    """The context manager ``pg.options(name=value, ...)`` returns; `overrides` maps names to raw
+    (encoded) values."""
+    return _override(pg, list(overrides.items()))
 
 
 class MoodistOptions:

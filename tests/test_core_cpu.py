@@ -382,16 +382,33 @@ def test_options_object():
 
 
 def test_process_group_is_a_c10d_process_group():
+    # reference: the Python type IS a torch.distributed.ProcessGroup (wrapper/module.cc:851-865)
     import torch.distributed as dist
 
     world = moodist_amd.LocalWorld(3, 0)
     for r, pg in enumerate(world):
-        assert isinstance(pg.c10d, dist.ProcessGroup)
+        assert isinstance(pg, dist.ProcessGroup) and isinstance(pg, moodist_amd.MoodistProcessGroup)
         assert pg.rank() == r and pg.size() == 3
-        assert pg.moodist_name() == "moodist-local-%d-of-3-world%d" % (r, world.serial)
+        assert pg.moodist_name().startswith("moodist-local-%d-of-3-world" % r)
         assert moodist_amd.find_process_group(pg.moodist_name()) is pg
+        assert pg.world is world
+    assert len({pg.moodist_name() for pg in world}) == 3
     with pytest.raises(RuntimeError, match="send is not supported"):
         world.groups[0].send([torch.zeros(1)], 1, 0)
+
+
+def test_torch_distributed_functions_take_the_group():
+    # torch.distributed's own functions accept the object as group= and reach the overrides; with
+    # CPU tensors the core then refuses (this build has no CPU path), which shows where the call went
+    import torch.distributed as dist
+
+    pg = moodist_amd.LocalWorld(2, 0).groups[0]
+    with pytest.raises(RuntimeError, match="all_gather input is a CPU tensor"):
+        dist.all_gather_into_tensor(torch.zeros(4), torch.zeros(2), group=pg)
+    with pytest.raises(RuntimeError, match="reduce_scatter input is a CPU tensor"):
+        dist.reduce_scatter_tensor(torch.zeros(2), torch.zeros(4), group=pg)
+    with pytest.raises(RuntimeError, match="allreduce tensor is a CPU tensor"):
+        dist.all_reduce(torch.zeros(4), group=pg)
 
 
 def test_reference_constructor_joins_ranks_through_the_store():
@@ -402,14 +419,23 @@ def test_reference_constructor_joins_ranks_through_the_store():
     store = dist.HashStore()
     pgs = [moodist_amd.MoodistProcessGroup(store, r, 4) for r in range(4)]
     assert [pg.rank() for pg in pgs] == [0, 1, 2, 3] and all(pg.size() == 4 for pg in pgs)
-    assert len({id(pg.world) for pg in pgs}) == 1
-    assert moodist_amd.MoodistProcessGroup(store, 2, 4) is pgs[2]
+    assert all(pg._store is store for pg in pgs)
+    with pytest.raises(RuntimeError, match="rank 2 of this store's group already exists"):
+        moodist_amd.MoodistProcessGroup(store, 2, 4)
     other = moodist_amd.MoodistProcessGroup(dist.HashStore(), 0, 4)
-    assert other.world is not pgs[0].world
-    with pytest.raises(ValueError, match="already serves a group of 4 ranks"):
+    assert other._store is not store
+    with pytest.raises(RuntimeError, match="already serves a group of 4 ranks"):
         moodist_amd.MoodistProcessGroup(store, 0, 8)
-    with pytest.raises(ValueError, match="outside a group"):
+    with pytest.raises(RuntimeError, match="outside a group"):
         moodist_amd.MoodistProcessGroup(store, 4, 4)
+    # a rank that has gone can be made again; a store whose ranks have all gone serves a new group
+    del pgs[2]
+    pgs.insert(2, moodist_amd.MoodistProcessGroup(store, 2, 4))
+    assert pgs[2].rank() == 2
+    del pgs, other
+    again = moodist_amd.MoodistProcessGroup(store, 0, 8)
+    assert again.size() == 8
+    pgs = [moodist_amd.MoodistProcessGroup(dist.HashStore(), 0, 4)]
     # prefer_kernel_less as setter and as context manager (py/moodist/backend.py:17-43)
     pg = pgs[0]
     pg.prefer_kernel_less(True)

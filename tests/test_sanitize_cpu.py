@@ -13,7 +13,7 @@ import pytest
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CORE = os.path.join(ROOT, "moodist_amd", "csrc", "core")
-FLAGS = ["-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined",
+FLAGS = ["-std=c++20", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined",
          "-I" + CORE, "-I" + os.path.join(ROOT, "include")]
 
 
@@ -36,3 +36,27 @@ def test_c_api_handle_lifetimes_under_sanitizers(tmp_path):
     r = build_and_run(tmp_path, "c_api_driver.cc", ["planner.cc", "processgroup.cc", "c_api.cc", "hip_loader.cc"])
     assert r.returncode == 0, r.stderr[-3000:]
     assert "c api driver done" in r.stdout
+
+
+def test_plugin_entry_and_reference_lifetimes_under_sanitizers(tmp_path):
+    # moodistGetApi -> CoreApi table with a fake WrapperApi: handshake, off-path slots, handle
+    # ownership, and tensor references held from a rank's post until the collective's launch
+    r = build_and_run(tmp_path, "plugin_driver.cc",
+                      ["planner.cc", "processgroup.cc", "c_api.cc", "hip_loader.cc", "plugin.cc"])
+    assert r.returncode == 0, (r.stdout[-2000:], r.stderr[-3000:])
+    assert "plugin driver done" in r.stdout
+
+
+@pytest.mark.skipif(os.path.exists("/dev/kfd"), reason="the driver's tensors are fake addresses: on a machine with a "
+                    "GPU the launch it provokes would really run and fault")
+def test_plugin_entry_of_the_built_library_through_dlsym(tmp_path):
+    # the same walk against the shipped libmoodist.so: dlopen + dlsym("moodistGetApi"), the
+    # driver's own destroy() going back through the table
+    lib = os.path.join(ROOT, "moodist_amd", "libmoodist.so")
+    exe = str(tmp_path / "driver")
+    subprocess.run(["g++", "-std=c++20", "-O1", "-g", "-DMOODIST_DRIVER_DLOPEN", "-I" + os.path.join(ROOT, "include"),
+                    os.path.join(HERE, "sanitize", "plugin_driver.cc"), "-ldl", "-o", exe],
+                   check=True, capture_output=True, text=True)
+    r = subprocess.run([exe, lib], cwd=str(tmp_path), capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, (r.stdout[-2000:], r.stderr[-3000:])
+    assert "plugin driver done" in r.stdout
