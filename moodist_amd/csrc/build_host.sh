@@ -17,7 +17,10 @@ for f in hip_loader planner processgroup c_api plugin; do
   objs+=("$o")
 done
 wait
-"$cxx" -shared -o "$pkg/libmoodist.so" "${objs[@]}" -ldl -lpthread -Wl,--no-undefined
+# exports: the plugin entry and the plain C functions, nothing else (no C++ symbols leak out)
+printf '{ global: moodist*; local: *; };\n' > "$here/build/exports.map"
+"$cxx" -shared -o "$pkg/libmoodist.so" "${objs[@]}" -ldl -lpthread -Wl,--no-undefined \
+  -Wl,--version-script="$here/build/exports.map"
 echo "built $pkg/libmoodist.so"
 if [ "${MOODIST_SKIP_WRAPPER:-0}" != "1" ] && [ -f "$here/wrapper/module.cc" ]; then
   python3 "$here/wrapper/build_wrapper.py"

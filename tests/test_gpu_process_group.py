@@ -357,3 +357,134 @@ def test_stress_large_tensors(world, dev):
         each_rank(world, lambda r, pg: pg._allgather_base(outs[r], ins[r]))
     for q in range(P):
         assert torch.equal(outs[q], torch.arange(P, device=dev).float().repeat_interleave(chunk))
+
+
+# ---- through the plugin entry: the core's table, torch.distributed's own functions, lifetimes ----
+
+
+def test_reduce_scatter_through_the_core_api_table_matches_the_oracle(world, dev):
+    # _C resolves one symbol, moodistGetApi, and calls processGroupReduceScatter through the table it
+    # returns (reference: wrapper/moodist_loader.cc:363-386, wrapper/processgroup_wrapper.cc:150-157);
+    # here via torch.distributed's own function with the group passed as group=
+    from moodist_amd import _C
+
+    assert _C.core_api_info()["entry"] == "moodistGetApi"
+    n = 40000 + 3  # ragged: not a multiple of 16 bytes
+    srcs = random_sources(P, P * n, torch.float32, seed=11)
+    ins = [s.to(dev) for s in srcs]
+    outs = [torch.zeros(n, device=dev) for _ in range(P)]
+    # async_op=True: the blocking form waits on the work at once, which a single thread playing
+    # every rank cannot do before the other ranks have called
+    works = []
+    for r, pg in enumerate(world):
+        assert isinstance(pg, dist.ProcessGroup)
+        works.append(dist.reduce_scatter_tensor(outs[r], ins[r], group=pg, async_op=True))
+    for w in works:
+        w.wait()
+    torch.cuda.synchronize()
+    for r in range(P):
+        chunks = [bits(s[r * n:(r + 1) * n]) for s in srcs]
+        assert same_bits(bits(outs[r]), oracle.reduce(chunks, r, oracle.DT_F32, oracle.OP_SUM))
+
+
+def test_all_gather_and_all_reduce_through_torch_distributed(world, dev):
+    n = 1000
+    ins = [torch.arange(r * n, (r + 1) * n, device=dev, dtype=torch.float32) for r in range(P)]
+    outs = [torch.zeros(P * n, device=dev) for _ in range(P)]
+    works = [dist.all_gather_into_tensor(outs[r], ins[r], group=pg, async_op=True) for r, pg in enumerate(world)]
+    ts = [torch.full((P * 13 + 5,), float(r + 1), device=dev) for r in range(P)]  # needs the padded temporary
+    works += [dist.all_reduce(ts[r], group=pg, async_op=True) for r, pg in enumerate(world)]
+    for w in works:
+        w.wait()
+    torch.cuda.synchronize()
+    for r in range(P):
+        assert torch.equal(outs[r], torch.arange(P * n, device=dev, dtype=torch.float32))
+        assert torch.equal(ts[r], torch.full((P * 13 + 5,), P * (P + 1) / 2, device=dev))
+
+
+def test_posted_tensors_outlive_their_python_references(world, dev):
+    # A rank posts and drops every reference to its tensors; many other allocations follow before
+    # the peers arrive.  The core holds the posted tensors until the launch (the reference ties
+    # their lifetime to the operation, core/processgroup.cc:3239-3245), so the caching allocator
+    # cannot hand their memory out in between.
+    n = 1 << 16
+    srcs = random_sources(P, P * n, torch.float32, seed=5)
+    outs = [torch.zeros(n, device=dev) for _ in range(P)]
+
+    def post_and_forget(r):
+        t = srcs[r].to(dev)
+        world.groups[r]._reduce_scatter_base(outs[r], t)
+
+    post_and_forget(0)
+    torch.cuda.synchronize()
+    churn = [torch.full((P * n,), 7.0, device=dev) for _ in range(100)]  # would reuse a freed input's block
+    del churn
+    for r in range(1, P):
+        post_and_forget(r)
+    torch.cuda.synchronize()
+    for r in range(P):
+        chunks = [bits(s[r * n:(r + 1) * n]) for s in srcs]
+        assert same_bits(bits(outs[r]), oracle.reduce(chunks, r, oracle.DT_F32, oracle.OP_SUM))
+
+
+def test_allreduce_coalesced_many_tensors_of_awkward_sizes(world, dev):
+    # 48 tensors none of whose sizes divides by the group size: every one goes through a padded
+    # temporary that must live until the LAST rank has made its call
+    sizes = [P * k + 1 + (k % (P - 1)) for k in range(1, 49)]
+    assert all(s % P for s in sizes)
+    per_rank = [[torch.full((s,), float(r + 1) + 0.25 * i, device=dev) for i, s in enumerate(sizes)] for r in range(P)]
+    works = [pg.allreduce_coalesced(per_rank[r]) for r, pg in enumerate(world)]
+    for w in works:
+        w.wait()
+    torch.cuda.synchronize()
+    for r in range(P):
+        for i, s in enumerate(sizes):
+            want = sum(float(q + 1) + 0.25 * i for q in range(P))
+            assert torch.equal(per_rank[r][i], torch.full((s,), want, device=dev)), (r, i)
+
+
+def test_input_changed_between_a_ranks_call_and_the_launch(world, dev):
+    # The collective is launched when the last rank calls, on stream order at THAT moment: what a
+    # rank does to its input after its own call but before the last rank's call is seen by the
+    # collective (c10d and the reference see the value at call time).  snapshot_inputs copies
+    # every posted input at the call's position in the stream and restores c10d's meaning.
+    n = 4096
+    for snapshot in (False, True):
+        for pg in world:
+            pg.options().snapshot_inputs = snapshot
+        ins = [torch.full((P * n,), float(r + 1), device=dev) for r in range(P)]
+        outs = [torch.zeros(n, device=dev) for _ in range(P)]
+        works = []
+        for r, pg in enumerate(world):
+            works.append(pg._reduce_scatter_base(outs[r], ins[r]))
+            if r == 0:
+                ins[0].fill_(100.0)  # after rank 0's call, before the launch
+        for w in works:
+            w.wait()
+        torch.cuda.synchronize()
+        first = 1.0 if snapshot else 100.0
+        want = first + sum(float(q + 1) for q in range(1, P))
+        for r in range(P):
+            assert torch.equal(outs[r], torch.full((n,), want, device=dev)), (snapshot, r)
+    for pg in world:
+        pg.options().snapshot_inputs = False
+
+
+def test_snapshot_inputs_with_allreduce_and_allgather(world, dev):
+    for pg in world:
+        pg.options().snapshot_inputs = True
+    n = 999  # not divisible: padded temporary
+    ts = [torch.full((n,), float(r + 1), device=dev) for r in range(P)]
+    ev = [torch.full((P * 64,), float(r + 1), device=dev) for r in range(P)]
+    ins = [torch.full((100,), float(r), device=dev) for r in range(P)]
+    outs = [torch.zeros(P * 100, device=dev) for _ in range(P)]
+    for r, pg in enumerate(world):
+        pg.allreduce([ts[r]])
+        pg.allreduce([ev[r]])
+        pg._allgather_base(outs[r], ins[r])
+        ins[r].fill_(-1.0)  # after the call: must not be seen
+    torch.cuda.synchronize()
+    for r in range(P):
+        assert torch.equal(ts[r], torch.full((n,), P * (P + 1) / 2, device=dev))
+        assert torch.equal(ev[r], torch.full((P * 64,), P * (P + 1) / 2, device=dev))
+        assert torch.equal(outs[r], torch.arange(P, device=dev, dtype=torch.float32).repeat_interleave(100))
