@@ -77,8 +77,10 @@ int moodist_pg_rank(moodist_pg* pg);
 int moodist_pg_size(moodist_pg* pg);
 /* processGroupGetOption / processGroupSetOption (api/processgroup_api.h:39-40).
  * Names as in the reference (core/processgroup.cc:2455-2488): prefer_kernel_less,
- * force_kernel_less, num_chunks, chunk_size, method; and snapshot_inputs (not in the
- * reference; needs a core loaded through moodistGetApi).  Unknown name -> error. */
+ * force_kernel_less, num_chunks, chunk_size, method; and, not in the reference,
+ * snapshot_inputs (needs a core loaded through moodistGetApi) and the read-only counters
+ * kernel_less_copies_1d / kernel_less_copies_2d (copy-engine calls the world's kernel-less
+ * all_gathers have made).  Unknown name -> error. */
 int moodist_pg_get_option(moodist_pg* pg, const char* name, int64_t* value);
 int moodist_pg_set_option(moodist_pg* pg, const char* name, int64_t value);
 
@@ -139,6 +141,15 @@ int moodist_op_call(moodist_op* op, const moodist_tensor* inputs, size_t n_input
 /* futureWait (api/moodist_api.h:253-255; core/processgroup.cc:2650-2661) */
 int moodist_future_wait(moodist_future* future, void* stream);
 void moodist_future_destroy(moodist_future* future);
+
+/* How the kernel-less all_gather would group `n` source buffers of `bytes` bytes each into
+ * copy-engine calls: ranks whose buffers are evenly spaced form one run, as the reference
+ * groups the sources a peer holds into Copy2d{offset, length, pitch, num}
+ * (core/processgroup.cc:114-119, :618-704).  Writes first, count, src_pitch per run into out
+ * (3 values each, as far as capacity allows) and returns the number of runs.  A rank whose
+ * source is dst + rank*bytes is in place and belongs to no run (dst may be NULL). */
+int64_t moodist_kernel_less_runs(const void* const* srcs, size_t n, size_t bytes, const void* dst, int64_t* out,
+    size_t capacity);
 
 /* The plan of the calling rank, as the reference's CustomOpDescriptor holds it
  * (core/cputhread.h:296-322), for inspection.  what: 0 reads, 1 inputCopies, 2 outputCopies,

@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define MDH_ABI_VERSION 1
+#define MDH_ABI_VERSION 2
 
 /* error codes */
 #define MDH_OK 0
@@ -148,6 +148,32 @@ typedef struct mdh_box {
  * buffer exists.  Destination boxes must not overlap each other or any source.
  */
 int mdh_copy_boxes(const mdh_box* boxes, int nboxes, int itemsize, void* stream);
+
+/*
+ * The same copies, prepared once and replayed: what a compiled custom op runs on every call.
+ *
+ * Replaces: the split the reference makes between compileOpFull, which computes the reads and
+ * copies of an op once (core/processgroup.cc:2761-3104), and customOp, which on every call only
+ * checks sizes and enqueues them (core/processgroup.cc:3172-3256).  Here everything about the
+ * launches except the tensors' addresses is decided at create time -- boxes merged and split,
+ * vector widths, tiles, grids, the kernels' argument blocks -- and a launch patches addresses
+ * into a copy of those blocks and enqueues the kernels.
+ *
+ * create: boxes[i].src / boxes[i].dst hold BYTE OFFSETS from base number src_slots[i] /
+ * dst_slots[i] of a table of `nbases` base addresses that is supplied at launch (a custom op's
+ * input and output tensors).  Shapes and strides as in mdh_copy_boxes.  Needs no device.
+ * launch: bases[] are device addresses; the result is that of mdh_copy_boxes on the boxes with
+ * the offsets added to the bases.  Plans are prepared for 16-byte aligned bases (torch
+ * allocations are); a table with a less aligned base is served through mdh_copy_boxes.
+ * A plan is immutable after create: launches of one plan may run concurrently.
+ * launches: how many kernels one launch of the plan enqueues (-1 for NULL).
+ */
+typedef struct mdh_copy_plan mdh_copy_plan;
+int mdh_copy_plan_create(const mdh_box* boxes, const int32_t* src_slots, const int32_t* dst_slots, int nboxes,
+    int itemsize, int nbases, mdh_copy_plan** plan);
+int mdh_copy_plan_launch(const mdh_copy_plan* plan, const void* const* bases, int nbases, void* stream);
+int mdh_copy_plan_launches(const mdh_copy_plan* plan);
+void mdh_copy_plan_destroy(mdh_copy_plan* plan);
 
 /*
  * Launch-shape knobs, for measurement; 0 (the default) lets the library choose

@@ -16,11 +16,12 @@ DTYPE_INT32, DTYPE_INT64, DTYPE_FLOAT16, DTYPE_FLOAT32, DTYPE_FLOAT64, DTYPE_BFL
 OP_SUM, OP_AVG, OP_MIN, OP_MAX, OP_PREMUL_SUM = 0, 1, 3, 4, 8
 MAX_SOURCES = 64
 MAX_DIMS = 10
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 SYMBOLS = (
     "mdh_abi_version", "mdh_error_string", "mdh_last_error", "mdh_reduce", "mdh_gather", "mdh_copy_boxes",
-    "mdh_set_tuning", "mdh_get_tuning",
+    "mdh_set_tuning", "mdh_get_tuning", "mdh_copy_plan_create", "mdh_copy_plan_launch", "mdh_copy_plan_launches",
+    "mdh_copy_plan_destroy",
 )
 
 
@@ -65,6 +66,15 @@ def lib():
     L.mdh_gather.restype = ctypes.c_int
     L.mdh_copy_boxes.argtypes = [ctypes.POINTER(Box), ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
     L.mdh_copy_boxes.restype = ctypes.c_int
+    L.mdh_copy_plan_create.argtypes = [ctypes.POINTER(Box), ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32),
+                                       ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_void_p)]
+    L.mdh_copy_plan_create.restype = ctypes.c_int
+    L.mdh_copy_plan_launch.argtypes = [ctypes.c_void_p, vpp, ctypes.c_int, ctypes.c_void_p]
+    L.mdh_copy_plan_launch.restype = ctypes.c_int
+    L.mdh_copy_plan_launches.argtypes = [ctypes.c_void_p]
+    L.mdh_copy_plan_launches.restype = ctypes.c_int
+    L.mdh_copy_plan_destroy.argtypes = [ctypes.c_void_p]
+    L.mdh_copy_plan_destroy.restype = None
     L.mdh_set_tuning.argtypes = [ctypes.c_char_p, ctypes.c_int]
     L.mdh_set_tuning.restype = ctypes.c_int
     L.mdh_get_tuning.argtypes = [ctypes.c_char_p, ctypes.POINTER(ctypes.c_int)]
@@ -109,6 +119,32 @@ def make_box(src_ptr, dst_ptr, shape, src_strides, dst_strides):
 def copy_boxes(boxes, itemsize, stream=0):
     arr = (Box * max(len(boxes), 1))(*boxes)
     check(lib().mdh_copy_boxes(arr, len(boxes), itemsize, stream))
+
+
+class CopyPlan:
+    """A prepared set of box copies (mdh_copy_plan): `boxes` carry byte offsets in src/dst, relative to
+    bases[src_slots[i]] / bases[dst_slots[i]] of the table given to launch()."""
+
+    def __init__(self, boxes, src_slots, dst_slots, itemsize, nbases):
+        n = len(boxes)
+        arr = (Box * max(n, 1))(*boxes)
+        ss = (ctypes.c_int32 * max(n, 1))(*src_slots)
+        ds = (ctypes.c_int32 * max(n, 1))(*dst_slots)
+        self._plan = ctypes.c_void_p()
+        self.nbases = nbases
+        check(lib().mdh_copy_plan_create(arr, ss, ds, n, itemsize, nbases, ctypes.byref(self._plan)))
+
+    def launch(self, bases, stream=0):
+        check(lib().mdh_copy_plan_launch(self._plan, ptr_table(bases), len(bases), stream))
+
+    @property
+    def launches(self):
+        return lib().mdh_copy_plan_launches(self._plan)
+
+    def __del__(self):
+        if getattr(self, "_plan", None):
+            lib().mdh_copy_plan_destroy(self._plan)
+            self._plan = None
 
 
 def set_tuning(name, value):

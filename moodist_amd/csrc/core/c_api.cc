@@ -253,6 +253,23 @@ void moodist_future_destroy(moodist_future* future) {
   delete future;
 }
 
+int64_t moodist_kernel_less_runs(const void* const* srcs, size_t n, size_t bytes, const void* dst, int64_t* out,
+    size_t capacity) {
+  if (!srcs && n) {
+    return -1;
+  }
+  std::vector<const void*> s(srcs, srcs + n);
+  std::vector<bool> in_place(n, false);
+  for (size_t j = 0; dst && j < n; ++j) {
+    in_place[j] = (const char*)dst + bytes * j == s[j];
+  }
+  const std::vector<GatherRun> runs = gather_runs(s, in_place, bytes);
+  for (size_t i = 0; i < runs.size() && out && 3 * i + 2 < capacity; ++i) {
+    out[3 * i] = (int64_t)runs[i].first, out[3 * i + 1] = (int64_t)runs[i].count, out[3 * i + 2] = (int64_t)runs[i].src_pitch;
+  }
+  return (int64_t)runs.size();
+}
+
 int64_t moodist_op_plan_count(moodist_op* op, int what) {
   if (!op) {
     return -1;

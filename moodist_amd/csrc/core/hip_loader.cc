@@ -79,6 +79,9 @@ HipRuntime load() {
   resolve(kl, kn, "mdh_reduce", r.reduce);
   resolve(kl, kn, "mdh_gather", r.gather);
   resolve(kl, kn, "mdh_copy_boxes", r.copy_boxes);
+  resolve(kl, kn, "mdh_copy_plan_create", r.copy_plan_create);
+  resolve(kl, kn, "mdh_copy_plan_launch", r.copy_plan_launch);
+  resolve(kl, kn, "mdh_copy_plan_destroy", r.copy_plan_destroy);
   if (r.abi_version() != MDH_ABI_VERSION) {
     throw std::runtime_error("moodist: libmoodist_hip.so has ABI version " + std::to_string(r.abi_version()) +
                              ", this core expects " + std::to_string(MDH_ABI_VERSION));

@@ -39,6 +39,9 @@ struct HipRuntime {
   decltype(&mdh_reduce) reduce;
   decltype(&mdh_gather) gather;
   decltype(&mdh_copy_boxes) copy_boxes;
+  decltype(&mdh_copy_plan_create) copy_plan_create;
+  decltype(&mdh_copy_plan_launch) copy_plan_launch;
+  decltype(&mdh_copy_plan_destroy) copy_plan_destroy;
 };
 
 constexpr int kHipMemcpyDeviceToDevice = 3;

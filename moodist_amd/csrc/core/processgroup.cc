@@ -154,6 +154,10 @@ int64_t ProcessGroup::get_option(const std::string& name) const {
     return options.method;
   } else if (name == "snapshot_inputs") {
     return options.snapshotInputs ? 1 : 0;
+  } else if (name == "kernel_less_copies_1d") { // read-only counters of the world
+    return (int64_t)world->kernel_less_copies_1d;
+  } else if (name == "kernel_less_copies_2d") {
+    return (int64_t)world->kernel_less_copies_2d;
   }
   throw std::runtime_error("Unknown option: " + name);
 }
@@ -410,6 +414,96 @@ std::shared_ptr<Collective> ProcessGroup::custom_op(const std::shared_ptr<Compil
   return last = world->post(Kind::custom, next_seq++, rank, std::move(p), 0, 1.0f, 0, op->dtype, op->id, op);
 }
 
+// ---------------------------------------------------------------- kernel-less runs
+
+std::vector<GatherRun> gather_runs(const std::vector<const void*>& srcs, const std::vector<bool>& in_place,
+    size_t bytes) {
+  std::vector<GatherRun> runs;
+  const size_t n = srcs.size();
+  // a 2-D copy's pitches are kept inside 31 bits; anything sparser goes rank by rank
+  const uintptr_t max_pitch = 0x7fffffffu;
+  size_t i = 0;
+  while (i < n) {
+    if (in_place[i]) {
+      ++i;
+      continue;
+    }
+    GatherRun run{i, 1, bytes};
+    if (i + 1 < n && !in_place[i + 1]) {
+      const uintptr_t a = (uintptr_t)srcs[i], b = (uintptr_t)srcs[i + 1];
+      if (b > a && b - a >= bytes && b - a <= max_pitch) {
+        const uintptr_t pitch = b - a;
+        size_t k = i + 1;
+        while (k + 1 < n && !in_place[k + 1] && (uintptr_t)srcs[k + 1] > (uintptr_t)srcs[k] &&
+               (uintptr_t)srcs[k + 1] - (uintptr_t)srcs[k] == pitch) {
+          ++k;
+        }
+        run.count = k - i + 1;
+        run.src_pitch = (size_t)pitch;
+      }
+    }
+    runs.push_back(run);
+    i += run.count;
+  }
+  return runs;
+}
+
+// ---------------------------------------------------------------- prepared transfers
+
+PreparedTransfers::~PreparedTransfers() {
+  if (plan) {
+    hip().copy_plan_destroy(plan);
+  }
+}
+
+namespace {
+
+std::unique_ptr<PreparedTransfers> prepare_transfers(const RankPlan& plan, size_t itemsize) {
+  auto pt = std::make_unique<PreparedTransfers>();
+  pt->n_outputs = plan.outputs.size();
+  std::vector<mdh_box> boxes(plan.transfers.size());
+  std::vector<int32_t> src_slots(plan.transfers.size()), dst_slots(plan.transfers.size());
+  for (size_t i = 0; i < plan.transfers.size(); ++i) {
+    const Transfer& t = plan.transfers[i];
+    size_t slot = 0;
+    for (; slot < pt->sources.size(); ++slot) {
+      if (pt->sources[slot].rank == t.srcRank && pt->sources[slot].input == t.srcInput) {
+        break;
+      }
+    }
+    if (slot == pt->sources.size()) {
+      pt->sources.push_back({t.srcRank, t.srcInput});
+    }
+    src_slots[i] = (int32_t)slot;
+    MD_CHECK(t.dstOutput < pt->n_outputs);
+    mdh_box& b = boxes[i];
+    const size_t nd = t.shape.size();
+    b.ndim = (int32_t)nd;
+    b.reserved = 0;
+    int64_t ss = 1, ds = 1;
+    for (size_t d = nd; d-- > 0;) {
+      b.shape[d] = t.shape[d];
+      b.src_strides[d] = ss;
+      b.dst_strides[d] = ds;
+      ss *= t.srcShape[d];
+      ds *= t.dstShape[d];
+    }
+    // byte offsets from the tensors' first bytes; the addresses come with each call
+    b.src = (const void*)(uintptr_t)(linear_offset(t.srcOffset, t.srcShape) * itemsize);
+    b.dst = (void*)(uintptr_t)(linear_offset(t.dstOffset, t.dstShape) * itemsize);
+  }
+  for (size_t i = 0; i < plan.transfers.size(); ++i) {
+    dst_slots[i] = (int32_t)(pt->sources.size() + plan.transfers[i].dstOutput);
+  }
+  const int nbases = (int)(pt->sources.size() + pt->n_outputs);
+  check_mdh(hip().copy_plan_create(boxes.data(), src_slots.data(), dst_slots.data(), (int)boxes.size(), (int)itemsize,
+      nbases, &pt->plan));
+  pt->bases.assign((size_t)nbases, nullptr);
+  return pt;
+}
+
+} // namespace
+
 // ---------------------------------------------------------------- World
 
 World::World(int size, int device) : size(size), device(device) {
@@ -614,12 +708,25 @@ void World::launch(Collective& c, const std::shared_ptr<CompiledOp>& op) {
           }
         }
       } else if (pq.kernel_less) {
-        // copy-engine form (core/processgroup.cc:706-833): one device-to-device copy per shard
+        // copy-engine form (core/processgroup.cc:706-833): ranks whose buffers are evenly spaced
+        // -- slices of one staging allocation, with or without padding between them -- move as
+        // one copy: 1-D when they are adjacent, 2-D (hipMemcpy2DAsync, the reference's
+        // cuMemcpy2DAsync :806-820) when there is a pitch; the others one copy per rank
+        std::vector<bool> in_place((size_t)size);
         for (int j = 0; j < size; ++j) {
-          void* dst = (char*)pq.output.data + c.bytes * (size_t)j;
-          if (dst != srcs[(size_t)j]) {
-            check_hip(h.MemcpyAsync(dst, srcs[(size_t)j], c.bytes, kHipMemcpyDeviceToDevice, pq.stream),
+          in_place[(size_t)j] = (char*)pq.output.data + c.bytes * (size_t)j == srcs[(size_t)j];
+        }
+        for (const GatherRun& run : gather_runs(srcs, in_place, c.bytes)) {
+          void* dst = (char*)pq.output.data + c.bytes * run.first;
+          if (run.count == 1 || run.src_pitch == c.bytes) {
+            check_hip(h.MemcpyAsync(dst, srcs[run.first], c.bytes * run.count, kHipMemcpyDeviceToDevice, pq.stream),
                 "hipMemcpyAsync");
+            ++kernel_less_copies_1d;
+          } else {
+            check_hip(h.Memcpy2DAsync(dst, c.bytes, srcs[run.first], run.src_pitch, c.bytes, run.count,
+                          kHipMemcpyDeviceToDevice, pq.stream),
+                "hipMemcpy2DAsync");
+            ++kernel_less_copies_2d;
           }
         }
       } else {
@@ -635,35 +742,34 @@ void World::launch(Collective& c, const std::shared_ptr<CompiledOp>& op) {
     }
   } else {
     // Every read of every rank, with its staging copies folded in, as strided box copies
-    // straight from the source rank's tensor into the destination tensor.
+    // straight from the source rank's tensor into the destination tensor.  The launches were
+    // prepared when the op first ran (box geometry, tiles, grids, kernel arguments): a call
+    // fills in the tensors' addresses and enqueues them.
     MD_CHECK(op != nullptr);
+    if (op->prepared.size() != (size_t)size) {
+      op->prepared.resize((size_t)size);
+    }
     for (int q = 0; q < size; ++q) {
       const Posting& pq = c.post[(size_t)q];
       const RankPlan& plan = op->plans[(size_t)q];
       if (plan.transfers.empty()) {
         continue;
       }
-      std::vector<mdh_box> boxes(plan.transfers.size());
-      for (size_t i = 0; i < plan.transfers.size(); ++i) {
-        const Transfer& t = plan.transfers[i];
-        const Posting& ps = c.post[t.srcRank];
-        MD_CHECK(t.srcInput < ps.inputs.size() && t.dstOutput < pq.outputs.size());
-        mdh_box& b = boxes[i];
-        const size_t nd = t.shape.size();
-        b.ndim = (int32_t)nd;
-        b.reserved = 0;
-        int64_t ss = 1, ds = 1;
-        for (size_t d = nd; d-- > 0;) {
-          b.shape[d] = t.shape[d];
-          b.src_strides[d] = ss;
-          b.dst_strides[d] = ds;
-          ss *= t.srcShape[d];
-          ds *= t.dstShape[d];
-        }
-        b.src = (const char*)ps.inputs[t.srcInput].data + linear_offset(t.srcOffset, t.srcShape) * op->itemsize;
-        b.dst = (char*)pq.outputs[t.dstOutput].data + linear_offset(t.dstOffset, t.dstShape) * op->itemsize;
+      if (!op->prepared[(size_t)q]) {
+        op->prepared[(size_t)q] = prepare_transfers(plan, op->itemsize);
       }
-      check_mdh(h.copy_boxes(boxes.data(), (int)boxes.size(), (int)op->itemsize, pq.stream));
+      PreparedTransfers& pt = *op->prepared[(size_t)q];
+      MD_CHECK(pt.n_outputs == pq.outputs.size());
+      size_t k = 0;
+      for (const PreparedTransfers::Source& src : pt.sources) {
+        const Posting& ps = c.post[src.rank];
+        MD_CHECK(src.input < ps.inputs.size());
+        pt.bases[k++] = ps.inputs[src.input].data;
+      }
+      for (const moodist_tensor& o : pq.outputs) {
+        pt.bases[k++] = o.data;
+      }
+      check_mdh(h.copy_plan_launch(pt.plan, pt.bases.data(), (int)pt.bases.size(), pq.stream));
     }
   }
   order_streams_after(c);

@@ -15,6 +15,7 @@
 #include <vector>
 
 #include "moodist_core.h"
+#include "moodist_hip.h"
 #include "planner.h"
 
 namespace moodist {
@@ -75,6 +76,20 @@ struct Options { // core/processgroup.cc:334-340
   bool snapshotInputs = false;
 };
 
+// A rank's transfers as the kernel library has prepared them (mdh_copy_plan): made at the op's
+// first launch, replayed by every later one with only the tensors' addresses filled in.
+struct PreparedTransfers {
+  mdh_copy_plan* plan = nullptr;
+  // base table of the plan: first the source tensors in order of first use, then this rank's outputs
+  struct Source {
+    uint32_t rank, input;
+  };
+  std::vector<Source> sources;
+  size_t n_outputs = 0;
+  std::vector<const void*> bases; // scratch for a launch (launches are serialized by the world's mutex)
+  ~PreparedTransfers();
+};
+
 struct CompiledOp {
   uint32_t id;
   int dtype;
@@ -82,6 +97,7 @@ struct CompiledOp {
   std::vector<RankPlan> plans; // every rank's, computed identically by every rank
   PlanWire wire;               // wire[sender][receiver]
   size_t ndim = 0;
+  std::vector<std::unique_ptr<PreparedTransfers>> prepared; // per rank, filled at the first launch
 };
 
 class ProcessGroup {
@@ -152,6 +168,8 @@ public:
   const int size;
   const int device;
   DeviceAllocator allocator; // empty unless the loader supplied one
+  // how many copy-engine calls the kernel-less all_gathers of this world have made so far
+  uint64_t kernel_less_copies_1d = 0, kernel_less_copies_2d = 0;
 
 private:
   void launch(Collective& c, const std::shared_ptr<CompiledOp>& op);
@@ -165,5 +183,19 @@ private:
 };
 
 size_t dtype_size(int dtype);
+
+// The copy-engine form of all_gather groups source ranks whose buffers are evenly spaced into
+// one 2-D copy, as the reference groups the sources a peer holds into Copy2d{offset, length,
+// pitch, num} runs for cuMemcpy2DAsync (core/processgroup.cc:114-119, :618-704, :806-820).
+// A run is ranks first .. first+count-1 whose source addresses advance by src_pitch bytes
+// (>= bytes); count == 1 is a plain 1-D copy.  Ranks whose source already is its place in the
+// destination (in_place[j]) belong to no run.
+struct GatherRun {
+  size_t first;
+  size_t count;
+  size_t src_pitch;
+};
+std::vector<GatherRun> gather_runs(const std::vector<const void*>& srcs, const std::vector<bool>& in_place,
+    size_t bytes);
 
 } // namespace moodist

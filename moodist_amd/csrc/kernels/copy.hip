@@ -14,6 +14,7 @@
 #include "device_common.h"
 
 #include <algorithm>
+#include <memory>
 #include <vector>
 
 namespace mdh {
@@ -281,8 +282,23 @@ int vec_width(const HostBox& h) {
   return (int)(bits & (~bits + 1)); // lowest set bit: 1, 2, 4, 8 or 16
 }
 
+// One kernel launch of a copy, with everything but the base addresses decided: what a
+// prepared plan replays.
+struct Step {
+  enum Kind { kFlat, kBoxes16, kBoxes } kind;
+  int vec;    // kBoxes: bytes per vector
+  int unroll; // sub-tiles
+  uint32_t grid;
+  size_t lds;
+  FlatArgs flat;   // kFlat
+  CopyArgs boxes;  // kBoxes16, kBoxes
+};
+
+int launch_step(const Step& st, const FlatArgs* flat, const CopyArgs* boxes, hipStream_t stream);
+
 struct Launcher {
   hipStream_t stream;
+  std::vector<Step>* record = nullptr; // when set, launches are recorded here instead of enqueued
   std::vector<BoxDesc> pending[5]; // by log2(VEC)
   std::vector<BoxDesc> pending16;  // 16-byte vectors, spans inside 32 bits: copy_boxes16_kernel
   struct Segment {
@@ -357,31 +373,31 @@ struct Launcher {
       if (t.copy_max_blocks > 0 && grid > (uint32_t)t.copy_max_blocks) {
         grid = (uint32_t)t.copy_max_blocks;
       }
-      dim3 g(grid), b(kBlock);
-      switch (U) {
-      case 1:
-        hipLaunchKernelGGL((copy_flat_kernel<1>), g, b, lds, stream, a);
-        break;
-      case 2:
-        hipLaunchKernelGGL((copy_flat_kernel<2>), g, b, lds, stream, a);
-        break;
-      case 4:
-        hipLaunchKernelGGL((copy_flat_kernel<4>), g, b, lds, stream, a);
-        break;
-      default:
-        hipLaunchKernelGGL((copy_flat_kernel<8>), g, b, lds, stream, a);
-        break;
-      }
-      int r = check_launch("copy_flat_kernel");
-      if (r != MDH_OK) {
-        rc = r;
-      }
+      Step st;
+      st.kind = Step::kFlat, st.vec = 16, st.unroll = U, st.grid = grid, st.lds = lds;
+      submit(st, &a, nullptr);
     }
     flat.clear();
   }
 
-  template<int VEC>
-  void launch(CopyArgs& a) {
+  // Enqueues the step now, or files it for a plan.
+  void submit(Step& st, const FlatArgs* f, const CopyArgs* c) {
+    if (record) {
+      if (f) {
+        st.flat = *f;
+      } else {
+        st.boxes = *c;
+      }
+      record->push_back(st);
+      return;
+    }
+    const int r = launch_step(st, f, c, stream);
+    if (r != MDH_OK) {
+      rc = r;
+    }
+  }
+
+  void launch_boxes(CopyArgs& a, int vec, bool buffer16) {
     const Tuning& t = tuning();
     uint32_t grid = a.total_tiles;
     if (t.copy_max_blocks > 0 && grid > (uint32_t)t.copy_max_blocks) {
@@ -390,52 +406,10 @@ struct Launcher {
     if (grid > 0x7fffffffu) {
       grid = 0x7fffffffu;
     }
-    dim3 g(grid), b(kBlock);
-    switch (unroll) {
-    case 1:
-      hipLaunchKernelGGL((copy_boxes_kernel<VEC, 1>), g, b, 0, stream, a);
-      break;
-    case 2:
-      hipLaunchKernelGGL((copy_boxes_kernel<VEC, 2>), g, b, 0, stream, a);
-      break;
-    case 4:
-      hipLaunchKernelGGL((copy_boxes_kernel<VEC, 4>), g, b, 0, stream, a);
-      break;
-    default:
-      hipLaunchKernelGGL((copy_boxes_kernel<VEC, 8>), g, b, 0, stream, a);
-      break;
-    }
-    int r = check_launch("copy_boxes_kernel");
-    if (r != MDH_OK) {
-      rc = r;
-    }
-  }
-
-  void launch16(CopyArgs& a) {
-    const Tuning& t = tuning();
-    uint32_t grid = a.total_tiles;
-    if (t.copy_max_blocks > 0 && grid > (uint32_t)t.copy_max_blocks) {
-      grid = (uint32_t)t.copy_max_blocks;
-    }
-    dim3 g(grid), b(kBlock);
-    switch (unroll) {
-    case 1:
-      hipLaunchKernelGGL((copy_boxes16_kernel<1>), g, b, lds, stream, a);
-      break;
-    case 2:
-      hipLaunchKernelGGL((copy_boxes16_kernel<2>), g, b, lds, stream, a);
-      break;
-    case 4:
-      hipLaunchKernelGGL((copy_boxes16_kernel<4>), g, b, lds, stream, a);
-      break;
-    default:
-      hipLaunchKernelGGL((copy_boxes16_kernel<8>), g, b, lds, stream, a);
-      break;
-    }
-    int r = check_launch("copy_boxes16_kernel");
-    if (r != MDH_OK) {
-      rc = r;
-    }
+    Step st;
+    st.kind = buffer16 ? Step::kBoxes16 : Step::kBoxes;
+    st.vec = vec, st.unroll = unroll, st.grid = grid, st.lds = buffer16 ? lds : 0;
+    submit(st, nullptr, &a);
   }
 
   void flush_class(int lg) {
@@ -491,26 +465,7 @@ struct Launcher {
       if (tiles == 0) {
         continue;
       }
-      switch (lg) {
-      case 5:
-        launch16(a);
-        break;
-      case 4:
-        launch<16>(a);
-        break;
-      case 3:
-        launch<8>(a);
-        break;
-      case 2:
-        launch<4>(a);
-        break;
-      case 1:
-        launch<2>(a);
-        break;
-      default:
-        launch<1>(a);
-        break;
-      }
+      launch_boxes(a, lg == 5 ? 16 : 1 << lg, lg == 5);
     }
     list.clear();
   }
@@ -706,8 +661,302 @@ bool canonicalise(const char* src, char* dst, int ndim, const int64_t* shape, co
   return true;
 }
 
+template<int VEC>
+void launch_boxes_vec(const Step& st, const CopyArgs& a, hipStream_t stream) {
+  dim3 g(st.grid), b(kBlock);
+  switch (st.unroll) {
+  case 1:
+    hipLaunchKernelGGL((copy_boxes_kernel<VEC, 1>), g, b, 0, stream, a);
+    break;
+  case 2:
+    hipLaunchKernelGGL((copy_boxes_kernel<VEC, 2>), g, b, 0, stream, a);
+    break;
+  case 4:
+    hipLaunchKernelGGL((copy_boxes_kernel<VEC, 4>), g, b, 0, stream, a);
+    break;
+  default:
+    hipLaunchKernelGGL((copy_boxes_kernel<VEC, 8>), g, b, 0, stream, a);
+    break;
+  }
+}
+
+int launch_step(const Step& st, const FlatArgs* flat, const CopyArgs* boxes, hipStream_t stream) {
+  dim3 g(st.grid), b(kBlock);
+  switch (st.kind) {
+  case Step::kFlat:
+    switch (st.unroll) {
+    case 1:
+      hipLaunchKernelGGL((copy_flat_kernel<1>), g, b, st.lds, stream, *flat);
+      break;
+    case 2:
+      hipLaunchKernelGGL((copy_flat_kernel<2>), g, b, st.lds, stream, *flat);
+      break;
+    case 4:
+      hipLaunchKernelGGL((copy_flat_kernel<4>), g, b, st.lds, stream, *flat);
+      break;
+    default:
+      hipLaunchKernelGGL((copy_flat_kernel<8>), g, b, st.lds, stream, *flat);
+      break;
+    }
+    return check_launch("copy_flat_kernel");
+  case Step::kBoxes16:
+    switch (st.unroll) {
+    case 1:
+      hipLaunchKernelGGL((copy_boxes16_kernel<1>), g, b, st.lds, stream, *boxes);
+      break;
+    case 2:
+      hipLaunchKernelGGL((copy_boxes16_kernel<2>), g, b, st.lds, stream, *boxes);
+      break;
+    case 4:
+      hipLaunchKernelGGL((copy_boxes16_kernel<4>), g, b, st.lds, stream, *boxes);
+      break;
+    default:
+      hipLaunchKernelGGL((copy_boxes16_kernel<8>), g, b, st.lds, stream, *boxes);
+      break;
+    }
+    return check_launch("copy_boxes16_kernel");
+  default:
+    switch (st.vec) {
+    case 16:
+      launch_boxes_vec<16>(st, *boxes, stream);
+      break;
+    case 8:
+      launch_boxes_vec<8>(st, *boxes, stream);
+      break;
+    case 4:
+      launch_boxes_vec<4>(st, *boxes, stream);
+      break;
+    case 2:
+      launch_boxes_vec<2>(st, *boxes, stream);
+      break;
+    default:
+      launch_boxes_vec<1>(st, *boxes, stream);
+      break;
+    }
+    return check_launch("copy_boxes_kernel");
+  }
+}
+
+// Checks shared by mdh_copy_boxes and mdh_copy_plan_create.  Returns MDH_OK, or an error with
+// the message set; *empty is set when the box moves nothing.
+int check_box(const char* who, const mdh_box& b, int i, int itemsize, bool* empty) {
+  *empty = false;
+  if (b.ndim < 0 || b.ndim > MDH_MAX_DIMS) {
+    set_error("%s: box %d has %d dimensions (0..%d allowed)", who, i, b.ndim, MDH_MAX_DIMS);
+    return MDH_EINVAL;
+  }
+  int64_t numel = 1;
+  for (int d = 0; d < b.ndim; ++d) {
+    if (b.shape[d] < 0 || b.src_strides[d] < 0 || b.dst_strides[d] < 0) {
+      set_error("%s: box %d has a negative extent or stride", who, i);
+      return MDH_EINVAL;
+    }
+    if (b.shape[d] && numel > ((int64_t)1 << 48) / b.shape[d]) {
+      set_error("%s: box %d is not a plausible device size", who, i);
+      return MDH_EINVAL;
+    }
+    numel *= b.shape[d];
+  }
+  if (numel == 0) {
+    *empty = true;
+    return MDH_OK;
+  }
+  // the bytes a side spans must be a plausible device size too (keeps every later offset
+  // computation inside 64 bits)
+  unsigned __int128 sspan = 0, dspan = 0;
+  for (int d = 0; d < b.ndim; ++d) {
+    sspan += (unsigned __int128)(b.shape[d] - 1) * (unsigned __int128)b.src_strides[d];
+    dspan += (unsigned __int128)(b.shape[d] - 1) * (unsigned __int128)b.dst_strides[d];
+  }
+  if (sspan > ((unsigned __int128)1 << 48) || dspan > ((unsigned __int128)1 << 48)) {
+    set_error("%s: box %d spans more than a plausible device size", who, i);
+    return MDH_EINVAL;
+  }
+  (void)itemsize;
+  return MDH_OK;
+}
+
+// ---- prepared plans ----
+//
+// While a plan is being prepared, base address number `slot` is stood in for by a made-up
+// address (slot + 1) << kSlotShift, 16-byte aligned like every real base a plan accepts; the
+// boxes' offsets ride in the low bits through all the splitting and merging above.  Afterwards
+// every address in the recorded kernel arguments is taken apart again into (slot, offset).
+constexpr int kSlotShift = 44;
+constexpr uint64_t kOffsetMask = ((uint64_t)1 << kSlotShift) - 1;
+
+struct Patch {
+  uint32_t step;
+  uint32_t entry;
+  int32_t src_slot, dst_slot;
+  uint64_t src_off, dst_off;
+};
+
 } // namespace
 } // namespace mdh
+
+struct mdh_copy_plan {
+  std::vector<mdh::Step> steps;
+  std::vector<mdh::Patch> patches;
+  std::vector<mdh_box> boxes; // as given (offsets in src/dst), for bases that are not 16-byte aligned
+  std::vector<int32_t> src_slot, dst_slot;
+  int itemsize = 0;
+  int nbases = 0;
+};
+
+extern "C" int mdh_copy_plan_create(const mdh_box* boxes, const int32_t* src_slots, const int32_t* dst_slots, int nboxes,
+    int itemsize, int nbases, mdh_copy_plan** plan) {
+  using namespace mdh;
+  if (!plan) {
+    set_error("mdh_copy_plan_create: null out pointer");
+    return MDH_EINVAL;
+  }
+  *plan = nullptr;
+  if (nboxes < 0 || (nboxes > 0 && (!boxes || !src_slots || !dst_slots)) || nbases < 0 || nbases > 4096) {
+    set_error("mdh_copy_plan_create: bad table");
+    return MDH_EINVAL;
+  }
+  if (itemsize < 1 || itemsize > 16 || (itemsize & (itemsize - 1))) {
+    set_error("mdh_copy_plan_create: itemsize %d is not 1, 2, 4, 8 or 16", itemsize);
+    return MDH_EINVAL;
+  }
+  std::unique_ptr<mdh_copy_plan> p(new mdh_copy_plan);
+  p->itemsize = itemsize;
+  p->nbases = nbases;
+  Launcher L;
+  L.stream = nullptr;
+  L.record = &p->steps;
+  for (int i = 0; i < nboxes; ++i) {
+    const mdh_box& b = boxes[i];
+    if (src_slots[i] < 0 || src_slots[i] >= nbases || dst_slots[i] < 0 || dst_slots[i] >= nbases) {
+      set_error("mdh_copy_plan_create: box %d names a base outside 0..%d", i, nbases - 1);
+      return MDH_EINVAL;
+    }
+    bool empty;
+    const int rc = check_box("mdh_copy_plan_create", b, i, itemsize, &empty);
+    if (rc != MDH_OK) {
+      return rc;
+    }
+    const uint64_t so = (uint64_t)(uintptr_t)b.src, dof = (uint64_t)(uintptr_t)b.dst;
+    uint64_t sspan = 0, dspan = 0;
+    for (int d = 0; d < b.ndim; ++d) {
+      sspan += (uint64_t)(b.shape[d] ? b.shape[d] - 1 : 0) * (uint64_t)b.src_strides[d];
+      dspan += (uint64_t)(b.shape[d] ? b.shape[d] - 1 : 0) * (uint64_t)b.dst_strides[d];
+    }
+    if (so + (sspan + 1) * (uint64_t)itemsize > kOffsetMask || dof + (dspan + 1) * (uint64_t)itemsize > kOffsetMask) {
+      set_error("mdh_copy_plan_create: box %d reaches past %llu bytes from its base", i, (unsigned long long)kOffsetMask);
+      return MDH_EINVAL;
+    }
+    if ((so | dof) % (unsigned)itemsize) {
+      set_error("mdh_copy_plan_create: box %d is not aligned to its element size", i);
+      return MDH_EINVAL;
+    }
+    p->boxes.push_back(b);
+    p->src_slot.push_back(src_slots[i]);
+    p->dst_slot.push_back(dst_slots[i]);
+    if (empty) {
+      continue;
+    }
+    const char* fake_src = (const char*)(uintptr_t)((((uint64_t)src_slots[i] + 1) << kSlotShift) + so);
+    char* fake_dst = (char*)(uintptr_t)((((uint64_t)dst_slots[i] + 1) << kSlotShift) + dof);
+    HostBox h;
+    if (canonicalise(fake_src, fake_dst, b.ndim, b.shape, b.src_strides, b.dst_strides, itemsize, h)) {
+      L.add(h);
+    }
+  }
+  if (L.rc == MDH_OK) {
+    L.flush();
+  }
+  if (L.rc != MDH_OK) {
+    return L.rc;
+  }
+  auto split = [](const void* fake, int32_t* slot, uint64_t* off) {
+    const uint64_t v = (uint64_t)(uintptr_t)fake;
+    *slot = (int32_t)(v >> kSlotShift) - 1;
+    *off = v & kOffsetMask;
+  };
+  for (size_t s = 0; s < p->steps.size(); ++s) {
+    Step& st = p->steps[s];
+    const uint32_t n = st.kind == Step::kFlat ? st.flat.nsegs : st.boxes.nboxes;
+    for (uint32_t k = 0; k < n; ++k) {
+      Patch pa;
+      pa.step = (uint32_t)s, pa.entry = k;
+      if (st.kind == Step::kFlat) {
+        split(st.flat.src[k], &pa.src_slot, &pa.src_off);
+        split(st.flat.dst[k], &pa.dst_slot, &pa.dst_off);
+      } else {
+        split(st.boxes.box[k].src, &pa.src_slot, &pa.src_off);
+        split(st.boxes.box[k].dst, &pa.dst_slot, &pa.dst_off);
+      }
+      p->patches.push_back(pa);
+    }
+  }
+  *plan = p.release();
+  return MDH_OK;
+}
+
+extern "C" void mdh_copy_plan_destroy(mdh_copy_plan* plan) {
+  delete plan;
+}
+
+extern "C" int mdh_copy_plan_launches(const mdh_copy_plan* plan) {
+  return plan ? (int)plan->steps.size() : -1;
+}
+
+extern "C" int mdh_copy_plan_launch(const mdh_copy_plan* plan, const void* const* bases, int nbases, void* stream) {
+  using namespace mdh;
+  if (!plan || nbases != plan->nbases || (nbases > 0 && !bases)) {
+    set_error("mdh_copy_plan_launch: the plan takes %d base addresses", plan ? plan->nbases : 0);
+    return MDH_EINVAL;
+  }
+  uintptr_t low = 0;
+  for (int i = 0; i < nbases; ++i) {
+    low |= (uintptr_t)bases[i];
+  }
+  if (low & 15) {
+    // prepared for 16-byte aligned bases (what decides the vector width of narrow rows): any
+    // other table goes the general way, box by box
+    std::vector<mdh_box> boxes(plan->boxes);
+    for (size_t i = 0; i < boxes.size(); ++i) {
+      boxes[i].src = (const char*)bases[plan->src_slot[i]] + (uintptr_t)plan->boxes[i].src;
+      boxes[i].dst = (char*)bases[plan->dst_slot[i]] + (uintptr_t)plan->boxes[i].dst;
+    }
+    return mdh_copy_boxes(boxes.data(), (int)boxes.size(), plan->itemsize, stream);
+  }
+  // a used base must exist
+  for (const Patch& pa : plan->patches) {
+    if (!bases[pa.src_slot] || !bases[pa.dst_slot]) {
+      set_error("mdh_copy_plan_launch: base %d is null", !bases[pa.src_slot] ? pa.src_slot : pa.dst_slot);
+      return MDH_EINVAL;
+    }
+  }
+  size_t at = 0;
+  for (size_t s = 0; s < plan->steps.size(); ++s) {
+    const Step& st = plan->steps[s];
+    int rc;
+    if (st.kind == Step::kFlat) {
+      FlatArgs a = st.flat;
+      for (; at < plan->patches.size() && plan->patches[at].step == s; ++at) {
+        const Patch& pa = plan->patches[at];
+        a.src[pa.entry] = (const char*)bases[pa.src_slot] + pa.src_off;
+        a.dst[pa.entry] = (char*)bases[pa.dst_slot] + pa.dst_off;
+      }
+      rc = launch_step(st, &a, nullptr, (hipStream_t)stream);
+    } else {
+      CopyArgs a = st.boxes;
+      for (; at < plan->patches.size() && plan->patches[at].step == s; ++at) {
+        const Patch& pa = plan->patches[at];
+        a.box[pa.entry].src = (const char*)bases[pa.src_slot] + pa.src_off;
+        a.box[pa.entry].dst = (char*)bases[pa.dst_slot] + pa.dst_off;
+      }
+      rc = launch_step(st, nullptr, &a, (hipStream_t)stream);
+    }
+    if (rc != MDH_OK) {
+      return rc;
+    }
+  }
+  return MDH_OK;
+}
 
 extern "C" int mdh_copy_boxes(const mdh_box* boxes, int nboxes, int itemsize, void* stream) {
   using namespace mdh;
@@ -723,35 +972,13 @@ extern "C" int mdh_copy_boxes(const mdh_box* boxes, int nboxes, int itemsize, vo
   L.stream = (hipStream_t)stream;
   for (int i = 0; i < nboxes; ++i) {
     const mdh_box& b = boxes[i];
-    if (b.ndim < 0 || b.ndim > MDH_MAX_DIMS) {
-      set_error("mdh_copy_boxes: box %d has %d dimensions (0..%d allowed)", i, b.ndim, MDH_MAX_DIMS);
-      return MDH_EINVAL;
+    bool empty;
+    const int rc = check_box("mdh_copy_boxes", b, i, itemsize, &empty);
+    if (rc != MDH_OK) {
+      return rc;
     }
-    int64_t numel = 1;
-    for (int d = 0; d < b.ndim; ++d) {
-      if (b.shape[d] < 0 || b.src_strides[d] < 0 || b.dst_strides[d] < 0) {
-        set_error("mdh_copy_boxes: box %d has a negative extent or stride", i);
-        return MDH_EINVAL;
-      }
-      if (b.shape[d] && numel > ((int64_t)1 << 48) / b.shape[d]) {
-        set_error("mdh_copy_boxes: box %d is not a plausible device size", i);
-        return MDH_EINVAL;
-      }
-      numel *= b.shape[d];
-    }
-    if (numel == 0) {
+    if (empty) {
       continue;
-    }
-    // the bytes a side spans must be a plausible device size too (keeps every later offset
-    // computation inside 64 bits)
-    unsigned __int128 sspan = 0, dspan = 0;
-    for (int d = 0; d < b.ndim; ++d) {
-      sspan += (unsigned __int128)(b.shape[d] - 1) * (unsigned __int128)b.src_strides[d];
-      dspan += (unsigned __int128)(b.shape[d] - 1) * (unsigned __int128)b.dst_strides[d];
-    }
-    if (sspan > ((unsigned __int128)1 << 48) || dspan > ((unsigned __int128)1 << 48)) {
-      set_error("mdh_copy_boxes: box %d spans more than a plausible device size", i);
-      return MDH_EINVAL;
     }
     if (!b.src || !b.dst) {
       set_error("mdh_copy_boxes: box %d has a null pointer", i);

@@ -489,3 +489,41 @@ def test_compile_op_accepts_dtensor_like_specs():
     with pytest.raises(ValueError, match="same dtype"):
         moodist_amd.compile_op(world.groups[0], inputs=[rep],
                                outputs=[FakeDTensor([5, 4], torch.float64, [Shard(0)], Mesh([2], [0]))])
+
+
+def _runs(core, srcs, nbytes, dst=None):
+    core.moodist_kernel_less_runs.restype = ctypes.c_int64
+    core.moodist_kernel_less_runs.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_size_t, ctypes.c_size_t,
+                                              ctypes.c_void_p, ctypes.POINTER(ctypes.c_int64), ctypes.c_size_t]
+    tab = (ctypes.c_void_p * len(srcs))(*srcs)
+    out = (ctypes.c_int64 * (3 * len(srcs) + 3))()
+    n = core.moodist_kernel_less_runs(tab, len(srcs), nbytes, dst, out, len(out))
+    return [tuple(out[3 * i:3 * i + 3]) for i in range(n)]
+
+
+def test_kernel_less_runs_group_evenly_spaced_sources(core):
+    # The reference groups the sources a peer holds into Copy2d{offset, length, pitch, num} runs for
+    # cuMemcpy2DAsync (core/processgroup.cc:618-704); here the sources are the ranks' own buffers and a
+    # run is a stretch of ranks whose buffers are evenly spaced.  (first rank, count, source pitch):
+    b, n = 0x7f0000000000, 4096
+    # slices of one dense staging buffer: one run whose pitch equals the width (a single 1-D copy)
+    assert _runs(core, [b + j * n for j in range(8)], n) == [(0, 8, n)]
+    # rows of a padded staging buffer: one 2-D copy
+    assert _runs(core, [b + j * (n + 64) for j in range(8)], n) == [(0, 8, n + 64)]
+    # two staging buffers of four rows each, with different pitches
+    two = [b + j * (n + 64) for j in range(4)] + [b + (1 << 30) + j * (2 * n) for j in range(4)]
+    assert _runs(core, two, n) == [(0, 4, n + 64), (4, 4, 2 * n)]
+    # unrelated allocations, some closer together than a row is long or in descending order: rank by rank
+    odd = [b, b + 100, b + 50, b + (1 << 33), b + (1 << 32)]
+    assert _runs(core, odd, n) == [(j, 1, n) for j in range(5)]
+    # a pitch that changes mid-way ends the run; the leftover pair forms its own
+    bend = [b, b + 2 * n, b + 4 * n, b + 7 * n, b + 10 * n]
+    assert _runs(core, bend, n) == [(0, 3, 2 * n), (3, 2, 3 * n)]
+    # pitches beyond 31 bits are not handed to a 2-D copy
+    assert _runs(core, [b, b + (1 << 31), b + (1 << 32)], n) == [(0, 1, n), (1, 1, n), (2, 1, n)]
+    # in-place allreduce: rank 3's chunk already sits in the destination and splits the run
+    dst = b + (1 << 34)
+    srcs = [b + j * (n + 64) for j in range(8)]
+    srcs[3] = dst + 3 * n
+    assert _runs(core, srcs, n, dst) == [(0, 3, n + 64), (4, 4, n + 64)]
+    assert _runs(core, [], n) == []

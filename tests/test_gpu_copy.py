@@ -1,12 +1,16 @@
 """Parity of the HIP gather / box-copy kernels against the oracle and torch slicing, through the
 C ABI.  Everything here is byte-exact."""
 
+import os
+
 import numpy as np
 import pytest
 import torch
 
 import oracle
 from moodist_amd import _abi as abi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 pytestmark = pytest.mark.gpu
 
@@ -336,3 +340,106 @@ def test_gather_and_boxes_beyond_4_gib(dev):
     abi.copy_boxes([abi.make_box(big.data_ptr(), dst.data_ptr(), [rows, width], [pitch, 1], [width, 1])], 1, st())
     sync()
     assert torch.equal(dst.view(rows, width), big.view(rows, pitch)[:, :width])
+
+
+# ---- prepared plans (mdh_copy_plan_*): the compiled form of a set of box copies ----
+
+
+def _plan_vs_boxes(dev, specs, itemsize, base_misalign=0):
+    """specs: (src numel, dst numel, src offset, dst offset, shape, src strides, dst strides) per box, in
+    elements; every box has its own source tensor and they share one destination."""
+    g = torch.Generator().manual_seed(77)
+    dst_numel = max(s[1] for s in specs)
+    raw = lambda n: torch.randint(0, 256, (n * itemsize + 64,), dtype=torch.uint8, generator=g).to(dev)
+    srcs = [raw(s[0]) for s in specs]
+    want, got = raw(dst_numel), None
+    got = want.clone()
+    mis = base_misalign
+    boxes, offs, ss, ds = [], [], [], []
+    for i, (sn, dn, so, do, shape, sstr, dstr) in enumerate(specs):
+        boxes.append(abi.make_box(srcs[i].data_ptr() + mis + so * itemsize, want.data_ptr() + mis + do * itemsize,
+                                  shape, sstr, dstr))
+        offs.append(abi.make_box(so * itemsize, do * itemsize, shape, sstr, dstr))
+        ss.append(i)
+        ds.append(len(specs))
+    st = torch.cuda.current_stream().cuda_stream
+    abi.copy_boxes(boxes, itemsize, st)
+    plan = abi.CopyPlan(offs, ss, ds, itemsize, len(specs) + 1)
+    plan.launch([s.data_ptr() + mis for s in srcs] + [got.data_ptr() + mis], st)
+    plan.launch([s.data_ptr() + mis for s in srcs] + [got.data_ptr() + mis], st)  # replays are idempotent
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    return plan
+
+
+def test_plan_matches_copy_boxes_on_the_redistribution_shapes(dev):
+    # C5: 8 slabs [1024, 8192] -> column block [8192, 1024] (fp32 and bf16), and [8,512,1024] -> [64,512,128]
+    for itemsize in (4, 2):
+        specs = [(1024 * 8192, 8192 * 1024, 3 * 1024, s * 1024 * 1024, [1024, 1024], [8192, 1], [1024, 1])
+                 for s in range(8)]
+        assert _plan_vs_boxes(dev, specs, itemsize).launches == 1
+    specs = [(8 * 512 * 1024, 64 * 512 * 128, 5 * 128, s * 8 * 512 * 128, [8, 512, 128], [512 * 1024, 1024, 1],
+              [512 * 128, 128, 1]) for s in range(8)]
+    assert _plan_vs_boxes(dev, specs, 2).launches == 1
+
+
+@pytest.mark.parametrize("misalign", [0, 4, 2, 1])
+def test_plan_with_ragged_rows_dense_runs_and_unaligned_bases(dev, misalign):
+    # rows that are not a multiple of 16 bytes (body + tail boxes), a dense run (flat segment), a
+    # transposing box, a scalar; with bases that are not 16-byte aligned the plan goes the general way
+    itemsize = 1 if misalign in (1, 2) else 4
+    if misalign % itemsize:
+        pytest.skip("a base must be aligned to the element size")
+    specs = [
+        (40 * 1000, 70000, 7, 11, [37, 1001 // itemsize], [1000, 1], [1001 // itemsize + 3, 1]),
+        (65536, 70000, 0, 40000, [65536 // 4], [1], [1]),
+        (5000, 70000, 3, 60000, [40, 50], [1, 60], [50, 1]),
+        (16, 70000, 5, 69999, [], [], []),
+        (9000, 70000, 0, 38000, [3, 4, 5, 6], [2000, 400, 60, 1], [130, 31, 6, 1]),
+    ]
+    plan = _plan_vs_boxes(dev, specs, itemsize, base_misalign=misalign)
+    assert plan.launches >= 2
+
+
+def test_plan_random_boxes_against_copy_boxes(dev):
+    rng = np.random.RandomState(5)
+    for trial in range(25):
+        itemsize = int(rng.choice([1, 2, 4, 8]))
+        specs = []
+        dst_at = 0
+        for _ in range(int(rng.randint(1, 6))):
+            nd = int(rng.randint(1, 4))
+            shape = [int(rng.randint(1, 40)) for _ in range(nd)]
+            shape[-1] = int(rng.choice([1, 3, 8, 16, 64, 257]))
+            pad_s, pad_d = int(rng.randint(0, 5)), int(rng.randint(0, 5))
+            sstr, dstr = [1] * nd, [1] * nd
+            for d in range(nd - 2, -1, -1):
+                sstr[d] = sstr[d + 1] * shape[d + 1] + (pad_s if d == nd - 2 else 0)
+                dstr[d] = dstr[d + 1] * shape[d + 1] + (pad_d if d == nd - 2 else 0)
+            sn = sstr[0] * shape[0] + 8
+            dn = dstr[0] * shape[0]
+            specs.append((sn, 0, int(rng.randint(0, 8)), dst_at, shape, sstr, dstr))
+            dst_at += dn + int(rng.randint(0, 9))
+        specs = [(s[0], dst_at + 8) + s[2:] for s in specs]
+        _plan_vs_boxes(dev, specs, itemsize)
+
+
+def test_host_cost_of_a_compiled_redistribution_from_cpp(dev):
+    # the C++ loop: enqueuing a prepared plan must cost the host less than the general entry point,
+    # and less than the fp32 8192 x 8192 kernel takes (about 12 us)
+    import subprocess
+
+    exe = os.path.join(ROOT, "tests", "native", "host_cost_driver.bin")
+    if not os.path.exists(exe):
+        pytest.skip("tests/native/host_cost_driver.bin is not built (run __graft_entry__.build())")
+    r = subprocess.run([exe, abi.LIB_PATH], capture_output=True, text=True, timeout=300)
+    print(r.stdout)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    assert "host cost driver done" in r.stdout and "DIFFER" not in r.stdout
+    import re
+
+    rows = re.findall(r"general ([\d.]+)  prepared ([\d.]+)", r.stdout)
+    assert len(rows) == 3
+    for general, prepared in rows:
+        assert float(prepared) < float(general)
+        assert float(prepared) < 10.0

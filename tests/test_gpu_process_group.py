@@ -488,3 +488,44 @@ def test_snapshot_inputs_with_allreduce_and_allgather(world, dev):
         assert torch.equal(ts[r], torch.full((n,), P * (P + 1) / 2, device=dev))
         assert torch.equal(ev[r], torch.full((P * 64,), P * (P + 1) / 2, device=dev))
         assert torch.equal(outs[r], torch.arange(P, device=dev, dtype=torch.float32).repeat_interleave(100))
+
+
+def test_kernel_less_gather_from_padded_staging_equals_the_kernel_path(world, dev):
+    # The ranks' inputs are rows of ONE padded staging buffer (pitch > row bytes): with
+    # force_kernel_less the core groups them into a single hipMemcpy2DAsync (the reference's Copy2d +
+    # cuMemcpy2DAsync form, core/processgroup.cc:114-119, :618-704, :806-820); the kernel path
+    # moves the same rows as strided boxes.  Same bytes either way.
+    n, pad = 50000 + 3, 29
+    g = torch.Generator().manual_seed(3)
+    staging = torch.randn(P, n + pad, generator=g).to(dev)
+    ins = [staging[r, :n] for r in range(P)]
+    assert all(t.is_contiguous() for t in ins)
+    results = {}
+    for kernel_less in (False, True):
+        for pg in world:
+            pg.options().force_kernel_less = kernel_less
+        before = (world.groups[0]._get_option("kernel_less_copies_1d"), world.groups[0]._get_option("kernel_less_copies_2d"))
+        outs = [torch.full((P * n,), -1.0, device=dev) for _ in range(P)]
+        each_rank(world, lambda r, pg: pg._allgather_base(outs[r], ins[r]))
+        after = (world.groups[0]._get_option("kernel_less_copies_1d"), world.groups[0]._get_option("kernel_less_copies_2d"))
+        results[kernel_less] = outs
+        # one 2-D copy per rank's output in the kernel-less form, none in the kernel form
+        assert (after[0] - before[0], after[1] - before[1]) == ((0, P) if kernel_less else (0, 0))
+    want = staging[:, :n].reshape(-1)
+    for r in range(P):
+        assert torch.equal(results[False][r], want) and torch.equal(results[True][r], want)
+    # dense staging (pitch == row bytes): one 1-D copy of everything; separate allocations: one per rank
+    dense = torch.randn(P, n, generator=g).to(dev)
+    separate = [torch.randn(n, generator=g).to(dev) for _ in range(P)]
+    for ins2, want2, expect in (([dense[r] for r in range(P)], dense.reshape(-1), (P, 0)),
+                                (separate, torch.cat(separate), None)):
+        before = (world.groups[0]._get_option("kernel_less_copies_1d"), world.groups[0]._get_option("kernel_less_copies_2d"))
+        outs = [torch.zeros(P * n, device=dev) for _ in range(P)]
+        each_rank(world, lambda r, pg: pg._allgather_base(outs[r], ins2[r]))
+        after = (world.groups[0]._get_option("kernel_less_copies_1d"), world.groups[0]._get_option("kernel_less_copies_2d"))
+        if expect:
+            assert (after[0] - before[0], after[1] - before[1]) == expect
+        for r in range(P):
+            assert torch.equal(outs[r], want2)
+    for pg in world:
+        pg.options().force_kernel_less = False
