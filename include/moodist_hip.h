@@ -167,12 +167,19 @@ int mdh_copy_boxes(const mdh_box* boxes, int nboxes, int itemsize, void* stream)
  * allocations are); a table with a less aligned base is served through mdh_copy_boxes.
  * A plan is immutable after create: launches of one plan may run concurrently.
  * launches: how many kernels one launch of the plan enqueues (-1 for NULL).
+ * verify: replays the plan's kernels ON THE HOST -- every tile, every slot, through the very
+ * index functions the device code is built from -- against bases of the given byte sizes, and
+ * checks that no access leaves its base or is clipped by a box's buffer descriptor, that every
+ * destination byte the boxes name is written exactly once, and that it receives the source byte
+ * the boxes name.  Needs no device; walks byte by byte (bases up to 2 GiB).  No counterpart in
+ * the reference (its coverage check is on the plan, core/processgroup.cc:3079-3081).
  */
 typedef struct mdh_copy_plan mdh_copy_plan;
 int mdh_copy_plan_create(const mdh_box* boxes, const int32_t* src_slots, const int32_t* dst_slots, int nboxes,
     int itemsize, int nbases, mdh_copy_plan** plan);
 int mdh_copy_plan_launch(const mdh_copy_plan* plan, const void* const* bases, int nbases, void* stream);
 int mdh_copy_plan_launches(const mdh_copy_plan* plan);
+int mdh_copy_plan_verify(const mdh_copy_plan* plan, const uint64_t* base_bytes, int nbases);
 void mdh_copy_plan_destroy(mdh_copy_plan* plan);
 
 /*
@@ -183,7 +190,9 @@ void mdh_copy_plan_destroy(mdh_copy_plan* plan);
  * "reduce_max_blocks" (waves of the grid; 0 = chosen by size), "reduce_wg_per_cu" (2..8
  * caps the workgroups resident on a CU, 9 = never cap), "copy_unroll" (1, 2,
  * 4, 8; contiguous segments), "box_unroll" (1, 2, 4, 8; strided boxes),
- * "copy_max_blocks", "copy_wg_per_cu" (2..8, 9 = never cap).  Returns MDH_EINVAL for an unknown name or value.
+ * "copy_max_blocks", "copy_wg_per_cu" (2..8, 9 = never cap), "box_policy" (loads of the
+ * strided-box kernel: 1 = plain, as chosen for sources whose rows are not adjacent, 2 = nt, as
+ * chosen for densely read sources).  Returns MDH_EINVAL for an unknown name or value.
  * No counterpart in the reference, whose grid is fixed at 4/16/64 blocks
  * (core/kernels.cc:547-556).
  */

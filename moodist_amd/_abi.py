@@ -21,7 +21,7 @@ ABI_VERSION = 2
 SYMBOLS = (
     "mdh_abi_version", "mdh_error_string", "mdh_last_error", "mdh_reduce", "mdh_gather", "mdh_copy_boxes",
     "mdh_set_tuning", "mdh_get_tuning", "mdh_copy_plan_create", "mdh_copy_plan_launch", "mdh_copy_plan_launches",
-    "mdh_copy_plan_destroy",
+    "mdh_copy_plan_verify", "mdh_copy_plan_destroy",
 )
 
 
@@ -73,6 +73,8 @@ def lib():
     L.mdh_copy_plan_launch.restype = ctypes.c_int
     L.mdh_copy_plan_launches.argtypes = [ctypes.c_void_p]
     L.mdh_copy_plan_launches.restype = ctypes.c_int
+    L.mdh_copy_plan_verify.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint64), ctypes.c_int]
+    L.mdh_copy_plan_verify.restype = ctypes.c_int
     L.mdh_copy_plan_destroy.argtypes = [ctypes.c_void_p]
     L.mdh_copy_plan_destroy.restype = None
     L.mdh_set_tuning.argtypes = [ctypes.c_char_p, ctypes.c_int]
@@ -136,6 +138,11 @@ class CopyPlan:
 
     def launch(self, bases, stream=0):
         check(lib().mdh_copy_plan_launch(self._plan, ptr_table(bases), len(bases), stream))
+
+    def verify(self, base_bytes):
+        """Host-side replay of the plan's kernels against bases of these sizes (no GPU needed)."""
+        arr = (ctypes.c_uint64 * max(len(base_bytes), 1))(*base_bytes)
+        check(lib().mdh_copy_plan_verify(self._plan, arr, len(base_bytes)))
 
     @property
     def launches(self):

@@ -30,8 +30,3 @@ done
 printf '%s\n' "${cmds[@]}" | xargs -P "$jobs" -I{} bash -c '{} 2> >(grep -v "packed-fp32-ops" >&2)'
 /opt/rocm/bin/hipcc -shared -fPIC --offload-arch=gfx950 -o "$out" "${objs[@]}"
 echo "built $out"
-# the streaming-ceiling microbenchmark the kernels' rates are compared with (moodist_amd/hbm_ceilings.bin)
-if [ -z "$extra" ] && [ "$out" = "$here/../libmoodist_hip.so" ]; then
-  /opt/rocm/bin/hipcc -O3 -std=c++17 --offload-arch=gfx950 -o "$here/../hbm_ceilings.bin" "$here/bench/hbm_ceilings.hip"
-  echo "built $here/../hbm_ceilings.bin"
-fi

@@ -86,6 +86,9 @@ int* knob(const char* name) {
   if (!std::strcmp(name, "copy_wg_per_cu")) {
     return &t.copy_wg_per_cu;
   }
+  if (!std::strcmp(name, "box_policy")) {
+    return &t.box_policy;
+  }
   if (!std::strcmp(name, "copy_max_blocks")) {
     return &t.copy_max_blocks;
   }
@@ -106,7 +109,7 @@ extern "C" int mdh_set_tuning(const char* name, int value) {
       mdh::set_error("mdh_set_tuning: %s does not take %d", name, value);
       return MDH_EINVAL;
     }
-  } else if (value < 0 || (std::strstr(name, "wg_per_cu") && value > 9)) {
+  } else if (value < 0 || (std::strstr(name, "wg_per_cu") && value > 9) || (!std::strcmp(name, "box_policy") && value > 2)) {
     mdh::set_error("mdh_set_tuning: %s does not take %d", name, value);
     return MDH_EINVAL;
   }

@@ -74,56 +74,89 @@ constexpr uint32_t ilog2(uint32_t x) {
   return x <= 1 ? 0 : 1 + ilog2(x >> 1);
 }
 
+// ---- index arithmetic, shared by the kernels and by the host-side verifier of a plan ----
+
+#define MDH_HD __host__ __device__ __forceinline__
+
+struct TileLoc {
+  uint32_t box; // which box of the table
+  uint32_t rt;  // row of tiles inside the box
+  uint32_t ct;  // column of tiles
+};
+
+// Which box a tile belongs to.  Equal boxes (the shards of a gather or of a redistribution): one
+// division.  Otherwise the cumulative ends are scanned: they ascend, so the last one at or
+// below the tile names the box; written as selects of scalars so that on the device the whole
+// scan stays on the scalar unit (the table sits in the kernel arguments).
+template<bool MAY_DIVIDE>
+MDH_HD TileLoc locate_tile(const CopyArgs& a, uint32_t tile) {
+  uint32_t b = 0, start = 0;
+  if (MAY_DIVIDE && a.tiles_per_box) {
+    b = tile / a.tiles_per_box;
+    start = b * a.tiles_per_box;
+  } else {
+#pragma unroll
+    for (int k = 0; k < kMaxBoxes - 1; ++k) {
+      const uint32_t e = a.tile_end[k];
+      b = tile >= e ? (uint32_t)(k + 1) : b;
+      start = tile >= e ? e : start;
+    }
+  }
+  const uint32_t local = tile - start;
+  const uint32_t rt = local / a.box[b].nct;
+  return TileLoc{b, rt, local - rt * a.box[b].nct};
+}
+
+// Slot `slot` of a tile (kBlock*U slots shaped 2^(log2slots-log2tc) rows x 2^log2tc columns):
+// byte offsets of its vector from the box's src and dst.  Returns false for a slot outside the
+// box (the ragged right and bottom edges).
+template<typename Off>
+MDH_HD bool slot_offsets(const BoxDesc& B, const TileLoc& t, uint32_t slot, uint32_t log2slots, uint32_t vec, Off* so,
+    Off* dof) {
+  const uint32_t log2tc = B.log2tc;
+  const uint32_t log2tr = log2slots - log2tc;
+  const uint32_t tcmask = (1u << log2tc) - 1u;
+  const uint32_t col = (t.ct << log2tc) + (slot & tcmask);
+  uint32_t row = (t.rt << log2tr) + (slot >> log2tc);
+  const bool ok = col < B.cols && row < B.rows;
+  Off s, d;
+  if (B.nouter <= 1) {
+    s = (Off)row * (Off)B.src_stride[0];
+    d = (Off)row * (Off)B.dst_stride[0];
+  } else {
+    s = 0, d = 0;
+    for (uint32_t k = 0; k + 1 < B.nouter; ++k) {
+      const uint32_t q = row / B.outer[k];
+      const uint32_t i = row - q * B.outer[k];
+      s += (Off)i * (Off)B.src_stride[k];
+      d += (Off)i * (Off)B.dst_stride[k];
+      row = q;
+    }
+    s += (Off)row * (Off)B.src_stride[B.nouter - 1];
+    d += (Off)row * (Off)B.dst_stride[B.nouter - 1];
+  }
+  *so = s + (Off)col * (Off)vec;
+  *dof = d + (Off)col * (Off)vec;
+  return ok;
+}
+
 template<int VEC, int U>
 __global__ __launch_bounds__(kBlock) void copy_boxes_kernel(CopyArgs a) {
   using V = typename VecType<VEC>::type;
   constexpr uint32_t log2slots = ilog2(kBlock * U);
-  for (uint32_t tile = blockIdx.x; tile < a.total_tiles; tile += gridDim.x) {
-    // which box: count the cumulative ends at or below this tile (all scalar,
-    // the table sits in the kernel arguments)
-    uint32_t b = 0, start = 0;
-#pragma unroll
-    for (int k = 0; k < kMaxBoxes - 1; ++k) {
-      const uint32_t e = a.tile_end[k];
-      // ends ascend, so the last one at or below the tile names the box; written as selects
-      // of scalars so that the whole scan stays on the scalar unit
-      b = tile >= e ? (uint32_t)(k + 1) : b;
-      start = tile >= e ? e : start;
-    }
-    const BoxDesc& B = a.box[b];
-    const uint32_t local = tile - start;
-    const uint32_t rt = local / B.nct;
-    const uint32_t ct = local - rt * B.nct;
-    const uint32_t log2tc = B.log2tc;
-    const uint32_t log2tr = log2slots - log2tc;
-    const uint32_t tcmask = (1u << log2tc) - 1u;
+  // The grid never exceeds the tile count, so the first tile needs no test: the scalar loads of
+  // the whole table header are then issued together instead of behind a first load-and-branch.
+  uint32_t tile = blockIdx.x;
+  do {
+    const TileLoc t = locate_tile<false>(a, tile);
+    const BoxDesc& B = a.box[t.box];
     V v[U];
     bool ok[U];
     int64_t doff[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const uint32_t slot = (uint32_t)u * kBlock + threadIdx.x;
-      const uint32_t col = (ct << log2tc) + (slot & tcmask);
-      uint32_t row = (rt << log2tr) + (slot >> log2tc);
-      ok[u] = col < B.cols && row < B.rows;
-      int64_t so, dof;
-      if (B.nouter <= 1) {
-        so = (int64_t)row * B.src_stride[0];
-        dof = (int64_t)row * B.dst_stride[0];
-      } else {
-        so = 0, dof = 0;
-        for (uint32_t k = 0; k + 1 < B.nouter; ++k) {
-          const uint32_t q = row / B.outer[k];
-          const uint32_t i = row - q * B.outer[k];
-          so += (int64_t)i * B.src_stride[k];
-          dof += (int64_t)i * B.dst_stride[k];
-          row = q;
-        }
-        so += (int64_t)row * B.src_stride[B.nouter - 1];
-        dof += (int64_t)row * B.dst_stride[B.nouter - 1];
-      }
-      so += (int64_t)col * VEC;
-      doff[u] = dof + (int64_t)col * VEC;
+      int64_t so;
+      ok[u] = slot_offsets<int64_t>(B, t, (uint32_t)u * kBlock + threadIdx.x, log2slots, VEC, &so, &doff[u]);
       if (ok[u]) {
         v[u] = stream_load((const V*)(B.src + so));
       }
@@ -134,7 +167,8 @@ __global__ __launch_bounds__(kBlock) void copy_boxes_kernel(CopyArgs a) {
         stream_store((V*)(B.dst + doff[u]), v[u]);
       }
     }
-  }
+    tile += gridDim.x;
+  } while (tile < a.total_tiles);
 }
 
 // The same tiling for boxes whose byte span fits 32 bits on both sides (all but
@@ -143,68 +177,59 @@ __global__ __launch_bounds__(kBlock) void copy_boxes_kernel(CopyArgs a) {
 // a slot costs two integer multiplies instead of 64-bit address arithmetic, and
 // an out-of-range slot is given the offset just past the descriptor's end -- its
 // load returns zero and its store is dropped -- instead of a predicate.
-template<int U>
+//
+// EQUAL: every box of the table has the same number of tiles (the shards of a gather or of a
+// redistribution).  The grid is then two-dimensional -- blockIdx.y is the box, blockIdx.x the
+// tile inside it -- so the address of the box's descriptor is known when the wave starts and
+// all of its scalar loads go out in one batch; nothing of the table header is read.  On the
+// 16 MiB redistribution, whose whole launch lasts 5 us, that is 0.5 us.
+//
+// SPARSE selects the cache policy of the loads: plain when the source rows are not adjacent in
+// memory (a redistribution reads one block of columns out of every row), nt when the source is
+// read densely (a gather into a padded destination).  Stores are nt+sc1 either way.  Measured
+// on MI355X, us per launch (loads plain / nt):
+//   [64,512,1024] bf16 dim0->dim2, 16 MiB moved    3.92 /  4.60      8192^2 bf16, 32 MiB    6.92 /  7.79
+//   8192^2 fp32, 64 MiB                           10.91 / 12.85      16384^2 fp32, 256 MiB  40.85 / 44.61
+//   gather 8 x [4096,4096] bf16 into pitch 4160   85.25 / 81.63      8 x [1024,4096]        24.28 / 23.38
+// (with sc1 stores and nt loads, the former policy, the first four took 4.49 / 7.52 / 11.93 / 44.6
+// and the gather 83.9.)
+template<int U, bool EQUAL, bool SPARSE>
 __global__ __launch_bounds__(kBlock) void copy_boxes16_kernel(CopyArgs a) {
+  constexpr int kLoad = SPARSE ? 0 : 2;
+  constexpr int kStore = 18;
   constexpr uint32_t log2slots = ilog2(kBlock * U);
-  for (uint32_t tile = blockIdx.x; tile < a.total_tiles; tile += gridDim.x) {
-    uint32_t b = 0, start = 0;
-    if (a.tiles_per_box) {
-      b = tile / a.tiles_per_box; // equal boxes (the shards of a gather or of a redistribution)
-      start = b * a.tiles_per_box;
+  uint32_t tile = blockIdx.x; // first tile untested, as above
+  do {
+    TileLoc t;
+    if (EQUAL) {
+      const uint32_t nct = a.box[blockIdx.y].nct;
+      const uint32_t rt = blockIdx.x / nct;
+      t = TileLoc{blockIdx.y, rt, blockIdx.x - rt * nct};
     } else {
-#pragma unroll
-      for (int k = 0; k < kMaxBoxes - 1; ++k) {
-        const uint32_t e = a.tile_end[k];
-        // ends ascend, so the last one at or below the tile names the box; written as selects
-        // of scalars so that the whole scan stays on the scalar unit
-        b = tile >= e ? (uint32_t)(k + 1) : b;
-        start = tile >= e ? e : start;
-      }
+      t = locate_tile<true>(a, tile);
     }
-    const BoxDesc& B = a.box[b];
-    const uint32_t local = tile - start;
-    const uint32_t rt = local / B.nct;
-    const uint32_t ct = local - rt * B.nct;
-    const uint32_t log2tc = B.log2tc;
-    const uint32_t log2tr = log2slots - log2tc;
-    const uint32_t tcmask = (1u << log2tc) - 1u;
+    const BoxDesc& B = a.box[t.box];
     const __amdgpu_buffer_rsrc_t rs = tile_rsrc(B.src, B.src_span);
     const __amdgpu_buffer_rsrc_t rd = tile_rsrc(B.dst, B.dst_span);
     u32x4 v[U];
     uint32_t doff[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const uint32_t slot = (uint32_t)u * kBlock + threadIdx.x;
-      const uint32_t col = (ct << log2tc) + (slot & tcmask);
-      uint32_t row = (rt << log2tr) + (slot >> log2tc);
-      const bool ok = col < B.cols && row < B.rows;
       uint32_t so, dof;
-      if (B.nouter <= 1) {
-        so = row * (uint32_t)B.src_stride[0];
-        dof = row * (uint32_t)B.dst_stride[0];
-      } else {
-        so = 0, dof = 0;
-        for (uint32_t k = 0; k + 1 < B.nouter; ++k) {
-          const uint32_t q = row / B.outer[k];
-          const uint32_t i = row - q * B.outer[k];
-          so += i * (uint32_t)B.src_stride[k];
-          dof += i * (uint32_t)B.dst_stride[k];
-          row = q;
-        }
-        so += row * (uint32_t)B.src_stride[B.nouter - 1];
-        dof += row * (uint32_t)B.dst_stride[B.nouter - 1];
-      }
-      so += col * 16u;
-      dof += col * 16u;
+      const bool ok = slot_offsets<uint32_t>(B, t, (uint32_t)u * kBlock + threadIdx.x, log2slots, 16u, &so, &dof);
       // the span itself is the first offset past the descriptor's end
       doff[u] = ok ? dof : B.dst_span;
-      v[u] = tile_load(rs, ok ? so : B.src_span);
+      v[u] = tile_load<kLoad>(rs, ok ? so : B.src_span);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      tile_store(rd, doff[u], v[u]);
+      tile_store<kStore>(rd, doff[u], v[u]);
     }
-  }
+    if (EQUAL) {
+      break; // one tile per workgroup
+    }
+    tile += gridDim.x;
+  } while (tile < a.total_tiles);
 }
 
 // Contiguous segments (the shards of a dense all-gather, or any box that
@@ -225,26 +250,35 @@ struct FlatArgs {
 };
 static_assert(sizeof(FlatArgs) <= 4096, "kernel arguments are limited to 4 KiB");
 
-template<int U>
+// Which segment a tile belongs to, and the tile's first byte inside it (same two ways as for boxes).
+MDH_HD uint32_t locate_segment(const FlatArgs& a, uint32_t tile, uint32_t* local) {
+  uint32_t seg;
+  if (a.tiles_per_seg) {
+    seg = tile / a.tiles_per_seg;
+    *local = tile - seg * a.tiles_per_seg;
+  } else {
+    seg = 0;
+    uint32_t start = 0;
+#pragma unroll
+    for (int k = 0; k < kMaxSegments - 1; ++k) {
+      const uint32_t e = a.tile_end[k];
+      seg = tile >= e ? (uint32_t)(k + 1) : seg;
+      start = tile >= e ? e : start;
+    }
+    *local = tile - start;
+  }
+  return seg;
+}
+
+// EQUAL: as for the boxes -- segments of equal tile count, blockIdx.y the segment, blockIdx.x the tile.
+template<int U, bool EQUAL>
 __global__ __launch_bounds__(kBlock) void copy_flat_kernel(FlatArgs a) {
   constexpr uint32_t tile_bytes = kBlock * U * 16;
   const uint32_t lane_byte = threadIdx.x * 16;
-  for (uint32_t tile = blockIdx.x; tile < a.total_tiles; tile += gridDim.x) {
-    uint32_t seg, local;
-    if (a.tiles_per_seg) {
-      seg = tile / a.tiles_per_seg;
-      local = tile - seg * a.tiles_per_seg;
-    } else {
-      seg = 0;
-      uint32_t start = 0;
-#pragma unroll
-      for (int k = 0; k < kMaxSegments - 1; ++k) {
-        const uint32_t e = a.tile_end[k];
-        seg = tile >= e ? (uint32_t)(k + 1) : seg;
-        start = tile >= e ? e : start;
-      }
-      local = tile - start;
-    }
+  uint32_t tile = blockIdx.x; // first tile untested, as in the box kernels
+  do {
+    uint32_t local;
+    const uint32_t seg = EQUAL ? (local = blockIdx.x, blockIdx.y) : locate_segment(a, tile, &local);
     const uint64_t off = (uint64_t)local * tile_bytes;
     const uint64_t left = a.bytes[seg] - off;
     const uint32_t n = left < tile_bytes ? (uint32_t)left : tile_bytes;
@@ -259,7 +293,11 @@ __global__ __launch_bounds__(kBlock) void copy_flat_kernel(FlatArgs a) {
     for (int u = 0; u < U; ++u) {
       tile_store(rd, lane_byte + (uint32_t)u * (kBlock * 16), v[u]);
     }
-  }
+    if (EQUAL) {
+      break;
+    }
+    tile += gridDim.x;
+  } while (tile < a.total_tiles);
 }
 
 // ---- host side: reduce a box to the kernel's form ----
@@ -289,6 +327,8 @@ struct Step {
   int vec;    // kBoxes: bytes per vector
   int unroll; // sub-tiles
   uint32_t grid;
+  uint32_t grid_y; // > 0: the two-dimensional form for equal boxes / segments (grid x grid_y workgroups)
+  bool sparse_source; // kBoxes16: the source rows are not adjacent in memory (plain instead of nt loads)
   size_t lds;
   FlatArgs flat;   // kFlat
   CopyArgs boxes;  // kBoxes16, kBoxes
@@ -317,6 +357,7 @@ struct Launcher {
   // with a padded row pitch; at 64 MiB and below a cap gains nothing or costs.
   static constexpr uint64_t kLongCopyBytes = (uint64_t)128 << 20;
   size_t lds = 0; // of the launch being assembled
+  bool sparse_source = false;
 
   void choose_cap(uint64_t bytes) {
     int cap = tuning().copy_wg_per_cu;
@@ -374,7 +415,11 @@ struct Launcher {
         grid = (uint32_t)t.copy_max_blocks;
       }
       Step st;
-      st.kind = Step::kFlat, st.vec = 16, st.unroll = U, st.grid = grid, st.lds = lds;
+      st.kind = Step::kFlat, st.vec = 16, st.unroll = U, st.grid = grid, st.grid_y = 0, st.lds = lds;
+      st.sparse_source = false;
+      if (a.tiles_per_seg && grid == a.total_tiles && a.nsegs > 1) {
+        st.grid = a.tiles_per_seg, st.grid_y = a.nsegs;
+      }
       submit(st, &a, nullptr);
     }
     flat.clear();
@@ -408,7 +453,11 @@ struct Launcher {
     }
     Step st;
     st.kind = buffer16 ? Step::kBoxes16 : Step::kBoxes;
-    st.vec = vec, st.unroll = unroll, st.grid = grid, st.lds = buffer16 ? lds : 0;
+    st.vec = vec, st.unroll = unroll, st.grid = grid, st.grid_y = 0, st.lds = buffer16 ? lds : 0;
+    st.sparse_source = sparse_source;
+    if (buffer16 && a.tiles_per_box && grid == a.total_tiles) {
+      st.grid = a.tiles_per_box, st.grid_y = a.nboxes;
+    }
     submit(st, nullptr, &a);
   }
 
@@ -419,6 +468,13 @@ struct Launcher {
       all_vectors += (uint64_t)d.rows * d.cols;
     }
     choose_cap(lg == 5 ? all_vectors * 16 : 0); // the 16-byte buffer kernel only
+    sparse_source = false;
+    for (const BoxDesc& d : list) {
+      sparse_source = sparse_source || (d.rows > 1 && d.src_stride[0] != (int64_t)d.cols * 16);
+    }
+    if (tuning().box_policy) {
+      sparse_source = tuning().box_policy == 1;
+    }
     // strided boxes: two sub-tiles measured best on large gathers (6.1 against 5.9 TB/s with four)
     const int U = tuning().box_unroll ? tuning().box_unroll : auto_unroll(all_vectors, 2);
     unroll = U;
@@ -681,40 +737,53 @@ void launch_boxes_vec(const Step& st, const CopyArgs& a, hipStream_t stream) {
 }
 
 int launch_step(const Step& st, const FlatArgs* flat, const CopyArgs* boxes, hipStream_t stream) {
-  dim3 g(st.grid), b(kBlock);
+  const bool equal = st.grid_y > 0;
+  dim3 g(st.grid, equal ? st.grid_y : 1), b(kBlock);
+#define MDH_COMMA ,
+#define MDH_LAUNCH_COPY(kernel, more, args)                                                  \
+  switch (st.unroll) {                                                                 \
+  case 1:                                                                              \
+    if (equal) {                                                                       \
+      hipLaunchKernelGGL((kernel<1, true more>), g, b, st.lds, stream, args);               \
+    } else {                                                                           \
+      hipLaunchKernelGGL((kernel<1, false more>), g, b, st.lds, stream, args);              \
+    }                                                                                  \
+    break;                                                                             \
+  case 2:                                                                              \
+    if (equal) {                                                                       \
+      hipLaunchKernelGGL((kernel<2, true more>), g, b, st.lds, stream, args);               \
+    } else {                                                                           \
+      hipLaunchKernelGGL((kernel<2, false more>), g, b, st.lds, stream, args);              \
+    }                                                                                  \
+    break;                                                                             \
+  case 4:                                                                              \
+    if (equal) {                                                                       \
+      hipLaunchKernelGGL((kernel<4, true more>), g, b, st.lds, stream, args);               \
+    } else {                                                                           \
+      hipLaunchKernelGGL((kernel<4, false more>), g, b, st.lds, stream, args);              \
+    }                                                                                  \
+    break;                                                                             \
+  default:                                                                             \
+    if (equal) {                                                                       \
+      hipLaunchKernelGGL((kernel<8, true more>), g, b, st.lds, stream, args);               \
+    } else {                                                                           \
+      hipLaunchKernelGGL((kernel<8, false more>), g, b, st.lds, stream, args);              \
+    }                                                                                  \
+    break;                                                                             \
+  }
   switch (st.kind) {
   case Step::kFlat:
-    switch (st.unroll) {
-    case 1:
-      hipLaunchKernelGGL((copy_flat_kernel<1>), g, b, st.lds, stream, *flat);
-      break;
-    case 2:
-      hipLaunchKernelGGL((copy_flat_kernel<2>), g, b, st.lds, stream, *flat);
-      break;
-    case 4:
-      hipLaunchKernelGGL((copy_flat_kernel<4>), g, b, st.lds, stream, *flat);
-      break;
-    default:
-      hipLaunchKernelGGL((copy_flat_kernel<8>), g, b, st.lds, stream, *flat);
-      break;
-    }
+    MDH_LAUNCH_COPY(copy_flat_kernel, , *flat)
     return check_launch("copy_flat_kernel");
   case Step::kBoxes16:
-    switch (st.unroll) {
-    case 1:
-      hipLaunchKernelGGL((copy_boxes16_kernel<1>), g, b, st.lds, stream, *boxes);
-      break;
-    case 2:
-      hipLaunchKernelGGL((copy_boxes16_kernel<2>), g, b, st.lds, stream, *boxes);
-      break;
-    case 4:
-      hipLaunchKernelGGL((copy_boxes16_kernel<4>), g, b, st.lds, stream, *boxes);
-      break;
-    default:
-      hipLaunchKernelGGL((copy_boxes16_kernel<8>), g, b, st.lds, stream, *boxes);
-      break;
+    if (st.sparse_source) {
+      MDH_LAUNCH_COPY(copy_boxes16_kernel, MDH_COMMA true, *boxes)
+    } else {
+      MDH_LAUNCH_COPY(copy_boxes16_kernel, MDH_COMMA false, *boxes)
     }
     return check_launch("copy_boxes16_kernel");
+#undef MDH_LAUNCH_COPY
+#undef MDH_COMMA
   default:
     switch (st.vec) {
     case 16:
@@ -892,6 +961,188 @@ extern "C" int mdh_copy_plan_create(const mdh_box* boxes, const int32_t* src_slo
     }
   }
   *plan = p.release();
+  return MDH_OK;
+}
+
+// Host-side replay of a plan's kernels: every tile and every slot goes through the same index
+// functions the device code uses, against made-up bases of the given sizes.
+extern "C" int mdh_copy_plan_verify(const mdh_copy_plan* plan, const uint64_t* base_bytes, int nbases) {
+  using namespace mdh;
+  if (!plan || nbases != plan->nbases || (nbases > 0 && !base_bytes)) {
+    set_error("mdh_copy_plan_verify: the plan takes %d bases", plan ? plan->nbases : 0);
+    return MDH_EINVAL;
+  }
+  for (int i = 0; i < nbases; ++i) {
+    if (base_bytes[i] > ((uint64_t)1 << 31)) {
+      set_error("mdh_copy_plan_verify: base %d is larger than the 2 GiB this check walks byte by byte", i);
+      return MDH_EINVAL;
+    }
+  }
+  // For every destination byte: 1 + (source slot << 40 | source byte), 0 = not written.
+  std::vector<std::vector<uint64_t>> expect((size_t)nbases), got((size_t)nbases);
+  auto dest = [&](std::vector<std::vector<uint64_t>>& m, int slot) -> std::vector<uint64_t>& {
+    if (m[(size_t)slot].empty()) {
+      m[(size_t)slot].assign((size_t)base_bytes[slot], 0);
+    }
+    return m[(size_t)slot];
+  };
+  // what the boxes say, element by element
+  for (size_t i = 0; i < plan->boxes.size(); ++i) {
+    const mdh_box& b = plan->boxes[i];
+    const int ss = plan->src_slot[i], ds = plan->dst_slot[i];
+    int64_t idx[MDH_MAX_DIMS] = {0};
+    int64_t numel = 1;
+    for (int d = 0; d < b.ndim; ++d) {
+      numel *= b.shape[d];
+    }
+    std::vector<uint64_t>& m = dest(expect, ds);
+    for (int64_t e = 0; e < numel; ++e) {
+      uint64_t so = (uint64_t)(uintptr_t)b.src, dof = (uint64_t)(uintptr_t)b.dst;
+      for (int d = 0; d < b.ndim; ++d) {
+        so += (uint64_t)(idx[d] * b.src_strides[d]) * (uint64_t)plan->itemsize;
+        dof += (uint64_t)(idx[d] * b.dst_strides[d]) * (uint64_t)plan->itemsize;
+      }
+      if (so + (uint64_t)plan->itemsize > base_bytes[ss] || dof + (uint64_t)plan->itemsize > base_bytes[ds]) {
+        set_error("mdh_copy_plan_verify: box %zu itself reaches outside its bases", i);
+        return MDH_EINVAL;
+      }
+      for (int k = 0; k < plan->itemsize; ++k) {
+        if (m[dof + k]) {
+          set_error("mdh_copy_plan_verify: the boxes overlap in base %d at byte %llu", ds, (unsigned long long)(dof + k));
+          return MDH_EINVAL;
+        }
+        m[dof + k] = 1 + (((uint64_t)ss << 40) | (so + k));
+      }
+      for (int d = b.ndim - 1; d >= 0; --d) {
+        if (++idx[d] < b.shape[d]) {
+          break;
+        }
+        idx[d] = 0;
+      }
+    }
+  }
+  // what the kernels would do
+  auto split = [](const void* fake, int* slot, uint64_t* off) {
+    const uint64_t v = (uint64_t)(uintptr_t)fake;
+    *slot = (int)(v >> kSlotShift) - 1;
+    *off = v & kOffsetMask;
+  };
+  auto move = [&](int ss, uint64_t so, int ds, uint64_t dof, uint32_t n, size_t step) -> bool {
+    if (ss < 0 || ss >= nbases || ds < 0 || ds >= nbases || so + n > base_bytes[ss] || dof + n > base_bytes[ds]) {
+      set_error("mdh_copy_plan_verify: step %zu moves %u bytes from base %d + %llu to base %d + %llu: outside the bases", step, n,
+          ss, (unsigned long long)so, ds, (unsigned long long)dof);
+      return false;
+    }
+    std::vector<uint64_t>& m = dest(got, ds);
+    for (uint32_t k = 0; k < n; ++k) {
+      if (m[dof + k]) {
+        set_error("mdh_copy_plan_verify: step %zu writes base %d byte %llu a second time", step, ds, (unsigned long long)(dof + k));
+        return false;
+      }
+      m[dof + k] = 1 + (((uint64_t)ss << 40) | (so + k));
+    }
+    return true;
+  };
+  for (size_t s = 0; s < plan->steps.size(); ++s) {
+    const Step& st = plan->steps[s];
+    // every workgroup takes its first tile untested: the grid must not exceed the tile count
+    const uint32_t step_tiles = st.kind == Step::kFlat ? st.flat.total_tiles : st.boxes.total_tiles;
+    if (st.grid == 0 || st.grid > step_tiles) {
+      set_error("mdh_copy_plan_verify: step %zu has a grid of %u workgroups for %u tiles", s, st.grid, step_tiles);
+      return MDH_EINVAL;
+    }
+    if (st.grid_y) {
+      // two-dimensional form: workgroup (x, y) takes tile x of entry y and no other
+      const uint32_t per = st.kind == Step::kFlat ? st.flat.tiles_per_seg : st.boxes.tiles_per_box;
+      const uint32_t n = st.kind == Step::kFlat ? st.flat.nsegs : st.boxes.nboxes;
+      if (st.kind == Step::kBoxes || per == 0 || st.grid != per || st.grid_y != n || (uint64_t)per * n != step_tiles) {
+        set_error("mdh_copy_plan_verify: step %zu: a %u x %u grid does not match %u entries of %u tiles", s, st.grid,
+            st.grid_y, n, per);
+        return MDH_EINVAL;
+      }
+    }
+    if (st.kind == Step::kFlat) {
+      const FlatArgs& a = st.flat;
+      const uint32_t tile_bytes = (uint32_t)kBlock * (uint32_t)st.unroll * 16u;
+      for (uint32_t tile = 0; tile < a.total_tiles; ++tile) {
+        uint32_t local;
+        const uint32_t seg = locate_segment(a, tile, &local);
+        if (seg >= a.nsegs) {
+          set_error("mdh_copy_plan_verify: step %zu tile %u lands in segment %u of %u", s, tile, seg, a.nsegs);
+          return MDH_EINVAL;
+        }
+        const uint64_t off = (uint64_t)local * tile_bytes;
+        if (off >= a.bytes[seg]) {
+          set_error("mdh_copy_plan_verify: step %zu tile %u starts past the end of its segment", s, tile);
+          return MDH_EINVAL;
+        }
+        const uint64_t left = a.bytes[seg] - off;
+        const uint32_t n = left < tile_bytes ? (uint32_t)left : tile_bytes;
+        int ss, ds;
+        uint64_t so, dof;
+        split(a.src[seg], &ss, &so);
+        split(a.dst[seg], &ds, &dof);
+        if (!move(ss, so + off, ds, dof + off, n, s)) {
+          return MDH_EINVAL;
+        }
+      }
+      continue;
+    }
+    const CopyArgs& a = st.boxes;
+    const uint32_t slots = (uint32_t)kBlock * (uint32_t)st.unroll;
+    uint32_t log2slots = 0;
+    while ((1u << log2slots) < slots) {
+      ++log2slots;
+    }
+    const bool buffer16 = st.kind == Step::kBoxes16;
+    for (uint32_t tile = 0; tile < a.total_tiles; ++tile) {
+      const TileLoc t = buffer16 ? locate_tile<true>(a, tile) : locate_tile<false>(a, tile);
+      if (t.box >= a.nboxes) {
+        set_error("mdh_copy_plan_verify: step %zu tile %u lands in box %u of %u", s, tile, t.box, a.nboxes);
+        return MDH_EINVAL;
+      }
+      const BoxDesc& B = a.box[t.box];
+      int ss, ds;
+      uint64_t sbase, dbase;
+      split(B.src, &ss, &sbase);
+      split(B.dst, &ds, &dbase);
+      for (uint32_t slot = 0; slot < slots; ++slot) {
+        uint64_t so, dof;
+        if (buffer16) {
+          uint32_t so32, dof32;
+          if (!slot_offsets<uint32_t>(B, t, slot, log2slots, 16u, &so32, &dof32)) {
+            continue; // the kernel gives this slot the offset just past the descriptor
+          }
+          // an access the descriptor would clip is an access the kernel silently loses
+          if ((uint64_t)so32 + 16 > B.src_span || (uint64_t)dof32 + 16 > B.dst_span) {
+            set_error("mdh_copy_plan_verify: step %zu box %u: a vector lies outside the box's own descriptor", s, t.box);
+            return MDH_EINVAL;
+          }
+          so = so32, dof = dof32;
+        } else {
+          int64_t so64, dof64;
+          if (!slot_offsets<int64_t>(B, t, slot, log2slots, (uint32_t)st.vec, &so64, &dof64)) {
+            continue;
+          }
+          so = (uint64_t)so64, dof = (uint64_t)dof64;
+        }
+        if (!move(ss, sbase + so, ds, dbase + dof, buffer16 ? 16u : (uint32_t)st.vec, s)) {
+          return MDH_EINVAL;
+        }
+      }
+    }
+  }
+  for (int b = 0; b < nbases; ++b) {
+    const std::vector<uint64_t>&e = expect[(size_t)b], &g = got[(size_t)b];
+    for (size_t i = 0; i < (size_t)base_bytes[b]; ++i) {
+      const uint64_t x = e.empty() ? 0 : e[i], y = g.empty() ? 0 : g[i];
+      if (x != y) {
+        set_error("mdh_copy_plan_verify: base %d byte %zu: the boxes ask for source %llx, the kernels bring %llx", b, i,
+            (unsigned long long)x, (unsigned long long)y);
+        return MDH_EINVAL;
+      }
+    }
+  }
   return MDH_OK;
 }
 

@@ -64,12 +64,14 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t tile_rsrc(const void* base, ui
   return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, (int)bytes, 0x00020000);
 }
 
+template<int AUX = MDH_LOAD_AUX>
 __device__ __forceinline__ u32x4 tile_load(__amdgpu_buffer_rsrc_t rs, uint32_t byte_offset) {
-  return __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, (int)byte_offset, 0, MDH_LOAD_AUX));
+  return __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, (int)byte_offset, 0, AUX));
 }
 
+template<int AUX = MDH_STORE_AUX>
 __device__ __forceinline__ void tile_store(__amdgpu_buffer_rsrc_t rs, uint32_t byte_offset, u32x4 v) {
-  __builtin_amdgcn_raw_buffer_store_b128(v, rs, (int)byte_offset, 0, MDH_STORE_AUX);
+  __builtin_amdgcn_raw_buffer_store_b128(v, rs, (int)byte_offset, 0, AUX);
 }
 
 // ---- host side ----
@@ -88,6 +90,7 @@ struct Tuning {
   int box_unroll = 0;  // strided boxes
   int copy_max_blocks = 0;
   int copy_wg_per_cu = 0; // as reduce_wg_per_cu, for the copy kernels
+  int box_policy = 0;     // loads of the strided-box kernel: 0 by layout, 1 plain, 2 nt
 };
 Tuning& tuning();
 

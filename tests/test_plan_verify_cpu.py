@@ -1,0 +1,99 @@
+"""Prepared copy plans checked on the CPU: mdh_copy_plan_verify replays a plan's kernels on the
+host, tile by tile and slot by slot, through the same index functions the device code is compiled
+from, and compares every destination byte with what the boxes ask for.  The three compiled
+redistributions of the benchmark, the strided gather, ragged and awkward boxes, and random ones.
+No GPU: this is the bounds check of the kernels' indexing that runs before anything is launched.
+"""
+
+import numpy as np
+import pytest
+
+from moodist_amd import _abi as abi
+
+
+def plan_for(specs, itemsize):
+    """specs: (src bytes, src offset elems, dst offset elems, shape, src strides, dst strides); one source
+    base per box and one shared destination base (the last)."""
+    boxes = [abi.make_box(so * itemsize, do * itemsize, shape, sstr, dstr) for _, so, do, shape, sstr, dstr in specs]
+    n = len(specs)
+    return abi.CopyPlan(boxes, list(range(n)), [n] * n, itemsize, n + 1)
+
+
+def test_the_three_compiled_redistributions_of_the_benchmark():
+    # fp32 / bf16 8192 x 8192 row-sharded over 8 -> this rank's column block; [64,512,1024] bf16 dim0 -> dim2
+    for itemsize in (4, 2):
+        for k in (0, 3, 7):
+            specs = [(1024 * 8192 * itemsize, 1024 * k, s * 1024 * 1024, [1024, 1024], [8192, 1], [1024, 1])
+                     for s in range(8)]
+            p = plan_for(specs, itemsize)
+            assert p.launches == 1
+            p.verify([1024 * 8192 * itemsize] * 8 + [8192 * 1024 * itemsize])
+    for k in (0, 5):
+        specs = [(8 * 512 * 1024 * 2, 128 * k, s * 8 * 512 * 128, [8, 512, 128], [512 * 1024, 1024, 1], [512 * 128, 128, 1])
+                 for s in range(8)]
+        p = plan_for(specs, 2)
+        assert p.launches == 1
+        p.verify([8 * 512 * 1024 * 2] * 8 + [64 * 512 * 128 * 2])
+
+
+def test_strided_gather_and_dense_gather_shapes():
+    # [8, rows, cols] bf16 gather into a padded row pitch, scaled down 4x per side from the benchmark's
+    rows, cols, pad = 1024, 1024, 64
+    specs = [(rows * cols * 2, 0, s * rows * (cols + pad), [rows, cols], [cols, 1], [cols + pad, 1]) for s in range(8)]
+    plan_for(specs, 2).verify([rows * cols * 2] * 8 + [8 * rows * (cols + pad) * 2])
+    # dense: eight flat segments of unequal length (ragged last tiles, the scanned segment table)
+    lens = [100000, 65536, 16, 4096 * 3 + 16, 48, 1 << 20, 999984, 32]
+    at, specs = 0, []
+    for n in lens:
+        specs.append((n, 0, at, [n], [1], [1]))
+        at += n
+    plan_for(specs, 1).verify(lens + [at])
+
+
+@pytest.mark.parametrize("itemsize", [1, 2, 4, 8])
+def test_ragged_rows_transposes_and_many_dimensions(itemsize):
+    specs = [
+        (40 * 1000 * itemsize, 7, 11, [37, 1001], [1003, 1], [1004, 1]),          # rows not a multiple of 16 bytes
+        (5000 * itemsize, 3, 40000, [40, 50], [1, 60], [50, 1]),                   # transposing: one-element runs
+        (16 * itemsize, 5, 69999, [], [], []),                                     # a scalar
+        (9000 * itemsize, 0, 50000, [3, 4, 5, 6], [2000, 400, 60, 1], [130, 31, 6, 1]),  # four strided extents
+        (3000 * itemsize, 1, 60000, [2, 2, 2, 2, 2, 3], [1000, 500, 200, 90, 40, 1], [96, 48, 24, 12, 6, 1]),
+        (70000 * itemsize, 0, 62000, [17, 33], [37, 1], [33, 1]),                  # dense on one side only
+    ]
+    sizes = [s[0] + 64 for s in specs] + [80000 * itemsize]
+    plan_for(specs, itemsize).verify(sizes)
+
+
+def test_random_boxes():
+    rng = np.random.RandomState(11)
+    for trial in range(60):
+        itemsize = int(rng.choice([1, 2, 4, 8, 16]))
+        specs, sizes, dst_at = [], [], 0
+        for _ in range(int(rng.randint(1, 7))):
+            nd = int(rng.randint(1, 5))
+            shape = [int(rng.randint(1, 12)) for _ in range(nd)]
+            shape[-1] = int(rng.choice([1, 2, 5, 16, 64, 300]))
+            sstr, dstr = [1] * nd, [1] * nd
+            for d in range(nd - 2, -1, -1):
+                sstr[d] = sstr[d + 1] * shape[d + 1] + int(rng.randint(0, 4)) * (d == nd - 2)
+                dstr[d] = dstr[d + 1] * shape[d + 1] + int(rng.randint(0, 4)) * (d == nd - 2)
+            so = int(rng.randint(0, 9))
+            specs.append(((sstr[0] * shape[0] + so + 4) * itemsize, so, dst_at, shape, sstr, dstr))
+            dst_at += dstr[0] * shape[0] + int(rng.randint(0, 9))
+        plan_for(specs, itemsize).verify([s[0] for s in specs] + [(dst_at + 4) * itemsize])
+
+
+def test_the_verifier_notices_what_it_is_there_to_notice():
+    specs = [(4096, 0, 0, [16, 64], [64, 1], [64, 1])]
+    p = plan_for(specs, 4)
+    p.verify([4096, 4096])
+    with pytest.raises(abi.MoodistError, match="reaches outside its bases"):
+        p.verify([4095, 4096])  # source one byte short
+    with pytest.raises(abi.MoodistError, match="reaches outside its bases"):
+        p.verify([4096, 4000])
+    # overlapping destinations are a caller error the check reports
+    two = [(256, 0, 0, [64], [1], [1]), (256, 0, 32, [64], [1], [1])]
+    with pytest.raises(abi.MoodistError, match="boxes overlap"):
+        plan_for(two, 4).verify([256, 256, 1024])
+    with pytest.raises(abi.MoodistError, match="takes 2 bases"):
+        p.verify([4096])
