@@ -308,7 +308,11 @@ __global__ __launch_bounds__(kWave) void reduce_vec_kernel(ReduceArgs a) {
   constexpr uint64_t tile_bytes = (uint64_t)kWave * U * 16;
   const uint64_t body_bytes = a.nvec * 16;
   const uint64_t ntiles = (body_bytes + tile_bytes - 1) / tile_bytes;
-  for (uint64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+  // The grid never exceeds the tile count (a launch with no whole vector has one wave, whose
+  // descriptors are then empty), so the first tile needs no test and the scalar loads of the
+  // arguments are not held up behind a load-and-branch.
+  uint64_t tile = blockIdx.x;
+  do {
     const uint64_t tile_byte = tile * tile_bytes;
     const uint64_t left = body_bytes - tile_byte;
     const uint32_t n = (uint32_t)(left < tile_bytes ? left : tile_bytes);
@@ -317,7 +321,8 @@ __global__ __launch_bounds__(kWave) void reduce_vec_kernel(ReduceArgs a) {
     // fold, and a kernel's register budget is that of its hungriest path.  AVG is the plain
     // fold with one more multiply when the result is written (a wave-uniform test there).
     reduce_tile<T, F, U, CH, PREMUL ? kPremul : kPlain>(a, nsrc, tile_byte, n);
-  }
+    tile += gridDim.x;
+  } while (tile < ntiles);
   if (blockIdx.x == 0) {
     const uint64_t i = a.nvec * per_vec<T>() + threadIdx.x;
     if (i < a.numel) {
