@@ -23,9 +23,19 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 CLOCK_WARMUP_S = 0.3   # untimed launches before the first timed window
 TIMED_WINDOWS = 11     # windows of `steps` launches; the median window is reported
 INFINITY_CACHE_BYTES = 256 << 20
-# (65568.73 KiB x 1.99971 fetched + 16384.00 KiB x 1.00000 written) per launch of the fp32 P=8 reduction
-MEASURED_TRAFFIC_BYTES = {"reduce_fp32_p8": 151031143}
-
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch), each
+# scaled by what the same counter reads for the flat copy of exactly 256 MiB (FETCH_SIZE x 1.99983,
+# WRITE_SIZE x 1.00000): profiles/hbm_traffic_pmc_reduce_and_copy_kernels.md.  E.g. the headline:
+# 65,557.91 x 1.99983 + 16,384.00 KiB = 147,488.5 KiB.  Workloads without an entry were not measured.
+MEASURED_TRAFFIC_BYTES = {
+    "reduce_fp32_p8": 151028193,
+    "reduce_bf16_p16": 1141025530,
+    "reduce_fp32_p64_sum": 272661846,
+    "allgather_bf16_p8": 536870912,
+    "allgather_bf16_p8_strided": 536886266,
+    "redistribute_fp32_8192": 67155282,
+    "redistribute_bf16_3d": 16825499,
+}
 
 def build_workload(name, torch, abi, dev):
     """Returns (describe, algorithmic_bytes, launch(i), check(), kernel name) for a named workload.
@@ -227,6 +237,8 @@ def main():
     ap.add_argument("--workload", default="reduce_fp32_p8")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
+    ap.add_argument("--clock-warmup", type=float, default=CLOCK_WARMUP_S, metavar="SECONDS",
+                    help="untimed launches before the first timed window (0 under a counter-collecting profiler)")
     ap.add_argument("--tuning", action="append", default=[], metavar="KNOB=VALUE",
                     help="force a launch-shape knob of the kernel library (mdh_set_tuning), e.g. reduce_unroll=8")
     args = ap.parse_args()
@@ -257,7 +269,7 @@ def main():
     # wall time have passed.  These launches are not timed.
     clock_launches = 0
     t_warm = time.perf_counter()
-    while time.perf_counter() - t_warm < CLOCK_WARMUP_S:
+    while time.perf_counter() - t_warm < args.clock_warmup:
         for i in range(50):
             launch(clock_launches + i)
         clock_launches += 50
@@ -331,7 +343,7 @@ def main():
             "frac": round(gbs / HBM_PEAK_GBS, 4),
             "algorithmic_bytes_per_launch": alg_bytes,
             # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by the
-            # same counter's reading on a copy of known size (recorded for the headline workload only)
+            # same counter's reading on a copy of known size; null for a workload not measured
             "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
         },
     }
