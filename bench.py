@@ -312,6 +312,7 @@ def main():
     ms_per_step = ms / args.steps
     desc["timed_windows"] = TIMED_WINDOWS
     desc["window_ms_min_median_max"] = [round(min(window_ms), 5), round(ms, 5), round(max(window_ms), 5)]
+    desc["clock_warmup_s"] = args.clock_warmup
     desc["clock_warmup_launches"] = clock_launches
     if not args.no_check:
         check()
