@@ -180,6 +180,15 @@ int mdh_copy_plan_create(const mdh_box* boxes, const int32_t* src_slots, const i
 int mdh_copy_plan_launch(const mdh_copy_plan* plan, const void* const* bases, int nbases, void* stream);
 int mdh_copy_plan_launches(const mdh_copy_plan* plan);
 int mdh_copy_plan_verify(const mdh_copy_plan* plan, const uint64_t* base_bytes, int nbases);
+/*
+ * Introspection, no reference counterpart: the kernel-argument block and the launch shape
+ * that launch number `step` (0 .. mdh_copy_plan_launches-1) passes for these 16-byte aligned
+ * bases.  `*size` receives the block's size; `out` may be NULL to ask for the size only.
+ * Enqueues nothing.  For checks of what a stream capture recorded against what an eager
+ * launch passes.
+ */
+int mdh_copy_plan_step_arguments(const mdh_copy_plan* plan, const void* const* bases, int nbases, int step, void* out,
+    size_t capacity, size_t* size, uint32_t* grid_x, uint32_t* grid_y, uint32_t* block, uint32_t* lds);
 void mdh_copy_plan_destroy(mdh_copy_plan* plan);
 
 /*

@@ -14,6 +14,7 @@
 #include "device_common.h"
 
 #include <algorithm>
+#include <cstring>
 #include <memory>
 #include <vector>
 
@@ -1154,6 +1155,25 @@ extern "C" int mdh_copy_plan_launches(const mdh_copy_plan* plan) {
   return plan ? (int)plan->steps.size() : -1;
 }
 
+// Writes the caller's addresses into a copy of launch `s`'s argument block; `at` is the first
+// patch of that launch, the return value the first patch of the next.
+static size_t patch_step(const mdh_copy_plan& plan, size_t s, size_t at, const void* const* bases, mdh::FlatArgs* flat,
+    mdh::CopyArgs* boxes) {
+  for (; at < plan.patches.size() && plan.patches[at].step == s; ++at) {
+    const mdh::Patch& pa = plan.patches[at];
+    const char* src = (const char*)bases[pa.src_slot] + pa.src_off;
+    char* dst = (char*)bases[pa.dst_slot] + pa.dst_off;
+    if (flat) {
+      flat->src[pa.entry] = src;
+      flat->dst[pa.entry] = dst;
+    } else {
+      boxes->box[pa.entry].src = src;
+      boxes->box[pa.entry].dst = dst;
+    }
+  }
+  return at;
+}
+
 extern "C" int mdh_copy_plan_launch(const mdh_copy_plan* plan, const void* const* bases, int nbases, void* stream) {
   using namespace mdh;
   if (!plan || nbases != plan->nbases || (nbases > 0 && !bases)) {
@@ -1187,24 +1207,64 @@ extern "C" int mdh_copy_plan_launch(const mdh_copy_plan* plan, const void* const
     int rc;
     if (st.kind == Step::kFlat) {
       FlatArgs a = st.flat;
-      for (; at < plan->patches.size() && plan->patches[at].step == s; ++at) {
-        const Patch& pa = plan->patches[at];
-        a.src[pa.entry] = (const char*)bases[pa.src_slot] + pa.src_off;
-        a.dst[pa.entry] = (char*)bases[pa.dst_slot] + pa.dst_off;
-      }
+      at = patch_step(*plan, s, at, bases, &a, nullptr);
       rc = launch_step(st, &a, nullptr, (hipStream_t)stream);
     } else {
       CopyArgs a = st.boxes;
-      for (; at < plan->patches.size() && plan->patches[at].step == s; ++at) {
-        const Patch& pa = plan->patches[at];
-        a.box[pa.entry].src = (const char*)bases[pa.src_slot] + pa.src_off;
-        a.box[pa.entry].dst = (char*)bases[pa.dst_slot] + pa.dst_off;
-      }
+      at = patch_step(*plan, s, at, bases, nullptr, &a);
       rc = launch_step(st, nullptr, &a, (hipStream_t)stream);
     }
     if (rc != MDH_OK) {
       return rc;
     }
+  }
+  return MDH_OK;
+}
+
+extern "C" int mdh_copy_plan_step_arguments(const mdh_copy_plan* plan, const void* const* bases, int nbases, int step,
+    void* out, size_t capacity, size_t* size, uint32_t* grid_x, uint32_t* grid_y, uint32_t* block, uint32_t* lds) {
+  using namespace mdh;
+  if (!plan || nbases != plan->nbases || (nbases > 0 && !bases) || step < 0 || (size_t)step >= plan->steps.size() ||
+      !size) {
+    set_error("mdh_copy_plan_step_arguments: bad plan, base table or launch number");
+    return MDH_EINVAL;
+  }
+  for (int i = 0; i < nbases; ++i) {
+    if ((uintptr_t)bases[i] & 15) {
+      set_error("mdh_copy_plan_step_arguments: base %d is not 16-byte aligned (such a call is not served from the "
+                "prepared launches)", i);
+      return MDH_EINVAL;
+    }
+  }
+  const Step& st = plan->steps[(size_t)step];
+  size_t at = 0;
+  while (at < plan->patches.size() && plan->patches[at].step < (size_t)step) {
+    ++at;
+  }
+  FlatArgs flat;
+  CopyArgs boxes;
+  const void* from;
+  if (st.kind == Step::kFlat) {
+    flat = st.flat;
+    patch_step(*plan, (size_t)step, at, bases, &flat, nullptr);
+    from = &flat;
+    *size = sizeof(FlatArgs);
+  } else {
+    boxes = st.boxes;
+    patch_step(*plan, (size_t)step, at, bases, nullptr, &boxes);
+    from = &boxes;
+    *size = sizeof(CopyArgs);
+  }
+  if (grid_x) *grid_x = st.grid;
+  if (grid_y) *grid_y = st.grid_y > 0 ? st.grid_y : 1;
+  if (block) *block = (uint32_t)kBlock;
+  if (lds) *lds = (uint32_t)st.lds;
+  if (out) {
+    if (capacity < *size) {
+      set_error("mdh_copy_plan_step_arguments: the block is %zu bytes", *size);
+      return MDH_EINVAL;
+    }
+    std::memcpy(out, from, *size);
   }
   return MDH_OK;
 }

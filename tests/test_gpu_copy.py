@@ -443,3 +443,18 @@ def test_host_cost_of_a_compiled_redistribution_from_cpp(dev):
     for general, prepared in rows:
         assert float(prepared) < float(general)
         assert float(prepared) < 10.0
+
+
+def test_a_stream_capture_records_the_launches_an_eager_call_passes(dev):
+    # Host-side reading of a captured graph's kernel nodes (grid, block, LDS, argument bytes)
+    # against mdh_copy_plan_step_arguments; the graph is destroyed without being instantiated,
+    # so nothing is replayed.
+    import subprocess
+
+    exe = os.path.join(ROOT, "tests", "native", "capture_probe.bin")
+    if not os.path.exists(exe):
+        pytest.skip("tests/native/capture_probe.bin is not built (run __graft_entry__.build())")
+    r = subprocess.run([exe, abi.LIB_PATH], capture_output=True, text=True, timeout=120)
+    print(r.stdout)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    assert r.stdout.count(": same") == 5 and "DIFFERENT" not in r.stdout
