@@ -104,6 +104,22 @@ int moodist_pg_reduce_scatter(moodist_pg* pg, const moodist_tensor* output, cons
  * elements, same dtype), or NULL when numel divides evenly. */
 int moodist_pg_allreduce(moodist_pg* pg, const moodist_tensor* tensor, const moodist_tensor* scratch, int reduce_op,
     void* stream, float premul_value, moodist_work** work);
+/* No counterpart in the reference.  moodist_pg_allreduce for callers that cannot allocate
+ * device memory and have no temporary to pass (code under stream capture, tight serving
+ * loops, harnesses that forbid hipMalloc): the padded temporary is this rank's slice of the
+ * kernel library's fixed workspace (mdh_static_workspace in moodist_hip.h, 64 MiB per GPU,
+ * split evenly over the group's ranks and rounded down to 256 bytes).  Allocates and frees no
+ * device memory.  Same results as moodist_pg_allreduce.  Limits:
+ *  - roundup(numel, size) * itemsize must fit the rank's slice (8 MiB for 8 ranks), else error;
+ *  - a rank's next call is refused while its previous one still waits for other ranks;
+ *  - all calls on one GPU share the workspace: a rank's calls must be ordered on the GPU (one
+ *    stream, or the caller's own events), and two worlds on one GPU must not use it at the
+ *    same time -- calls that overlap race;
+ *  - the padding elements hold what the last call left there; they are reduced and thrown
+ *    away, nothing needs to start at zero.
+ * When numel is a multiple of the group size no temporary is used at all. */
+int moodist_pg_allreduce_static(moodist_pg* pg, const moodist_tensor* tensor, int reduce_op, void* stream,
+    float premul_value, moodist_work** work);
 /* No counterpart in the reference, where a peer's contribution is whatever that peer's own
  * collective call passes: posts this rank's input for the next collective without asking
  * for an output.  kind: 0 = all_gather, 1 = reduce_scatter. */

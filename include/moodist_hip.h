@@ -192,6 +192,18 @@ int mdh_copy_plan_step_arguments(const mdh_copy_plan* plan, const void* const* b
 void mdh_copy_plan_destroy(mdh_copy_plan* plan);
 
 /*
+ * Set-up call of the library's fixed workspace, no reference counterpart: a device array of
+ * MDH_STATIC_WORKSPACE_BYTES that belongs to the library (every GPU the library runs on
+ * holds one from the moment the library's code is loaded there until the process ends).
+ * Returns the array's address on the CURRENT device and its size; the first call on a
+ * device looks the address up (hipGetSymbolAddress), later calls return the kept value.
+ * Allocates nothing.  The memory keeps whatever its last user left in it, and all users on
+ * one GPU share it: moodist_pg_allreduce_static (moodist_core.h) is the one user.
+ */
+#define MDH_STATIC_WORKSPACE_BYTES (64u << 20)
+int mdh_static_workspace(void** address, size_t* bytes);
+
+/*
  * Launch-shape knobs, for measurement; 0 (the default) lets the library choose
  * by size.  Names: "reduce_unroll" (KiB of every source per tile: 1, 2, 4, 8, 16),
  * "reduce_chunk" (sources whose loads are in flight together: 1, 2, 4, 8; the pairs

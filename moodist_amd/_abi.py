@@ -21,7 +21,7 @@ ABI_VERSION = 2
 SYMBOLS = (
     "mdh_abi_version", "mdh_error_string", "mdh_last_error", "mdh_reduce", "mdh_gather", "mdh_copy_boxes",
     "mdh_set_tuning", "mdh_get_tuning", "mdh_copy_plan_create", "mdh_copy_plan_launch", "mdh_copy_plan_launches",
-    "mdh_copy_plan_verify", "mdh_copy_plan_destroy", "mdh_copy_plan_step_arguments",
+    "mdh_copy_plan_verify", "mdh_copy_plan_destroy", "mdh_copy_plan_step_arguments", "mdh_static_workspace",
 )
 
 

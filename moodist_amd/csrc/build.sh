@@ -15,7 +15,7 @@ bdir="$here/build"
 mkdir -p "$bdir"
 cmds=()
 objs=()
-for f in abi copy reduce; do
+for f in abi copy reduce workspace; do
   o="$bdir/$f$tag.o"
   objs+=("$o")
   cmds+=("/opt/rocm/bin/hipcc ${flags[*]} -c $here/kernels/$f.hip -o $o")

@@ -155,6 +155,16 @@ int moodist_pg_allreduce(moodist_pg* pg, const moodist_tensor* tensor, const moo
   });
 }
 
+int moodist_pg_allreduce_static(moodist_pg* pg, const moodist_tensor* tensor, int reduce_op, void* stream,
+    float premul_value, moodist_work** work) {
+  return guarded([&] {
+    if (!tensor) {
+      throw std::runtime_error("moodist: null tensor");
+    }
+    give(work, as_pg(pg)->allreduce_static(*tensor, reduce_op, stream, premul_value));
+  });
+}
+
 int moodist_pg_stage_input(moodist_pg* pg, int kind, const moodist_tensor* input, int reduce_op, void* stream,
     float premul_value, moodist_work** work) {
   return guarded([&] {

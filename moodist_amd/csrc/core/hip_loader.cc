@@ -82,6 +82,7 @@ HipRuntime load() {
   resolve(kl, kn, "mdh_copy_plan_create", r.copy_plan_create);
   resolve(kl, kn, "mdh_copy_plan_launch", r.copy_plan_launch);
   resolve(kl, kn, "mdh_copy_plan_destroy", r.copy_plan_destroy);
+  resolve(kl, kn, "mdh_static_workspace", r.static_workspace);
   if (r.abi_version() != MDH_ABI_VERSION) {
     throw std::runtime_error("moodist: libmoodist_hip.so has ABI version " + std::to_string(r.abi_version()) +
                              ", this core expects " + std::to_string(MDH_ABI_VERSION));

@@ -42,6 +42,7 @@ struct HipRuntime {
   decltype(&mdh_copy_plan_create) copy_plan_create;
   decltype(&mdh_copy_plan_launch) copy_plan_launch;
   decltype(&mdh_copy_plan_destroy) copy_plan_destroy;
+  decltype(&mdh_static_workspace) static_workspace;
 };
 
 constexpr int kHipMemcpyDeviceToDevice = 3;

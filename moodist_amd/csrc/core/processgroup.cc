@@ -344,6 +344,55 @@ std::shared_ptr<Collective> ProcessGroup::allreduce(const moodist_tensor& tensor
   return all_gather_impl(&whole, chunk, stream, &tensor, std::move(keep));
 }
 
+std::shared_ptr<Collective> ProcessGroup::allreduce_static(const moodist_tensor& tensor, int reduce_op, void* stream,
+    float premul, Keep keep) {
+  check_device_tensor(tensor, world->device, "allreduce tensor");
+  MD_CHECK(tensor.numel > 0);
+  if (tensor.numel % size == 0) {
+    return allreduce(tensor, nullptr, reduce_op, stream, premul, std::move(keep)); // in place, no temporary
+  }
+  const HipRuntime& h = hip();
+  // the workspace's address is per device: ask with the group's device current
+  int current = -1;
+  check_hip(h.GetDevice(&current), "hipGetDevice");
+  if (current != world->device) {
+    check_hip(h.SetDevice(world->device), "hipSetDevice");
+  }
+  void* base = nullptr;
+  size_t total = 0;
+  const int rc = h.static_workspace(&base, &total);
+  if (current != world->device) {
+    check_hip(h.SetDevice(current), "hipSetDevice");
+  }
+  check_mdh(rc);
+  // one slice per rank: every rank's temporary is alive at the same time
+  const size_t slice = total / (size_t)size / 256 * 256;
+  const size_t padded = ((size_t)tensor.numel + (size_t)size - 1) / (size_t)size * (size_t)size;
+  const size_t need = padded * (size_t)tensor.itemsize;
+  if (need > slice) {
+    throw std::runtime_error("moodist: allreduce_static needs " + std::to_string(need) +
+                             " bytes for its padded temporary, the fixed workspace gives each of the " +
+                             std::to_string(size) + " ranks " + std::to_string(slice) + " bytes (" +
+                             std::to_string(total) + " in all)");
+  }
+  // This call's copy into the slice is enqueued now; a previous call's kernels read the slice
+  // when ITS last rank posts.  Until then the slice is taken.
+  if (auto previous = static_user.lock()) {
+    if (!previous->launched && previous->error.empty()) {
+      throw std::runtime_error("moodist: allreduce_static: this rank's previous allreduce_static is still waiting "
+                               "for other ranks and holds the workspace");
+    }
+  }
+  moodist_tensor scratch = tensor;
+  scratch.data = (char*)base + (size_t)rank * slice;
+  scratch.numel = (int64_t)padded;
+  scratch.ndim = 1;
+  scratch.shape[0] = (int64_t)padded;
+  auto c = allreduce(tensor, &scratch, reduce_op, stream, premul, std::move(keep));
+  static_user = c;
+  return c;
+}
+
 std::shared_ptr<CompiledOp> ProcessGroup::compile_op_full(const Dims& shape, int dtype,
     const std::vector<SliceSpec>& inputs, const std::vector<SliceSpec>& outputs) {
   Busy guard(*this);

@@ -113,6 +113,10 @@ public:
       void* stream, float premul, Keep keep = {});
   std::shared_ptr<Collective> allreduce(const moodist_tensor& tensor, const moodist_tensor* scratch, int reduce_op,
       void* stream, float premul, Keep keep = {});
+  // allreduce whose padded temporary is this rank's slice of the kernel library's fixed
+  // workspace (mdh_static_workspace) instead of a tensor from the caller
+  std::shared_ptr<Collective> allreduce_static(const moodist_tensor& tensor, int reduce_op, void* stream, float premul,
+      Keep keep = {});
   std::shared_ptr<CompiledOp> compile_op_full(const Dims& shape, int dtype, const std::vector<SliceSpec>& inputs,
       const std::vector<SliceSpec>& outputs);
   std::shared_ptr<Collective> custom_op(const std::shared_ptr<CompiledOp>& op, const moodist_tensor* inputs,
@@ -133,6 +137,7 @@ private:
   // snapshot_inputs: replaces input.data by a copy made now on `stream`; the copy joins `keep`
   void snapshot(moodist_tensor& input, void* stream, Keep& keep);
   bool internal_input = false; // the second half of an allreduce: its input does not exist yet
+  std::weak_ptr<Collective> static_user; // the last collective that reads this rank's workspace slice
 
   // "Concurrent use of process group detected" guard (core/processgroup.cc:172-183)
   struct Busy {
