@@ -277,46 +277,77 @@ def main():
     # TIMED_WINDOWS windows of exactly `steps` launches each, every one bracketed by a
     # synchronize on both sides and by two HIP events on the launch stream; the reported step
     # time is the median window's (one window of 20 launches is 0.5 ms: a single one is noise).
-    window_ms, enqueue_ms, wall_ms = [], [], []
-    done = 0
-    blockers = None
-    if desc.get("queue_prefilled"):
-        # about 0.15 ms of unrelated GPU work per call; enough of them to outlast the host's
-        # enqueuing of one window (up to 12 us per launch)
-        blockers = [torch.empty(64 << 20, dtype=torch.float32, device=dev) for _ in range(3)]
-        n_blockers = 2 + int(args.steps * 12e-6 / 0.15e-3)
-    for w in range(TIMED_WINDOWS):
+    #
+    # Two kinds of window.  A plain one starts on an idle stream: the GPU waits for the host's
+    # first launch call (several microseconds), and that wait is part of the step time -- this is
+    # the job's throughput, `value`.  A pre-filled one is enqueued behind a spinning kernel, so
+    # that the launches are back to back when the first one starts: its step
+    # time is the kernel's own duration, what `roofline` is about and what a kernel trace shows.
+    # Launches shorter than the host's launch call (the compiled redistributions) would measure
+    # the host in a plain window: they get pre-filled windows only, and config.queue_prefilled
+    # says so.
+    # The work in front is a spin kernel that touches no memory (torch.cuda._sleep): a kernel
+    # that streams through HBM would leave the caches full of its dirty lines, and writing those
+    # back would be charged to the launches that follow.  Long enough to outlast the host's
+    # enqueuing of one window (up to 12 us per launch).
+    def spin_ms(cycles):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
-        if blockers is not None:
-            for _ in range(n_blockers):
-                torch.add(blockers[0], blockers[1], out=blockers[2])
-        e0 = torch.cuda.Event(enable_timing=True)
-        e1 = torch.cuda.Event(enable_timing=True)
-        t0 = time.perf_counter()
-        e0.record()  # on torch's current stream, the stream every launch above and below uses
-        for i in range(args.steps):
-            launch(done + i)
-        enqueue_ms.append((time.perf_counter() - t0) * 1e3)
+        e0.record()
+        torch.cuda._sleep(cycles)
         e1.record()
         torch.cuda.synchronize()
-        wall_ms.append((time.perf_counter() - t0) * 1e3)
-        window_ms.append(e0.elapsed_time(e1))
-        done += args.steps
+        return e0.elapsed_time(e1)
+
+    spin_ms(100_000)
+    cycles_per_ms = 4_000_000 / max(spin_ms(4_000_000), 1e-3)
+    spin_cycles = int(cycles_per_ms * (0.2 + args.steps * 12e-3))
+    desc["prefill_spin_ms"] = round(spin_cycles / cycles_per_ms, 3)
+    done = 0
 
     def median(v):
         v = sorted(v)
         return v[len(v) // 2]
 
-    ms = median(window_ms)
-    enqueue_ms, wall_ms = median(enqueue_ms), median(wall_ms)
-    ms_per_step = ms / args.steps
+    def timed_windows(prefilled):
+        nonlocal done
+        window_ms, enqueue_ms, wall_ms = [], [], []
+        for w in range(TIMED_WINDOWS):
+            torch.cuda.synchronize()
+            if prefilled:
+                torch.cuda._sleep(spin_cycles)
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            t0 = time.perf_counter()
+            e0.record()  # on torch's current stream, the stream every launch above and below uses
+            for i in range(args.steps):
+                launch(done + i)
+            enqueue_ms.append((time.perf_counter() - t0) * 1e3)
+            e1.record()
+            torch.cuda.synchronize()
+            wall_ms.append((time.perf_counter() - t0) * 1e3)
+            window_ms.append(e0.elapsed_time(e1))
+            done += args.steps
+        return window_ms, median(enqueue_ms), median(wall_ms)
+
+    prefilled_ms, enqueue_ms, wall_ms = timed_windows(True)
+    kernel_ms = median(prefilled_ms) / args.steps
     desc["timed_windows"] = TIMED_WINDOWS
+    if desc.get("queue_prefilled"):
+        window_ms = prefilled_ms
+    else:
+        window_ms, enqueue_ms, wall_ms = timed_windows(False)
+        desc["prefilled_window_ms_min_median_max"] = [round(min(prefilled_ms), 5), round(median(prefilled_ms), 5),
+                                                      round(max(prefilled_ms), 5)]
+    ms = median(window_ms)
+    ms_per_step = ms / args.steps
     desc["window_ms_min_median_max"] = [round(min(window_ms), 5), round(ms, 5), round(max(window_ms), 5)]
     desc["clock_warmup_s"] = args.clock_warmup
     desc["clock_warmup_launches"] = clock_launches
     if not args.no_check:
         check()
     gbs = alg_bytes / (ms_per_step * 1e-3) / 1e9
+    kernel_gbs = alg_bytes / (kernel_ms * 1e-3) / 1e9
     out = {
         "metric": "achieved HBM GB/s (% of peak) for 1-GPU local reduce-scatter, fp32 P=8"
         if args.workload == "reduce_fp32_p8" else "achieved HBM GB/s (% of peak), " + args.workload,
@@ -338,10 +369,12 @@ def main():
         "roofline": {
             "bound": "hbm",
             "kernel": kernel,
-            "achieved": round(gbs, 1),
+            # algorithmic bytes / the kernel's duration (back-to-back launches, pre-filled queue)
+            "achieved": round(kernel_gbs, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
-            "frac": round(gbs / HBM_PEAK_GBS, 4),
+            "frac": round(kernel_gbs / HBM_PEAK_GBS, 4),
+            "kernel_us": round(kernel_ms * 1e3, 3),
             "algorithmic_bytes_per_launch": alg_bytes,
             # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by the
             # same counter's reading on a copy of known size; null for a workload not measured
