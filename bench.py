@@ -7,6 +7,8 @@ before the timed region.  Prints one JSON line.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
                   [--tuning KNOB=VALUE ...]
+  NAME is one of the fixed workloads (the headline reduce_fp32_p8 by default) or, for size sweeps,
+  reduce:<fp32|bf16|fp16>:<sources>:<elements>[:<sum|avg|max>] and gather:<sources>:<bytes per shard>.
 """
 
 import argparse
@@ -37,17 +39,20 @@ MEASURED_TRAFFIC_BYTES = {
     "redistribute_bf16_3d": 16825499,
 }
 
-def build_workload(name, torch, abi, dev):
+def build_workload(name, torch, abi, dev, rotation_bytes):
     """Returns (describe, algorithmic_bytes, launch(i), check(), kernel name) for a named workload.
-    Every workload rotates over enough distinct buffer sets that their footprint exceeds twice
-    the 256 MB Infinity Cache, so no launch finds its operands cached by an earlier one."""
+    Every workload rotates over distinct buffer sets whose TOUCHED bytes add up to
+    rotation_bytes (default 4 GiB, sixteen times the 256 MB Infinity Cache), so that neither the
+    sources nor the outputs of a launch are still cached from an earlier one: a rotation of two
+    or three times the cache is not enough on this chip (see the measurement notes)."""
     L = abi.lib()
 
     def current():
         return torch.cuda.current_stream().cuda_stream
 
-    def nsets_for(set_bytes):
-        return max(2, -(-2 * INFINITY_CACHE_BYTES // set_bytes) + 1)
+    def nsets_for(touched_bytes):
+        # at most 512 sets: launches that touch less than 8 MiB rotate over less than 4 GiB
+        return min(512, max(2, -(-rotation_bytes // touched_bytes)))
 
     if name.startswith("reduce"):
         # reduce_fp32_p8 (headline), reduce_bf16_p16, reduce_fp32_p64_{sum,avg,max}
@@ -57,7 +62,17 @@ def build_workload(name, torch, abi, dev):
             "reduce_fp32_p64_sum": (64, 1048576, torch.float32, abi.DTYPE_FLOAT32, abi.OP_SUM, "rand", 1.0),
             "reduce_fp32_p64_avg": (64, 1048576, torch.float32, abi.DTYPE_FLOAT32, abi.OP_AVG, "rand", 1.0 / 64),
             "reduce_fp32_p64_max": (64, 1048576, torch.float32, abi.DTYPE_FLOAT32, abi.OP_MAX, "rand", 1.0),
-        }[name]
+        }.get(name)
+        if spec is None:
+            # reduce:<fp32|bf16|fp16>:<sources>:<elements>[:<sum|avg|max>] -- any size, for sweeps
+            parts = name.split(":")
+            if parts[0] != "reduce" or len(parts) not in (4, 5):
+                raise SystemExit("bench.py: unknown workload " + name)
+            tdt, code = {"fp32": (torch.float32, abi.DTYPE_FLOAT32), "bf16": (torch.bfloat16, abi.DTYPE_BFLOAT16),
+                         "fp16": (torch.float16, abi.DTYPE_FLOAT16)}[parts[1]]
+            P, N = int(parts[2]), int(parts[3])
+            op = {"sum": abi.OP_SUM, "avg": abi.OP_AVG, "max": abi.OP_MAX}[parts[4] if len(parts) == 5 else "sum"]
+            spec = (P, N, tdt, code, op, "rand", 1.0 / P if op == abi.OP_AVG else 1.0)
         P, N, tdt, code, op, dist, scale = spec
         isz = torch.empty(0, dtype=tdt).element_size()
         set_bytes = (P + 1) * N * isz
@@ -70,9 +85,10 @@ def build_workload(name, torch, abi, dev):
             elif dist == "randn1e-3":
                 x = (torch.randn(N) * 1e-3).to(tdt)
             else:
-                x = torch.rand(N) * 2 - 1
+                x = (torch.rand(N) * 2 - 1).to(tdt)
             base.append(x)
-        sets = [[b.to(dev) for b in base] for _ in range(nsets)]
+        on_device = [b.to(dev) for b in base]
+        sets = [on_device] + [[b.clone() for b in on_device] for _ in range(nsets - 1)]
         outs = [torch.empty(N, dtype=tdt, device=dev) for _ in range(nsets)]
         tabs = [abi.ptr_table([t.data_ptr() for t in s]) for s in sets]
 
@@ -100,6 +116,34 @@ def build_workload(name, torch, abi, dev):
                 "dtype": str(tdt).replace("torch.", ""), "fold_first": 0, "buffer_sets": nsets}
         return desc, set_bytes, launch, check, "reduce_vec_kernel"
 
+
+    if name.startswith("gather:"):
+        # gather:<sources>:<bytes per shard> -- dense assembly of any size, for sweeps
+        P, shard = (int(x) for x in name.split(":")[1:3])
+        set_bytes = 2 * P * shard
+        nsets = nsets_for(set_bytes)
+        g = torch.Generator().manual_seed(1)
+        base = [torch.randint(0, 256, (shard,), dtype=torch.uint8, generator=g) for _ in range(P)]
+        sets = [[b.to(dev) for b in base] for _ in range(nsets)]
+        outs = [torch.empty(P * shard, dtype=torch.uint8, device=dev) for _ in range(nsets)]
+        tabs = [abi.ptr_table([t.data_ptr() for t in s]) for s in sets]
+        out_ptrs = [o.data_ptr() for o in outs]
+
+        def launch(i):
+            k = i % nsets
+            rc = L.mdh_gather(tabs[k], P, out_ptrs[k], shard, 1, shard, shard, shard, current())
+            if rc:
+                abi.check(rc)
+
+        def check():
+            want = torch.cat(base)
+            for o in outs:
+                if not torch.equal(o.cpu(), want):
+                    raise SystemExit("bench: result differs from the expected gather")
+
+        desc = {"workload": name, "op": "all_gather_into_tensor chunk assembly", "sources": P, "shard_bytes": shard,
+                "dtype": "uint8", "buffer_sets": nsets}
+        return desc, set_bytes, launch, check, "copy_flat_kernel"
 
     if name == "allgather_bf16_p8" or name == "allgather_bf16_p8_strided":
         P, n = 8, 16777216
@@ -155,10 +199,12 @@ def build_workload(name, torch, abi, dev):
         for s in out_shape:
             out_numel *= s
         set_bytes = 2 * out_numel * isz
-        # the slabs are read only in part (this rank's columns), yet all of them must leave the cache
-        nsets = nsets_for(G.numel() * isz)
+        # the slabs are read only in part (this rank's columns): what counts for the caches is
+        # what a launch touches, not what the slabs occupy
+        nsets = nsets_for(set_bytes)
         k = 0  # this rank
-        sets = [[G[per * s:per * (s + 1)].contiguous().to(dev) for s in range(P)] for _ in range(nsets)]
+        on_device = [G[per * s:per * (s + 1)].contiguous().to(dev) for s in range(P)]
+        sets = [on_device] + [[t.clone() for t in on_device] for _ in range(nsets - 1)]
         outs = [torch.empty(out_shape, dtype=tdt, device=dev) for _ in range(nsets)]
         blk = out_numel // P
         # what a compiled custom op runs: the launches prepared once (mdh_copy_plan_create), every
@@ -235,6 +281,8 @@ def main():
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="reduce_fp32_p8")
+    ap.add_argument("--rotation-mib", type=int, default=4096,
+                    help="touched bytes of all buffer sets together (the launches rotate over them)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
     ap.add_argument("--clock-warmup", type=float, default=CLOCK_WARMUP_S, metavar="SECONDS",
@@ -257,7 +305,8 @@ def main():
     for item in args.tuning:  # before the workload is built: a prepared plan fixes its shape at create time
         knob, _, value = item.partition("=")
         abi.set_tuning(knob, int(value))
-    desc, alg_bytes, launch, check, kernel = build_workload(args.workload, torch, abi, dev)
+    desc, alg_bytes, launch, check, kernel = build_workload(args.workload, torch, abi, dev, args.rotation_mib << 20)
+    desc["rotation_mib"] = args.rotation_mib
     if args.tuning:
         desc["tuning"] = dict(item.split("=") for item in args.tuning)
 
@@ -360,7 +409,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": {"float32": "f32", "bfloat16": "bf16"}[desc["dtype"]],
+        "dtype": {"float32": "f32", "bfloat16": "bf16", "float16": "f16", "uint8": "u8"}[desc["dtype"]],
         "data": "synthetic",
         "config": desc,
         "percent_of_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),

@@ -208,12 +208,14 @@ int mdh_static_workspace(void** address, size_t* bytes);
  * by size.  Names: "reduce_unroll" (KiB of every source per tile: 1, 2, 4, 8, 16),
  * "reduce_chunk" (sources whose loads are in flight together: 1, 2, 4, 8; the pairs
  * compiled are 16x1, 16x2, 8x2, 4x4, 2x8, 1x8 and a call that forces another pair fails),
- * "reduce_max_blocks" (waves of the grid; 0 = chosen by size), "reduce_wg_per_cu" (2..8
+ * "reduce_max_blocks" (waves of the grid; 0 = chosen by size), "reduce_split_tiles" (tiles
+ * of one launch at most: longer reductions are cut into several launches; 0 = 4096),
+ * "reduce_wg_per_cu" (2..8
  * caps the workgroups resident on a CU, 9 = never cap), "copy_unroll" (1, 2,
  * 4, 8; contiguous segments), "box_unroll" (1, 2, 4, 8; strided boxes),
  * "copy_max_blocks", "copy_wg_per_cu" (2..8, 9 = never cap), "box_policy" (loads of the
- * strided-box kernel: 1 = plain, as chosen for sources whose rows are not adjacent, 2 = nt, as
- * chosen for densely read sources).  Returns MDH_EINVAL for an unknown name or value.
+ * strided-box kernel: 1 = plain, which pays when the sources are still in the Infinity Cache;
+ * 0 or 2 = nt, the default).  Returns MDH_EINVAL for an unknown name or value.
  * No counterpart in the reference, whose grid is fixed at 4/16/64 blocks
  * (core/kernels.cc:547-556).
  */

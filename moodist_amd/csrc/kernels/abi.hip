@@ -74,6 +74,9 @@ int* knob(const char* name) {
   if (!std::strcmp(name, "reduce_max_blocks")) {
     return &t.reduce_max_blocks;
   }
+  if (!std::strcmp(name, "reduce_split_tiles")) {
+    return &t.reduce_split_tiles;
+  }
   if (!std::strcmp(name, "reduce_wg_per_cu")) {
     return &t.reduce_wg_per_cu;
   }

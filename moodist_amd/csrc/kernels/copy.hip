@@ -185,18 +185,19 @@ __global__ __launch_bounds__(kBlock) void copy_boxes_kernel(CopyArgs a) {
 // all of its scalar loads go out in one batch; nothing of the table header is read.  On the
 // 16 MiB redistribution, whose whole launch lasts 5 us, that is 0.5 us.
 //
-// SPARSE selects the cache policy of the loads: plain when the source rows are not adjacent in
-// memory (a redistribution reads one block of columns out of every row), nt when the source is
-// read densely (a gather into a padded destination).  Stores are nt+sc1 either way.  Measured
-// on MI355X, us per launch (loads plain / nt):
-//   [64,512,1024] bf16 dim0->dim2, 16 MiB moved    3.92 /  4.60      8192^2 bf16, 32 MiB    6.92 /  7.79
-//   8192^2 fp32, 64 MiB                           10.91 / 12.85      16384^2 fp32, 256 MiB  40.85 / 44.61
-//   gather 8 x [4096,4096] bf16 into pitch 4160   85.25 / 81.63      8 x [1024,4096]        24.28 / 23.38
-// (with sc1 stores and nt loads, the former policy, the first four took 4.49 / 7.52 / 11.93 / 44.6
-// and the gather 83.9.)
-template<int U, bool EQUAL, bool SPARSE>
+// PLAIN selects the cache policy of the loads: nt (the default) or plain (the tuning knob
+// box_policy = 1).  Stores are nt+sc1 either way.  Measured on MI355X, us per launch, loads
+// plain / nt, with every operand coming from HBM (the launches rotate over 4 GiB of buffers):
+//   [64,512,1024] bf16 dim0->dim2, 16 MiB moved    4.98 /  4.71      8192^2 bf16, 32 MiB    8.56 /  8.03
+//   8192^2 fp32, 64 MiB                           13.90 / 12.87      gather 8 x [4096,4096] bf16 into pitch 4160   84.6 / 80.9
+// When the sources are partly still in the 256 MB Infinity Cache (the same few hundred MiB
+// copied again and again) the order turns round for the redistributions, which read one block
+// of columns out of every row: 3.92 / 4.60, 6.92 / 7.79 and 10.91 / 12.85 -- plain loads may then
+// hit in that cache, nt loads go past it.  A caller that knows its sources to be freshly
+// written and small can ask for them with the knob.
+template<int U, bool EQUAL, bool PLAIN>
 __global__ __launch_bounds__(kBlock) void copy_boxes16_kernel(CopyArgs a) {
-  constexpr int kLoad = SPARSE ? 0 : 2;
+  constexpr int kLoad = PLAIN ? 0 : 2;
   constexpr int kStore = 18;
   constexpr uint32_t log2slots = ilog2(kBlock * U);
   uint32_t tile = blockIdx.x; // first tile untested, as above
@@ -329,7 +330,7 @@ struct Step {
   int unroll; // sub-tiles
   uint32_t grid;
   uint32_t grid_y; // > 0: the two-dimensional form for equal boxes / segments (grid x grid_y workgroups)
-  bool sparse_source; // kBoxes16: the source rows are not adjacent in memory (plain instead of nt loads)
+  bool plain_loads; // kBoxes16: plain instead of nt loads (tuning knob)
   size_t lds;
   FlatArgs flat;   // kFlat
   CopyArgs boxes;  // kBoxes16, kBoxes
@@ -358,7 +359,7 @@ struct Launcher {
   // with a padded row pitch; at 64 MiB and below a cap gains nothing or costs.
   static constexpr uint64_t kLongCopyBytes = (uint64_t)128 << 20;
   size_t lds = 0; // of the launch being assembled
-  bool sparse_source = false;
+  bool plain_loads = false;
 
   void choose_cap(uint64_t bytes) {
     int cap = tuning().copy_wg_per_cu;
@@ -417,7 +418,7 @@ struct Launcher {
       }
       Step st;
       st.kind = Step::kFlat, st.vec = 16, st.unroll = U, st.grid = grid, st.grid_y = 0, st.lds = lds;
-      st.sparse_source = false;
+      st.plain_loads = false;
       if (a.tiles_per_seg && grid == a.total_tiles && a.nsegs > 1) {
         st.grid = a.tiles_per_seg, st.grid_y = a.nsegs;
       }
@@ -455,7 +456,7 @@ struct Launcher {
     Step st;
     st.kind = buffer16 ? Step::kBoxes16 : Step::kBoxes;
     st.vec = vec, st.unroll = unroll, st.grid = grid, st.grid_y = 0, st.lds = buffer16 ? lds : 0;
-    st.sparse_source = sparse_source;
+    st.plain_loads = plain_loads;
     if (buffer16 && a.tiles_per_box && grid == a.total_tiles) {
       st.grid = a.tiles_per_box, st.grid_y = a.nboxes;
     }
@@ -469,13 +470,7 @@ struct Launcher {
       all_vectors += (uint64_t)d.rows * d.cols;
     }
     choose_cap(lg == 5 ? all_vectors * 16 : 0); // the 16-byte buffer kernel only
-    sparse_source = false;
-    for (const BoxDesc& d : list) {
-      sparse_source = sparse_source || (d.rows > 1 && d.src_stride[0] != (int64_t)d.cols * 16);
-    }
-    if (tuning().box_policy) {
-      sparse_source = tuning().box_policy == 1;
-    }
+    plain_loads = tuning().box_policy == 1;
     // strided boxes: two sub-tiles measured best on large gathers (6.1 against 5.9 TB/s with four)
     const int U = tuning().box_unroll ? tuning().box_unroll : auto_unroll(all_vectors, 2);
     unroll = U;
@@ -777,7 +772,7 @@ int launch_step(const Step& st, const FlatArgs* flat, const CopyArgs* boxes, hip
     MDH_LAUNCH_COPY(copy_flat_kernel, , *flat)
     return check_launch("copy_flat_kernel");
   case Step::kBoxes16:
-    if (st.sparse_source) {
+    if (st.plain_loads) {
       MDH_LAUNCH_COPY(copy_boxes16_kernel, MDH_COMMA true, *boxes)
     } else {
       MDH_LAUNCH_COPY(copy_boxes16_kernel, MDH_COMMA false, *boxes)

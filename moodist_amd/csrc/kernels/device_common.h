@@ -85,12 +85,13 @@ struct Tuning {
   int reduce_unroll = 0; // KiB of each source per tile: 1, 2, 4, 8, 16
   int reduce_chunk = 0;  // sources in flight together: 1, 2, 4, 8
   int reduce_max_blocks = 0;
+  int reduce_split_tiles = 0; // tiles of one launch at most (longer reductions are cut into several launches)
   int reduce_wg_per_cu = 0; // cap on resident workgroups per CU (1..8; 9 = none), through an unused LDS allocation
   int copy_unroll = 0; // contiguous segments
   int box_unroll = 0;  // strided boxes
   int copy_max_blocks = 0;
   int copy_wg_per_cu = 0; // as reduce_wg_per_cu, for the copy kernels
-  int box_policy = 0;     // loads of the strided-box kernel: 0 by layout, 1 plain, 2 nt
+  int box_policy = 0;     // loads of the strided-box kernel: 1 plain, 0 or 2 nt
 };
 Tuning& tuning();
 

@@ -394,7 +394,51 @@ LaunchShape choose_shape(const ReduceArgs& a) {
 }
 
 template<typename T, int F, bool PREMUL = false>
+int launch_one(const ReduceArgs& a, hipStream_t stream);
+
+// Tiles of one launch at most.  While the waves of a launch walk the sources in step, the chip
+// reads one source at a time and writes in bursts; over many tiles per wave they drift apart,
+// reads and writes mix at the DRAM, and the rate falls towards that of a mixed stream (fp32
+// 8 sources: 84.8 % at 64 MiB per source, 82.0 % at 128 MiB, 76.5 % at 256 MiB, 73.8 % at
+// 512 MiB in one launch, whatever the grid).  A launch boundary lines the waves up again for the
+// price of one launch gap (1.6 us per 90 us and more).
+constexpr uint64_t kSplitTiles = 4096;
+
+template<typename T, int F, bool PREMUL = false>
 int launch_vec(const ReduceArgs& a, hipStream_t stream) {
+  const Tuning& t = tuning();
+  const LaunchShape whole = choose_shape<T, PREMUL>(a);
+  const uint64_t tile_vecs = (uint64_t)kWave * whole.unroll;
+  const uint64_t ntiles = (a.nvec + tile_vecs - 1) / tile_vecs;
+  const uint64_t limit = t.reduce_split_tiles > 0 ? (uint64_t)t.reduce_split_tiles : kSplitTiles;
+  if (ntiles <= limit + limit / 2) {
+    return launch_one<T, F, PREMUL>(a, stream);
+  }
+  // equal parts, each a whole number of passes of 512 waves
+  const uint64_t parts = (ntiles + limit - 1) / limit;
+  const uint64_t part_tiles = ((ntiles + parts - 1) / parts + 511) / 512 * 512;
+  const uint64_t part_vecs = part_tiles * tile_vecs;
+  constexpr uint64_t kElemsPerVec = 16 / sizeof(typename Traits<T>::elem_t);
+  for (uint64_t at = 0; at < a.nvec; at += part_vecs) {
+    ReduceArgs part = a;
+    for (int j = 0; j < a.nsrc; ++j) {
+      part.src[j] = (const char*)a.src[j] + at * 16;
+    }
+    part.dst = (char*)a.dst + at * 16;
+    const bool last = at + part_vecs >= a.nvec;
+    part.nvec = last ? a.nvec - at : part_vecs;
+    // the elements past the last whole vector belong to the last part
+    part.numel = last ? a.numel - at * kElemsPerVec : part_vecs * kElemsPerVec;
+    const int rc = launch_one<T, F, PREMUL>(part, stream);
+    if (rc != MDH_OK) {
+      return rc;
+    }
+  }
+  return MDH_OK;
+}
+
+template<typename T, int F, bool PREMUL>
+int launch_one(const ReduceArgs& a, hipStream_t stream) {
   const Tuning& t = tuning();
   const LaunchShape shape = choose_shape<T, PREMUL>(a);
   dim3 g((unsigned)shape.waves), b(kWave);

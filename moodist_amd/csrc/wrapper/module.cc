@@ -384,13 +384,14 @@ public:
       outs.push_back(describe(t));
     }
     moodist_tensor i = describe(inputs[0]);
+    auto result = c10::make_intrusive<WorkImpl>();
     moodist_work* w = nullptr;
     check(extra.moodist_pg_all_gather_list(c_, outs.data(), outs.size(), &i, stream_of(inputs[0]), &w));
+    result->parts.push_back(w);
     auto held = new std::vector<at::Tensor>(outputLists[0]);
     held->push_back(inputs[0]);
+    // the core owns `held` from the call on and releases it exactly once, also when it fails
     check(extra.moodist_pg_keep_alive(c_, held, release_tensors));
-    auto result = c10::make_intrusive<WorkImpl>();
-    result->parts.push_back(w);
     result->tensors = outputLists[0];
     return result;
   }

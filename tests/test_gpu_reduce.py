@@ -99,6 +99,38 @@ def test_large_sources_take_the_capped_shape_and_match(dev):
         del srcs, want, out
 
 
+def test_long_reductions_cut_into_several_launches(dev):
+    # Reductions of more tiles than reduce_split_tiles are run as several launches over
+    # consecutive parts.  With the limit at one tile every input of a few MiB is cut: ragged
+    # sizes, element tails, pointers that are not 16-byte aligned, guard elements around the output.
+    old = abi.get_tuning("reduce_split_tiles")
+    try:
+        abi.set_tuning("reduce_split_tiles", 1)
+        for dtype, P, n in ((torch.float32, 3, 786432 + 5), (torch.bfloat16, 5, 1572864 + 7), (torch.int64, 2, 400000 + 1),
+                            (torch.float64, 4, 393216 + 3), (torch.float16, 9, 3000000 + 1)):
+            raw = random_sources(P, n + 8, dtype, seed=n % 1000 + P)
+            views = [r[1 + i % 3:][:n] for i, r in enumerate(raw)]
+            dviews = [r.to(dev)[1 + i % 3:][:n] for i, r in enumerate(raw)]
+            canvas = torch.full((n + 8,), 7, dtype=dtype, device=dev)
+            out = canvas[3:3 + n]
+            for op in (oracle.OP_SUM, oracle.OP_MAX) + ((oracle.OP_AVG,) if dtype.is_floating_point else ()):
+                scale = scale_for(op, P)
+                gpu_reduce(dviews, P - 1, out, op, scale)
+                want = oracle.reduce([bits(v) for v in views], P - 1, TORCH_TO_CODE[dtype], op, scale)
+                assert same_bits(bits(out), want), (dtype, P, n, op)
+                assert (canvas[:3] == 7).all() and (canvas[3 + n:] == 7).all()
+    finally:
+        abi.set_tuning("reduce_split_tiles", old)
+    # and at the library's own limit: 160 MiB per source is 10,240 tiles, three launches
+    n = (160 << 20) // 4 + 3
+    g = torch.Generator().manual_seed(3)
+    srcs = [torch.randn(n, generator=g) for _ in range(2)]
+    want = oracle.reduce([bits(s) for s in srcs], 1, TORCH_TO_CODE[torch.float32], oracle.OP_SUM)
+    out = torch.zeros(n, dtype=torch.float32, device=dev)
+    gpu_reduce([s.to(dev) for s in srcs], 1, out, oracle.OP_SUM)
+    assert same_bits(bits(out), want)
+
+
 def test_golden_fixtures(dev):
     z = np.load(os.path.join(HERE, "golden", "reduce_cases.npz"))
     code_to_torch = {v: k for k, v in TORCH_TO_CODE.items()}
