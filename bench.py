@@ -3,7 +3,8 @@
 A step is one pass of the local multi-source reduction over one batch of staged chunks:
 reduce_scatter_tensor SUM, fp32, world size 8 seen from rank 0 -- eight staged 16 MiB chunks
 folded in rank order into one 16 MiB output (4,194,304 elements).  Inputs are resident in HBM
-before the timed region.  Prints one JSON line.
+before the timed region; the launches rotate over 4 GiB of distinct buffers, so that they are
+not in the 256 MB Infinity Cache either.  Prints one JSON line.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
                   [--tuning KNOB=VALUE ...]
@@ -24,19 +25,18 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 CLOCK_WARMUP_S = 0.3   # untimed launches before the first timed window
 TIMED_WINDOWS = 11     # windows of `steps` launches; the median window is reported
-INFINITY_CACHE_BYTES = 256 << 20
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch), each
-# scaled by what the same counter reads for the flat copy of exactly 256 MiB (FETCH_SIZE x 1.99983,
+# scaled by what the same counter reads for the flat copy of exactly 256 MiB (FETCH_SIZE x 1.99982,
 # WRITE_SIZE x 1.00000): profiles/hbm_traffic_pmc_reduce_and_copy_kernels.md.  E.g. the headline:
-# 65,557.91 x 1.99983 + 16,384.00 KiB = 147,488.5 KiB.  Workloads without an entry were not measured.
+# 65,557.94 x 1.99982 + 16,384.00 KiB = 147,488.3 KiB.  Workloads without an entry were not measured.
 MEASURED_TRAFFIC_BYTES = {
-    "reduce_fp32_p8": 151028193,
-    "reduce_bf16_p16": 1141025530,
-    "reduce_fp32_p64_sum": 272661846,
+    "reduce_fp32_p8": 151028042,
+    "reduce_bf16_p16": 1141022518,
+    "reduce_fp32_p64_sum": 272661006,
     "allgather_bf16_p8": 536870912,
-    "allgather_bf16_p8_strided": 536886266,
-    "redistribute_fp32_8192": 67155282,
-    "redistribute_bf16_3d": 16825499,
+    "allgather_bf16_p8_strided": 536886317,
+    "redistribute_fp32_8192": 67146423,
+    "redistribute_bf16_3d": 16815056,
 }
 
 def build_workload(name, torch, abi, dev, rotation_bytes):
@@ -394,6 +394,11 @@ def main():
     desc["clock_warmup_s"] = args.clock_warmup
     desc["clock_warmup_launches"] = clock_launches
     if not args.no_check:
+        # every set's output is checked: make sure each has been written (a short run may not
+        # have gone round the whole rotation)
+        for i in range(desc["buffer_sets"]):
+            launch(i)
+        torch.cuda.synchronize()
         check()
     gbs = alg_bytes / (ms_per_step * 1e-3) / 1e9
     kernel_gbs = alg_bytes / (kernel_ms * 1e-3) / 1e9

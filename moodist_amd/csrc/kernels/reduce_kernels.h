@@ -338,7 +338,10 @@ struct LaunchShape {
 };
 
 // Chosen by measurement on MI355X (percent of 8 TB/s, algorithmic bytes; one-wave workgroups;
-// tile KiB x sources in flight @ waves):
+// tile KiB x sources in flight @ waves).  These rows were measured with the launches rotating
+// over 0.6-1.2 GiB of buffers, where the 256 MB Infinity Cache still helps every shape by 2-4
+// points; rotating over 4-8 GiB the order is the same (8 x 16 MiB: 16x1@1024 82.2, 16x2 81.0,
+// 16x1@512 78.6, 8x2 76.8, 4x4 67.8; 64 x 4 MiB: 8x2 84.9, 16x2 77.5, 4x4 78.1, 16x1 61.7):
 //   fp32  8 x 16 MiB   16x1@1024: 84.4   16x1@512: 80.4   16x2@1024: 83.3   8x2@2048: 77.9   4x8@1024: 72.8
 //   fp32  8 x 64 MiB   16x1@512: 84.8    16x1@1024: 81.6  16x1@4096: 82.8   16x2@1024: 84.8  8x2@512: 83.8
 //   fp32 16 x 32 MiB   16x1@512: 86.8    16x1@1024: 85.2  16x2@1024: 86.3   8x1@1024: 84.2
