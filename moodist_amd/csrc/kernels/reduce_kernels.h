@@ -361,8 +361,15 @@ template<typename T, bool PREMUL>
 LaunchShape choose_shape(const ReduceArgs& a) {
   const Tuning& t = tuning();
   constexpr bool half = sizeof(typename Traits<T>::elem_t) == 2;
+  // The longest tile that still leaves this many tiles: 512 (a wave on every other SIMD), or
+  // 1024 for 16-bit types, whose arithmetic per byte needs every SIMD, and for sources of 2 MiB
+  // and less, where the launch is over before a second tile per wave would have paid.
+  // Measured from HBM, 8 sources, us per launch with 512 / 1024 tiles: bf16 2 MiB per source
+  // 5.87 / 5.05, 8 MiB 15.4 / 14.6, 16 MiB (1024 / 2048) 24.0 / 26.3; fp32 1 MiB 3.58 / 3.35,
+  // 2 MiB 5.24 / 5.00, 4 MiB 7.86 / 8.10, 8 MiB 12.7 / 13.0.
+  const uint64_t min_tiles = (half || a.nvec <= ((uint64_t)2 << 20) / 16) ? 1024 : 512;
   int u = 16;
-  while (u > 1 && a.nvec / ((uint64_t)kWave * u) < 512) {
+  while (u > 1 && a.nvec / ((uint64_t)kWave * u) < min_tiles) {
     u >>= 1;
   }
   if (PREMUL && half && u > 4) {
