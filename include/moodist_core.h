@@ -117,7 +117,10 @@ int moodist_pg_allreduce(moodist_pg* pg, const moodist_tensor* tensor, const moo
  *    same time -- calls that overlap race;
  *  - the padding elements hold what the last call left there; they are reduced and thrown
  *    away, nothing needs to start at zero.
- * When numel is a multiple of the group size no temporary is used at all. */
+ * When numel is a multiple of the group size no temporary is used at all.  The first call on
+ * a device looks the workspace's address up (and may load the kernel library's code there):
+ * a caller that captures streams makes one call, or calls mdh_static_workspace, before it
+ * starts capturing. */
 int moodist_pg_allreduce_static(moodist_pg* pg, const moodist_tensor* tensor, int reduce_op, void* stream,
     float premul_value, moodist_work** work);
 /* No counterpart in the reference, where a peer's contribution is whatever that peer's own
