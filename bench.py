@@ -28,15 +28,15 @@ TIMED_WINDOWS = 11     # windows of `steps` launches; the median window is repor
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch), each
 # scaled by what the same counter reads for the flat copy of exactly 256 MiB (FETCH_SIZE x 1.99982,
 # WRITE_SIZE x 1.00000): profiles/hbm_traffic_pmc_reduce_and_copy_kernels.md.  E.g. the headline:
-# 65,557.94 x 1.99982 + 16,384.00 KiB = 147,488.3 KiB.  Workloads without an entry were not measured.
+# 65,557.89 x 1.99982 + 16,384.00 KiB = 147,488.2 KiB.  Workloads without an entry were not measured.
 MEASURED_TRAFFIC_BYTES = {
-    "reduce_fp32_p8": 151028042,
-    "reduce_bf16_p16": 1141022518,
-    "reduce_fp32_p64_sum": 272661006,
+    "reduce_fp32_p8": 151027962,
+    "reduce_bf16_p16": 1140846489,
+    "reduce_fp32_p64_sum": 272661054,
     "allgather_bf16_p8": 536870912,
-    "allgather_bf16_p8_strided": 536886317,
-    "redistribute_fp32_8192": 67146423,
-    "redistribute_bf16_3d": 16815056,
+    "allgather_bf16_p8_strided": 536886304,
+    "redistribute_fp32_8192": 67145620,
+    "redistribute_bf16_3d": 16814970,
 }
 
 def build_workload(name, torch, abi, dev, rotation_bytes):

@@ -72,13 +72,15 @@ struct Traits<bf16_t> {
   static __device__ __forceinline__ float widen(uint16_t e) {
     return __uint_as_float((uint32_t)e << 16);
   }
-  // round to nearest even; NaN stays a quiet NaN
+  // Round to nearest even; a NaN keeps its sign and upper payload and gets the quiet bit.  That is
+  // what gfx950's v_cvt_pk_bf16_f32 does, to which this conversion compiles: for every one of the
+  // 2^32 fp32 bit patterns it returns ((u + 0x7fff + ((u >> 16) & 1)) >> 16), or (u >> 16) | 0x40
+  // for a NaN (checked exhaustively on the GPU by tests/native/bf16_narrow_check.cc).
   static __device__ __forceinline__ uint16_t narrow(float f) {
-    // both candidates are computed and one is selected: no divergent branch per element
-    const uint32_t u = __float_as_uint(f);
-    const uint32_t rounded = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-    const uint32_t quiet = (u >> 16) | 0x0040u;
-    return (uint16_t)((u & 0x7fffffffu) > 0x7f800000u ? quiet : rounded);
+    const __bf16 b = (__bf16)f;
+    uint16_t e;
+    __builtin_memcpy(&e, &b, 2);
+    return e;
   }
   static __device__ __forceinline__ float premul(float a, float s) {
     return widen(narrow(a * s));
@@ -393,10 +395,16 @@ LaunchShape choose_shape(const ReduceArgs& a) {
     ntiles = 1; // tail only
   }
   // From two tiles per SIMD on, 512 waves that walk the tiles keep fewer streams open (fp32
-  // 8 x 64 MiB: 84.8 % against 82.8 % with a wave per tile).  16-bit types spend three to four
-  // times the arithmetic per byte (widening), which a lone wave on a SIMD cannot overlap with its
-  // own loads: they keep a wave per tile (bf16 16 x 64 MiB: 84.0 % against 78.6 % with 512 waves).
-  s.waves = (ntiles >= 2048 && !half) ? 512 : ntiles;
+  // 8 x 64 MiB: 84.8 % against 82.8 % with a wave per tile).  16-bit types spend more arithmetic
+  // per byte (widening), which a lone wave on a SIMD overlaps less well with its own loads: they
+  // go to 512 waves from 4096 tiles on and take 1024 in between (bf16 16 x 64 MiB: 86.7 % with
+  // 512 waves, 83.0 % with 1024, 80.7 % with a wave per tile; 8 x 32 MiB, 2048 tiles: 78.9 / 81.2 /
+  // 78.7 %).
+  if (half) {
+    s.waves = ntiles >= 4096 ? 512 : ntiles >= 2048 ? 1024 : ntiles;
+  } else {
+    s.waves = ntiles >= 2048 ? 512 : ntiles;
+  }
   if (t.reduce_max_blocks > 0) {
     s.waves = ntiles < (uint64_t)t.reduce_max_blocks ? ntiles : (uint64_t)t.reduce_max_blocks;
   }

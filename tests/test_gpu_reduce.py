@@ -365,3 +365,17 @@ def test_reduce_beyond_4_gib_per_source(dev):
     out = torch.zeros(n, device=dev)
     gpu_reduce([a, b], 0, out, oracle.OP_MAX)
     assert torch.equal(out, torch.maximum(a, b))
+
+
+def test_bf16_narrowing_follows_the_rounding_rule_for_every_fp32_pattern(dev):
+    # the library narrows with the hardware conversion of gfx950; a device program compares it
+    # with the rule (nearest, ties to even, quiet NaN with its payload) on all 2^32 inputs
+    import subprocess
+
+    exe = os.path.join(os.path.dirname(HERE), "tests", "native", "bf16_narrow_check.bin")
+    if not os.path.exists(exe):
+        pytest.skip("tests/native/bf16_narrow_check.bin is not built (run __graft_entry__.build())")
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    print(r.stdout)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    assert "4294967296 fp32 patterns and 65536 bf16 patterns checked, 0 differ" in r.stdout
