@@ -318,10 +318,10 @@ __global__ __launch_bounds__(kWave) void reduce_vec_kernel(ReduceArgs a) {
     const uint64_t tile_byte = tile * tile_bytes;
     const uint64_t left = body_bytes - tile_byte;
     const uint32_t n = (uint32_t)(left < tile_bytes ? left : tile_bytes);
-    // PREMUL_SUM is a kernel of its own: for 16-bit types every source element is rounded to the
-    // element type after the multiply, which takes several times the registers of the plain
-    // fold, and a kernel's register budget is that of its hungriest path.  AVG is the plain
-    // fold with one more multiply when the result is written (a wave-uniform test there).
+    // PREMUL_SUM is a kernel of its own, so that the plain fold carries neither its multiply nor,
+    // for 16-bit types, the rounding of every source element to the element type after it.  AVG
+    // is the plain fold with one more multiply when the result is written (a wave-uniform test
+    // there).
     reduce_tile<T, F, U, CH, PREMUL ? kPremul : kPlain>(a, nsrc, tile_byte, n);
     tile += gridDim.x;
   } while (tile < ntiles);
@@ -373,9 +373,6 @@ LaunchShape choose_shape(const ReduceArgs& a) {
   int u = 16;
   while (u > 1 && a.nvec / ((uint64_t)kWave * u) < min_tiles) {
     u >>= 1;
-  }
-  if (PREMUL && half && u > 4) {
-    u = 4; // the per-element rounding of PREMUL_SUM needs several registers per element
   }
   int ch = u >= 16 ? 1 : 16 / u > 8 ? 8 : 16 / u;
   if (t.reduce_unroll) {

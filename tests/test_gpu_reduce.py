@@ -97,6 +97,17 @@ def test_large_sources_take_the_capped_shape_and_match(dev):
         gpu_reduce([s.to(dev) for s in srcs], 5, out, oracle.OP_SUM)
         assert same_bits(bits(out), want), (dtype, P)
         del srcs, want, out
+    # PREMUL_SUM and AVG of 16-bit types on the longest tiles (16 MiB per source and more)
+    for dtype in (torch.bfloat16, torch.float16):
+        n = (16 << 20) // 2 + 3
+        srcs = random_sources(3, n, dtype, seed=77)
+        d = [s.to(dev) for s in srcs]
+        for op in (oracle.OP_PREMUL_SUM, oracle.OP_AVG):
+            scale = scale_for(op, 3)
+            want = oracle.reduce([bits(s) for s in srcs], 1, TORCH_TO_CODE[dtype], op, scale)
+            out = torch.zeros(n, dtype=dtype, device=dev)
+            gpu_reduce(d, 1, out, op, scale)
+            assert same_bits(bits(out), want), (dtype, op)
 
 
 def test_long_reductions_cut_into_several_launches(dev):
