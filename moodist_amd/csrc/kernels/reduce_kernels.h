@@ -26,7 +26,9 @@ struct ReduceArgs {
   const void* src[MDH_MAX_SOURCES]; // already rotated into fold order
   void* dst;
   uint64_t nvec;  // 16-byte vectors on the vector path
-  uint64_t numel; // all elements
+  uint64_t numel; // elements from the pointers on: the vectors' and the < 16 bytes after them
+  uint32_t head;  // elements BEFORE the pointers (fewer than 64 bytes): see mdh_reduce
+  uint32_t elem_wave; // 1: the last workgroup of the grid folds the head and tail elements, 0: there are none
   float scale;
   int nsrc;
   int mode;
@@ -213,21 +215,32 @@ __device__ __forceinline__ void fold_chunk(const ReduceArgs& a, int j0, uint64_t
   }
 }
 
+// One element, folded in source order.  The loads of eight sources are issued together: one
+// after the other, every source would cost this lane a whole memory round trip.
 template<typename T, int F>
-__device__ __forceinline__ void reduce_one_elem(const ReduceArgs& a, int nsrc, uint64_t i) {
+__device__ __forceinline__ void reduce_one_elem(const ReduceArgs& a, int nsrc, int64_t i) {
   using Tr = Traits<T>;
   using elem_t = typename Tr::elem_t;
   using acc_t = typename Tr::acc_t;
-  acc_t acc = Tr::widen(((const elem_t*)a.src[0])[i]);
-  if (a.mode == kPremul) {
-    acc = Tr::premul(acc, a.scale);
-  }
-  for (int j = 1; j < nsrc; ++j) {
-    acc_t x = Tr::widen(((const elem_t*)a.src[j])[i]);
-    if (a.mode == kPremul) {
-      x = Tr::premul(x, a.scale);
+  constexpr int kBatch = 8;
+  acc_t acc{};
+  for (int j0 = 0; j0 < nsrc; j0 += kBatch) {
+    elem_t v[kBatch];
+#pragma unroll
+    for (int k = 0; k < kBatch; ++k) {
+      const int j = j0 + k < nsrc ? j0 + k : nsrc - 1; // past the end: the last source once more, unused
+      v[k] = ((const elem_t*)a.src[j])[i];
     }
-    acc = fold<F>(acc, x);
+#pragma unroll
+    for (int k = 0; k < kBatch; ++k) {
+      if (j0 + k < nsrc) {
+        acc_t x = Tr::widen(v[k]);
+        if (a.mode == kPremul) {
+          x = Tr::premul(x, a.scale);
+        }
+        acc = j0 + k == 0 ? x : fold<F>(acc, x);
+      }
+    }
   }
   ((elem_t*)a.dst)[i] = Tr::template finish<F>(acc, a.mode, a.scale);
 }
@@ -302,15 +315,30 @@ __device__ __forceinline__ void reduce_tile(const ReduceArgs& a, int nsrc, uint6
 
 // A tile is kWave*U consecutive 16-byte vectors (U KiB); tiles are dealt to
 // waves round-robin.  Pointers need only element alignment: gfx950's
-// 16-byte buffer accesses take any byte address.  Elements past the last whole
-// vector (fewer than 16 bytes) are folded by workgroup 0.
+// 16-byte buffer accesses take any byte address.  Elements before the pointers (a.head, fewer
+// than 64 bytes) and past the last whole vector (fewer than 16 bytes) are folded by one more
+// workgroup at the end of the grid.
 template<typename T, int F, int U, int CH, bool PREMUL>
 __global__ __launch_bounds__(kWave) void reduce_vec_kernel(ReduceArgs a) {
   const int nsrc = a.nsrc;
   constexpr uint64_t tile_bytes = (uint64_t)kWave * U * 16;
   const uint64_t body_bytes = a.nvec * 16;
   const uint64_t ntiles = (body_bytes + tile_bytes - 1) / tile_bytes;
-  // The grid never exceeds the tile count (a launch with no whole vector has one wave, whose
+  // The head and tail elements have a workgroup of their own, the last of the grid: folded by a
+  // workgroup that also has tiles, their round trips would come on top of that wave's tiles and
+  // lengthen the whole launch (by 1.5 us of 23 for eight sources).
+  const uint32_t tile_waves = gridDim.x - a.elem_wave;
+  if (a.elem_wave != 0 && blockIdx.x == tile_waves) {
+    // one element per lane: the head before the pointers (indices -head .. -1, fewer than 64
+    // bytes), then the tail after the last whole vector (fewer than 16 bytes): at most 31 + 7 lanes
+    const int64_t lane = threadIdx.x, head = a.head;
+    const int64_t i = lane < head ? lane - head : (int64_t)(a.nvec * per_vec<T>()) + (lane - head);
+    if (i < (int64_t)a.numel) {
+      reduce_one_elem<T, F>(a, nsrc, i);
+    }
+    return;
+  }
+  // The tile waves never outnumber the tiles (a launch with no whole vector has one, whose
   // descriptors are then empty), so the first tile needs no test and the scalar loads of the
   // arguments are not held up behind a load-and-branch.
   uint64_t tile = blockIdx.x;
@@ -323,14 +351,8 @@ __global__ __launch_bounds__(kWave) void reduce_vec_kernel(ReduceArgs a) {
     // is the plain fold with one more multiply when the result is written (a wave-uniform test
     // there).
     reduce_tile<T, F, U, CH, PREMUL ? kPremul : kPlain>(a, nsrc, tile_byte, n);
-    tile += gridDim.x;
+    tile += tile_waves;
   } while (tile < ntiles);
-  if (blockIdx.x == 0) {
-    const uint64_t i = a.nvec * per_vec<T>() + threadIdx.x;
-    if (i < a.numel) {
-      reduce_one_elem<T, F>(a, nsrc, i);
-    }
-  }
 }
 
 struct LaunchShape {
@@ -440,6 +462,7 @@ int launch_vec(const ReduceArgs& a, hipStream_t stream) {
       part.src[j] = (const char*)a.src[j] + at * 16;
     }
     part.dst = (char*)a.dst + at * 16;
+    part.head = at == 0 ? a.head : 0;
     const bool last = at + part_vecs >= a.nvec;
     part.nvec = last ? a.nvec - at : part_vecs;
     // the elements past the last whole vector belong to the last part
@@ -453,10 +476,12 @@ int launch_vec(const ReduceArgs& a, hipStream_t stream) {
 }
 
 template<typename T, int F, bool PREMUL>
-int launch_one(const ReduceArgs& a, hipStream_t stream) {
+int launch_one(const ReduceArgs& a0, hipStream_t stream) {
   const Tuning& t = tuning();
-  const LaunchShape shape = choose_shape<T, PREMUL>(a);
-  dim3 g((unsigned)shape.waves), b(kWave);
+  const LaunchShape shape = choose_shape<T, PREMUL>(a0);
+  ReduceArgs a = a0;
+  a.elem_wave = (a.head != 0 || a.numel > a.nvec * (16 / sizeof(typename Traits<T>::elem_t))) ? 1u : 0u;
+  dim3 g((unsigned)shape.waves + a.elem_wave), b(kWave);
   // reduce_wg_per_cu (measurement only): an unused LDS allocation caps the waves resident on a CU
   const int cap = t.reduce_wg_per_cu >= 2 && t.reduce_wg_per_cu <= 8 ? t.reduce_wg_per_cu : 0;
   const size_t lds = kLdsForCap[cap];
