@@ -242,15 +242,36 @@ __global__ __launch_bounds__(kBlock) void copy_boxes16_kernel(CopyArgs a) {
 constexpr int kMaxSegments = 64;
 
 struct FlatArgs {
-  const char* src[kMaxSegments];
+  const char* src[kMaxSegments]; // first byte of the segment's whole vectors (after its head)
   char* dst[kMaxSegments];
   uint32_t tile_end[kMaxSegments]; // cumulative tiles; unused entries are ~0
-  uint64_t bytes[kMaxSegments];    // multiples of 16
+  uint64_t bytes[kMaxSegments];    // of whole vectors: multiples of 16
+  // The segment's first bytes, up to its destination's next 64-byte boundary, and its last
+  // < 16 bytes: they sit before src/dst and after src/dst + bytes, and are copied byte by byte
+  // by workgroups of their own (edge_wgs of them, in front of the tile workgroups).
+  uint8_t head[kMaxSegments]; // 0..63
+  uint8_t tail[kMaxSegments]; // 0..15
   uint32_t nsegs;
   uint32_t total_tiles;
   uint32_t tiles_per_seg; // non-zero when every segment has the same tile count
+  uint32_t edge_wgs;      // 0: no segment has a head or a tail
 };
 static_assert(sizeof(FlatArgs) <= 4096, "kernel arguments are limited to 4 KiB");
+
+// Edge bytes are numbered per segment: slots 0..63 are the head's bytes, 64..79 the tail's.
+constexpr uint32_t kEdgeSlots = 80;
+
+// The byte a slot stands for, as an offset from the segment's src/dst (negative in the head);
+// false for a slot the segment does not use.
+MDH_HD bool edge_offset(const FlatArgs& a, uint32_t seg, uint32_t slot, int64_t* off) {
+  if (slot < 64) {
+    const uint32_t head = a.head[seg];
+    *off = (int64_t)slot - (int64_t)head;
+    return slot < head;
+  }
+  *off = (int64_t)a.bytes[seg] + (int64_t)(slot - 64);
+  return slot - 64 < a.tail[seg];
+}
 
 // Which segment a tile belongs to, and the tile's first byte inside it (same two ways as for boxes).
 MDH_HD uint32_t locate_segment(const FlatArgs& a, uint32_t tile, uint32_t* local) {
@@ -272,15 +293,47 @@ MDH_HD uint32_t locate_segment(const FlatArgs& a, uint32_t tile, uint32_t* local
   return seg;
 }
 
-// EQUAL: as for the boxes -- segments of equal tile count, blockIdx.y the segment, blockIdx.x the tile.
+// Workgroup `wg` of `nwg` edge workgroups: one byte per lane and round.
+__device__ __forceinline__ void copy_edges(const FlatArgs& a, uint32_t wg, uint32_t nwg) {
+  const uint32_t all = a.nsegs * kEdgeSlots;
+  for (uint32_t idx = wg * kBlock + threadIdx.x; idx < all; idx += nwg * kBlock) {
+    const uint32_t seg = idx / kEdgeSlots, slot = idx - seg * kEdgeSlots;
+    int64_t off;
+    if (edge_offset(a, seg, slot, &off)) {
+      a.dst[seg][off] = a.src[seg][off];
+    }
+  }
+}
+
+// EQUAL: as for the boxes -- segments of equal tile count, blockIdx.y the segment, blockIdx.x the
+// tile.  Edge workgroups come FIRST in the grid -- row 0 (EQUAL) or workgroups 0 .. edge_wgs-1 --
+// so that their one round trip is over long before the tiles are.
 template<int U, bool EQUAL>
 __global__ __launch_bounds__(kBlock) void copy_flat_kernel(FlatArgs a) {
   constexpr uint32_t tile_bytes = kBlock * U * 16;
   const uint32_t lane_byte = threadIdx.x * 16;
-  uint32_t tile = blockIdx.x; // first tile untested, as in the box kernels
+  const uint32_t edge_wgs = a.edge_wgs;
+  uint32_t first_tile = blockIdx.x, tile_wgs = gridDim.x, row = blockIdx.y;
+  if (EQUAL) {
+    if (edge_wgs != 0) { // one more row, in front
+      if (row == 0) {
+        copy_edges(a, blockIdx.x, gridDim.x);
+        return;
+      }
+      row -= 1;
+    }
+  } else {
+    if (blockIdx.x < edge_wgs) {
+      copy_edges(a, blockIdx.x, edge_wgs);
+      return;
+    }
+    first_tile -= edge_wgs;
+    tile_wgs -= edge_wgs;
+  }
+  uint32_t tile = first_tile; // untested, as in the box kernels
   do {
     uint32_t local;
-    const uint32_t seg = EQUAL ? (local = blockIdx.x, blockIdx.y) : locate_segment(a, tile, &local);
+    const uint32_t seg = EQUAL ? (local = blockIdx.x, row) : locate_segment(a, tile, &local);
     const uint64_t off = (uint64_t)local * tile_bytes;
     const uint64_t left = a.bytes[seg] - off;
     const uint32_t n = left < tile_bytes ? (uint32_t)left : tile_bytes;
@@ -298,7 +351,7 @@ __global__ __launch_bounds__(kBlock) void copy_flat_kernel(FlatArgs a) {
     if (EQUAL) {
       break;
     }
-    tile += gridDim.x;
+    tile += tile_wgs;
   } while (tile < a.total_tiles);
 }
 
@@ -338,17 +391,31 @@ struct Step {
 
 int launch_step(const Step& st, const FlatArgs* flat, const CopyArgs* boxes, hipStream_t stream);
 
+// The grid a step is launched with: st.grid (x st.grid_y) tile workgroups, and for a flat step
+// with edges the edge workgroups in front of them (one more row in the two-dimensional form).
+inline void launch_dims(const Step& st, const FlatArgs* flat, uint32_t* x, uint32_t* y) {
+  const uint32_t edge_wgs = st.kind == Step::kFlat && flat ? flat->edge_wgs : 0;
+  if (st.grid_y > 0) {
+    *x = st.grid;
+    *y = st.grid_y + (edge_wgs ? 1u : 0u);
+  } else {
+    *x = st.grid + edge_wgs;
+    *y = 1;
+  }
+}
+
 struct Launcher {
   hipStream_t stream;
   std::vector<Step>* record = nullptr; // when set, launches are recorded here instead of enqueued
   std::vector<BoxDesc> pending[5]; // by log2(VEC)
   std::vector<BoxDesc> pending16;  // 16-byte vectors, spans inside 32 bits: copy_boxes16_kernel
   struct Segment {
-    const char* src;
+    const char* src; // of the whole vectors
     char* dst;
-    uint64_t bytes;
+    uint64_t bytes; // of whole vectors
+    uint8_t head, tail;
   };
-  std::vector<Segment> flat; // contiguous runs, a multiple of 16 bytes long
+  std::vector<Segment> flat; // contiguous runs: whole vectors plus head and tail bytes
   int rc = MDH_OK;
   int unroll = 2; // sub-tiles of the box launch being assembled
 
@@ -384,7 +451,7 @@ struct Launcher {
       a.nsegs = 0;
       uint64_t tiles = 0;
       uint64_t first_tiles = 0;
-      bool equal = true;
+      bool equal = true, edges = false;
       while (i < flat.size() && a.nsegs < (uint32_t)kMaxSegments) {
         const Segment& g = flat[i];
         const uint64_t n = (g.bytes + tile_bytes - 1) / tile_bytes;
@@ -399,16 +466,22 @@ struct Launcher {
         a.src[a.nsegs] = g.src;
         a.dst[a.nsegs] = g.dst;
         a.bytes[a.nsegs] = g.bytes;
+        a.head[a.nsegs] = g.head;
+        a.tail[a.nsegs] = g.tail;
+        edges = edges || g.head || g.tail;
         a.tile_end[a.nsegs] = (uint32_t)tiles;
         ++a.nsegs;
         ++i;
       }
       for (uint32_t k = a.nsegs; k < (uint32_t)kMaxSegments; ++k) {
         a.src[k] = nullptr, a.dst[k] = nullptr, a.bytes[k] = 0;
+        a.head[k] = a.tail[k] = 0;
         a.tile_end[k] = 0xffffffffu;
       }
       a.total_tiles = (uint32_t)tiles;
       a.tiles_per_seg = equal ? (uint32_t)first_tiles : 0;
+      // one byte per lane: a workgroup for every kBlock edge slots, so that no lane goes round twice
+      a.edge_wgs = edges ? (a.nsegs * kEdgeSlots + (uint32_t)kBlock - 1) / (uint32_t)kBlock : 0;
       if (tiles == 0) {
         continue;
       }
@@ -591,9 +664,7 @@ struct Launcher {
     pending[lg].push_back(d);
   }
 
-  // A head box costs a share of one more (narrow) launch, about 0.05 us; below a few MiB the
-  // straddling stores cost less than that.
-  static constexpr int64_t kAlignDestinationFrom = (int64_t)4 << 20;
+  static constexpr int64_t kAlignDestinationFrom = 4096;
 
   // Splits what the kernel's 32-bit extents or kMaxOuter cannot hold.
   void add(HostBox h) {
@@ -601,33 +672,15 @@ struct Launcher {
       return;
     }
     if (h.nd == 0) {
-      // one contiguous run: cut runs too long for 32-bit column counts
-      // 16-byte buffer loads and stores take any byte alignment on gfx950, so the body of a run
-      // moves as whole vectors wherever it starts; only the last < 16 bytes go the narrow way.
-      // Stores want the destination on the 64-byte grid: off it by 4, 16 or 32 bytes a long copy
-      // loses 12-17 % (8 x 32 MiB: 80.6 us aligned or off by 64 B, 91.8 us off by 32 B, 95.5 us off
-      // by 4 B; sources off the grid: 80.8 us).  A long run whose destination is off the grid gives
-      // up its first bytes to the narrow way as well, and its vectors start on the grid.
-      const uintptr_t off_grid = (uintptr_t)h.dst & 63;
-      if (off_grid != 0 && h.run >= kAlignDestinationFrom) {
-        const int64_t head = 64 - (int64_t)off_grid;
-        HostBox p = h;
-        p.run = head;
-        emit(p); // one small box, at whatever vector width its addresses allow
-        p.src = h.src + head, p.dst = h.dst + head, p.run = h.run - head;
-        add(p);
-        return;
-      }
-      if (h.run >= 32 && (h.run & 15)) {
-        const int64_t body = h.run & ~(int64_t)15;
-        HostBox p = h;
-        p.run = body;
-        add(p);
-        p.src = h.src + body, p.dst = h.dst + body, p.run = h.run - body;
-        add(p);
-        return;
-      }
-      const int64_t max_run = (int64_t)1 << 30; // keeps column counts inside 32 bits at any vector width
+      // One contiguous run.  16-byte buffer loads and stores take any byte alignment on gfx950,
+      // so the run moves as whole vectors wherever it starts, and what is not a whole vector --
+      // the last < 16 bytes -- is copied byte by byte by the flat kernel's edge workgroups, in
+      // the same launch.  Stores want the destination on the 64-byte grid: off it by 4, 16 or 32
+      // bytes a long copy loses 12-17 % (8 x 32 MiB: 80.6 us aligned or off by 64 B, 91.8 us off by
+      // 32 B, 95.5 us off by 4 B; sources off the grid: 80.8 us).  A run of 4 KiB and more whose
+      // destination is off the grid therefore starts its vectors at the next 64-byte boundary
+      // and leaves the bytes before it to the edge workgroups as well.
+      const int64_t max_run = (int64_t)1 << 30; // keeps tile counts inside 32 bits
       if (h.run > max_run) {
         HostBox p = h;
         for (int64_t off = 0; off < h.run; off += max_run) {
@@ -637,9 +690,13 @@ struct Launcher {
         }
         return;
       }
-      if ((h.run & 15) == 0) {
+      if (h.run >= 32) {
+        const uintptr_t off_grid = (uintptr_t)h.dst & 63;
+        const int64_t head = off_grid != 0 && h.run >= kAlignDestinationFrom ? 64 - (int64_t)off_grid : 0;
+        const int64_t rest = h.run - head;
         if (count_piece()) {
-          flat.push_back(Segment{h.src, h.dst, (uint64_t)h.run});
+          flat.push_back(Segment{h.src + head, h.dst + head, (uint64_t)(rest & ~(int64_t)15), (uint8_t)head,
+              (uint8_t)(rest & 15)});
         }
         return;
       }
@@ -751,7 +808,9 @@ void launch_boxes_vec(const Step& st, const CopyArgs& a, hipStream_t stream) {
 
 int launch_step(const Step& st, const FlatArgs* flat, const CopyArgs* boxes, hipStream_t stream) {
   const bool equal = st.grid_y > 0;
-  dim3 g(st.grid, equal ? st.grid_y : 1), b(kBlock);
+  uint32_t gx, gy;
+  launch_dims(st, flat, &gx, &gy);
+  dim3 g(gx, gy), b(kBlock);
 #define MDH_COMMA ,
 #define MDH_LAUNCH_COPY(kernel, more, args)                                                  \
   switch (st.unroll) {                                                                 \
@@ -1099,6 +1158,37 @@ extern "C" int mdh_copy_plan_verify(const mdh_copy_plan* plan, const uint64_t* b
           return MDH_EINVAL;
         }
       }
+      // the edge workgroups: every slot of every segment, through the kernel's own mapping
+      if ((a.edge_wgs != 0) != [&] {
+            for (uint32_t seg = 0; seg < a.nsegs; ++seg) {
+              if (a.head[seg] || a.tail[seg]) {
+                return true;
+              }
+            }
+            return false;
+          }()) {
+        set_error("mdh_copy_plan_verify: step %zu: edge workgroups do not match the segments' heads and tails", s);
+        return MDH_EINVAL;
+      }
+      for (uint32_t seg = 0; seg < a.nsegs && a.edge_wgs; ++seg) {
+        int ss, ds;
+        uint64_t so, dof;
+        split(a.src[seg], &ss, &so);
+        split(a.dst[seg], &ds, &dof);
+        for (uint32_t slot = 0; slot < kEdgeSlots; ++slot) {
+          int64_t off;
+          if (!edge_offset(a, seg, slot, &off)) {
+            continue;
+          }
+          if (off < 0 && ((uint64_t)-off > so || (uint64_t)-off > dof)) {
+            set_error("mdh_copy_plan_verify: step %zu segment %u: head byte before its base", s, seg);
+            return MDH_EINVAL;
+          }
+          if (!move(ss, so + (uint64_t)off, ds, dof + (uint64_t)off, 1, s)) {
+            return MDH_EINVAL;
+          }
+        }
+      }
       continue;
     }
     const CopyArgs& a = st.boxes;
@@ -1267,8 +1357,10 @@ extern "C" int mdh_copy_plan_step_arguments(const mdh_copy_plan* plan, const voi
     from = &boxes;
     *size = sizeof(CopyArgs);
   }
-  if (grid_x) *grid_x = st.grid;
-  if (grid_y) *grid_y = st.grid_y > 0 ? st.grid_y : 1;
+  uint32_t gx, gy;
+  launch_dims(st, st.kind == Step::kFlat ? &flat : nullptr, &gx, &gy);
+  if (grid_x) *grid_x = gx;
+  if (grid_y) *grid_y = gy;
   if (block) *block = (uint32_t)kBlock;
   if (lds) *lds = (uint32_t)st.lds;
   if (out) {

@@ -28,7 +28,7 @@ struct ReduceArgs {
   uint64_t nvec;  // 16-byte vectors on the vector path
   uint64_t numel; // elements from the pointers on: the vectors' and the < 16 bytes after them
   uint32_t head;  // elements BEFORE the pointers (fewer than 64 bytes): see mdh_reduce
-  uint32_t elem_wave; // 1: the last workgroup of the grid folds the head and tail elements, 0: there are none
+  uint32_t elem_wave; // 1: the first workgroup of the grid folds the head and tail elements, 0: there are none
   float scale;
   int nsrc;
   int mode;
@@ -317,18 +317,18 @@ __device__ __forceinline__ void reduce_tile(const ReduceArgs& a, int nsrc, uint6
 // waves round-robin.  Pointers need only element alignment: gfx950's
 // 16-byte buffer accesses take any byte address.  Elements before the pointers (a.head, fewer
 // than 64 bytes) and past the last whole vector (fewer than 16 bytes) are folded by one more
-// workgroup at the end of the grid.
+// workgroup, the first of the grid.
 template<typename T, int F, int U, int CH, bool PREMUL>
 __global__ __launch_bounds__(kWave) void reduce_vec_kernel(ReduceArgs a) {
   const int nsrc = a.nsrc;
   constexpr uint64_t tile_bytes = (uint64_t)kWave * U * 16;
   const uint64_t body_bytes = a.nvec * 16;
   const uint64_t ntiles = (body_bytes + tile_bytes - 1) / tile_bytes;
-  // The head and tail elements have a workgroup of their own, the last of the grid: folded by a
+  // The head and tail elements have a workgroup of their own, the first of the grid: folded by a
   // workgroup that also has tiles, their round trips would come on top of that wave's tiles and
   // lengthen the whole launch (by 1.5 us of 23 for eight sources).
   const uint32_t tile_waves = gridDim.x - a.elem_wave;
-  if (a.elem_wave != 0 && blockIdx.x == tile_waves) {
+  if (blockIdx.x < a.elem_wave) {
     // one element per lane: the head before the pointers (indices -head .. -1, fewer than 64
     // bytes), then the tail after the last whole vector (fewer than 16 bytes): at most 31 + 7 lanes
     const int64_t lane = threadIdx.x, head = a.head;
@@ -341,7 +341,7 @@ __global__ __launch_bounds__(kWave) void reduce_vec_kernel(ReduceArgs a) {
   // The tile waves never outnumber the tiles (a launch with no whole vector has one, whose
   // descriptors are then empty), so the first tile needs no test and the scalar loads of the
   // arguments are not held up behind a load-and-branch.
-  uint64_t tile = blockIdx.x;
+  uint64_t tile = blockIdx.x - a.elem_wave;
   do {
     const uint64_t tile_byte = tile * tile_bytes;
     const uint64_t left = body_bytes - tile_byte;

@@ -50,6 +50,19 @@ def test_strided_gather_and_dense_gather_shapes():
     plan_for(specs, 1).verify(lens + [at])
 
 
+def test_ragged_dense_gathers_are_one_launch_with_heads_and_tails():
+    # shards whose byte length is not a multiple of 16 land at destinations off the 64-byte grid:
+    # the whole vectors start on the grid, heads and tails go to the same launch's edge workgroups
+    for shard, nshards in ((100000 * 2 + 2, 8), (4096 + 1, 64), (1 << 20 | 6, 3), (5000, 8), (33, 5)):
+        specs = [(shard + 64, 1, r * shard + 3, [shard], [1], [1]) for r in range(nshards)]
+        p = plan_for(specs, 1)
+        assert p.launches == 1, (shard, nshards, p.launches)
+        p.verify([shard + 64] * nshards + [nshards * shard + 64])
+    # shorter than two vectors: the narrow kernel's, still verified
+    specs = [(64, 1, r * 21 + 3, [21], [1], [1]) for r in range(4)]
+    plan_for(specs, 1).verify([64] * 4 + [200])
+
+
 @pytest.mark.parametrize("itemsize", [1, 2, 4, 8])
 def test_ragged_rows_transposes_and_many_dimensions(itemsize):
     specs = [
