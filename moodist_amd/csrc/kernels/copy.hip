@@ -248,18 +248,21 @@ struct FlatArgs {
   uint64_t bytes[kMaxSegments];    // of whole vectors: multiples of 16
   // The segment's first bytes, up to its destination's next 64-byte boundary, and its last
   // < 16 bytes: they sit before src/dst and after src/dst + bytes, and are copied byte by byte
-  // by workgroups of their own (edge_wgs of them, in front of the tile workgroups).
+  // by workgroups of their own, in front of the tile workgroups.
   uint8_t head[kMaxSegments]; // 0..63
   uint8_t tail[kMaxSegments]; // 0..15
   uint32_t nsegs;
   uint32_t total_tiles;
   uint32_t tiles_per_seg; // non-zero when every segment has the same tile count
-  uint32_t edge_wgs;      // 0: no segment has a head or a tail
+  uint32_t edge_wgs;      // non-zero: some segment has a head or a tail
 };
 static_assert(sizeof(FlatArgs) <= 4096, "kernel arguments are limited to 4 KiB");
 
 // Edge bytes are numbered per segment: slots 0..63 are the head's bytes, 64..79 the tail's.
 constexpr uint32_t kEdgeSlots = 80;
+// Workgroups that copy them (the one-dimensional form of the grid; segments with edges are never
+// launched in the two-dimensional form): one lane per slot of a full table.
+constexpr uint32_t kEdgeWgs = (kMaxSegments * kEdgeSlots + 255) / 256;
 
 // The byte a slot stands for, as an offset from the segment's src/dst (negative in the head);
 // false for a slot the segment does not use.
@@ -293,10 +296,17 @@ MDH_HD uint32_t locate_segment(const FlatArgs& a, uint32_t tile, uint32_t* local
   return seg;
 }
 
-// Workgroup `wg` of `nwg` edge workgroups: one byte per lane and round.
-__device__ __forceinline__ void copy_edges(const FlatArgs& a, uint32_t wg, uint32_t nwg) {
+// Workgroup `wg` of `nwg` edge workgroups: one byte per lane and round.  Out of line, reading the
+// arguments from the kernel's argument segment (FlatArgs is the kernel's only argument, so it
+// sits at the segment's start): inlined, its loads were scheduled in front of the tile
+// workgroups' own.
+__device__ __attribute__((noinline)) void copy_edges(const FlatArgs* args, uint32_t wg, uint32_t nwg, uint32_t lane) {
+  const FlatArgs& a = *args;
+  if (a.edge_wgs == 0) {
+    return;
+  }
   const uint32_t all = a.nsegs * kEdgeSlots;
-  for (uint32_t idx = wg * kBlock + threadIdx.x; idx < all; idx += nwg * kBlock) {
+  for (uint32_t idx = wg * kBlock + lane; idx < all; idx += nwg * kBlock) {
     const uint32_t seg = idx / kEdgeSlots, slot = idx - seg * kEdgeSlots;
     int64_t off;
     if (edge_offset(a, seg, slot, &off)) {
@@ -305,30 +315,24 @@ __device__ __forceinline__ void copy_edges(const FlatArgs& a, uint32_t wg, uint3
   }
 }
 
-// EQUAL: as for the boxes -- segments of equal tile count, blockIdx.y the segment, blockIdx.x the
-// tile.  Edge workgroups come FIRST in the grid -- row 0 (EQUAL) or workgroups 0 .. edge_wgs-1 --
-// so that their one round trip is over long before the tiles are.
+// EQUAL: as for the boxes -- segments of equal tile count and without heads or tails,
+// blockIdx.y the segment, blockIdx.x the tile.  Otherwise the first kEdgeWgs workgroups of the
+// grid are the edge workgroups -- ALWAYS, finding nothing to do when no segment has a head or a
+// tail: a tile workgroup then knows what it is from blockIdx alone, and its first loads do not
+// wait for a kernel argument to decide it.
 template<int U, bool EQUAL>
 __global__ __launch_bounds__(kBlock) void copy_flat_kernel(FlatArgs a) {
   constexpr uint32_t tile_bytes = kBlock * U * 16;
   const uint32_t lane_byte = threadIdx.x * 16;
-  const uint32_t edge_wgs = a.edge_wgs;
-  uint32_t first_tile = blockIdx.x, tile_wgs = gridDim.x, row = blockIdx.y;
-  if (EQUAL) {
-    if (edge_wgs != 0) { // one more row, in front
-      if (row == 0) {
-        copy_edges(a, blockIdx.x, gridDim.x);
-        return;
-      }
-      row -= 1;
-    }
-  } else {
-    if (blockIdx.x < edge_wgs) {
-      copy_edges(a, blockIdx.x, edge_wgs);
+  uint32_t first_tile = blockIdx.x, tile_wgs = 0;
+  const uint32_t row = blockIdx.y;
+  if (!EQUAL) {
+    if (blockIdx.x < kEdgeWgs) {
+      // the segment's address has to be taken here, in the kernel
+      copy_edges((const FlatArgs*)__builtin_amdgcn_kernarg_segment_ptr(), blockIdx.x, kEdgeWgs, threadIdx.x);
       return;
     }
-    first_tile -= edge_wgs;
-    tile_wgs -= edge_wgs;
+    first_tile = blockIdx.x - kEdgeWgs, tile_wgs = gridDim.x - kEdgeWgs;
   }
   uint32_t tile = first_tile; // untested, as in the box kernels
   do {
@@ -391,15 +395,14 @@ struct Step {
 
 int launch_step(const Step& st, const FlatArgs* flat, const CopyArgs* boxes, hipStream_t stream);
 
-// The grid a step is launched with: st.grid (x st.grid_y) tile workgroups, and for a flat step
-// with edges the edge workgroups in front of them (one more row in the two-dimensional form).
-inline void launch_dims(const Step& st, const FlatArgs* flat, uint32_t* x, uint32_t* y) {
-  const uint32_t edge_wgs = st.kind == Step::kFlat && flat ? flat->edge_wgs : 0;
+// The grid a step is launched with: st.grid (x st.grid_y) tile workgroups, and in the
+// one-dimensional form of a flat step the edge workgroups in front of them.
+inline void launch_dims(const Step& st, uint32_t* x, uint32_t* y) {
   if (st.grid_y > 0) {
     *x = st.grid;
-    *y = st.grid_y + (edge_wgs ? 1u : 0u);
+    *y = st.grid_y;
   } else {
-    *x = st.grid + edge_wgs;
+    *x = st.grid + (st.kind == Step::kFlat ? kEdgeWgs : 0u);
     *y = 1;
   }
 }
@@ -480,8 +483,7 @@ struct Launcher {
       }
       a.total_tiles = (uint32_t)tiles;
       a.tiles_per_seg = equal ? (uint32_t)first_tiles : 0;
-      // one byte per lane: a workgroup for every kBlock edge slots, so that no lane goes round twice
-      a.edge_wgs = edges ? (a.nsegs * kEdgeSlots + (uint32_t)kBlock - 1) / (uint32_t)kBlock : 0;
+      a.edge_wgs = edges ? 1 : 0;
       if (tiles == 0) {
         continue;
       }
@@ -492,7 +494,7 @@ struct Launcher {
       Step st;
       st.kind = Step::kFlat, st.vec = 16, st.unroll = U, st.grid = grid, st.grid_y = 0, st.lds = lds;
       st.plain_loads = false;
-      if (a.tiles_per_seg && grid == a.total_tiles && a.nsegs > 1) {
+      if (a.tiles_per_seg && grid == a.total_tiles && a.nsegs > 1 && !edges) {
         st.grid = a.tiles_per_seg, st.grid_y = a.nsegs;
       }
       submit(st, &a, nullptr);
@@ -809,7 +811,7 @@ void launch_boxes_vec(const Step& st, const CopyArgs& a, hipStream_t stream) {
 int launch_step(const Step& st, const FlatArgs* flat, const CopyArgs* boxes, hipStream_t stream) {
   const bool equal = st.grid_y > 0;
   uint32_t gx, gy;
-  launch_dims(st, flat, &gx, &gy);
+  launch_dims(st, &gx, &gy);
   dim3 g(gx, gy), b(kBlock);
 #define MDH_COMMA ,
 #define MDH_LAUNCH_COPY(kernel, more, args)                                                  \
@@ -1158,6 +1160,10 @@ extern "C" int mdh_copy_plan_verify(const mdh_copy_plan* plan, const uint64_t* b
           return MDH_EINVAL;
         }
       }
+      if (st.grid_y && a.edge_wgs) {
+        set_error("mdh_copy_plan_verify: step %zu: the two-dimensional form has no edge workgroups", s);
+        return MDH_EINVAL;
+      }
       // the edge workgroups: every slot of every segment, through the kernel's own mapping
       if ((a.edge_wgs != 0) != [&] {
             for (uint32_t seg = 0; seg < a.nsegs; ++seg) {
@@ -1358,7 +1364,7 @@ extern "C" int mdh_copy_plan_step_arguments(const mdh_copy_plan* plan, const voi
     *size = sizeof(CopyArgs);
   }
   uint32_t gx, gy;
-  launch_dims(st, st.kind == Step::kFlat ? &flat : nullptr, &gx, &gy);
+  launch_dims(st, &gx, &gy);
   if (grid_x) *grid_x = gx;
   if (grid_y) *grid_y = gy;
   if (block) *block = (uint32_t)kBlock;

@@ -102,7 +102,6 @@ extern "C" int mdh_reduce(const void* const* srcs, int nsrc, int first, void* ds
   a.dst = dst;
   a.numel = numel;
   a.head = 0;
-  a.elem_wave = 0; // set where the grid is chosen
   // Stores want the destination on the 64-byte grid: a wave's 1 KiB store whose ends fall
   // inside 64-byte units costs about 6 % of a launch (22.8 us aligned or off by 64 B, 24.2 us off
   // by 4, 16 or 32 B), loads off the grid 1 %.  When the destination is off the grid and there is

@@ -28,7 +28,6 @@ struct ReduceArgs {
   uint64_t nvec;  // 16-byte vectors on the vector path
   uint64_t numel; // elements from the pointers on: the vectors' and the < 16 bytes after them
   uint32_t head;  // elements BEFORE the pointers (fewer than 64 bytes): see mdh_reduce
-  uint32_t elem_wave; // 1: the first workgroup of the grid folds the head and tail elements, 0: there are none
   float scale;
   int nsrc;
   int mode;
@@ -245,6 +244,20 @@ __device__ __forceinline__ void reduce_one_elem(const ReduceArgs& a, int nsrc, i
   ((elem_t*)a.dst)[i] = Tr::template finish<F>(acc, a.mode, a.scale);
 }
 
+// The head before the pointers (indices -head .. -1, fewer than 64 bytes) and the tail after the
+// last whole vector (fewer than 16 bytes), one element per lane: at most 31 + 7 lanes.  Kept out
+// of line: inlined into the kernel, its scalar loads were scheduled in front of the tile
+// workgroups' own and cost them a second scalar round trip (0.35 us of 23).
+template<typename T, int F>
+__device__ __attribute__((noinline)) void reduce_head_and_tail(const ReduceArgs* args, uint32_t lane_id) {
+  const ReduceArgs& a = *args;
+  const int64_t lane = lane_id, head = a.head;
+  const int64_t i = lane < head ? lane - head : (int64_t)(a.nvec * per_vec<T>()) + (lane - head);
+  if (i < (int64_t)a.numel) {
+    reduce_one_elem<T, F>(a, a.nsrc, i);
+  }
+}
+
 // The sources left over when the count is not a multiple of CH (1 .. CH-1 of them).
 template<typename T, int F, int U, int CH, int MODE, bool FIRST, int R = CH - 1>
 __device__ __forceinline__ void fold_rest(const ReduceArgs& a, int rest, int j0, uint64_t tile_byte,
@@ -316,32 +329,33 @@ __device__ __forceinline__ void reduce_tile(const ReduceArgs& a, int nsrc, uint6
 // A tile is kWave*U consecutive 16-byte vectors (U KiB); tiles are dealt to
 // waves round-robin.  Pointers need only element alignment: gfx950's
 // 16-byte buffer accesses take any byte address.  Elements before the pointers (a.head, fewer
-// than 64 bytes) and past the last whole vector (fewer than 16 bytes) are folded by one more
-// workgroup, the first of the grid.
+// than 64 bytes) and past the last whole vector (fewer than 16 bytes) are folded by workgroup 0,
+// which has no tiles.
 template<typename T, int F, int U, int CH, bool PREMUL>
 __global__ __launch_bounds__(kWave) void reduce_vec_kernel(ReduceArgs a) {
   const int nsrc = a.nsrc;
   constexpr uint64_t tile_bytes = (uint64_t)kWave * U * 16;
   const uint64_t body_bytes = a.nvec * 16;
   const uint64_t ntiles = (body_bytes + tile_bytes - 1) / tile_bytes;
-  // The head and tail elements have a workgroup of their own, the first of the grid: folded by a
-  // workgroup that also has tiles, their round trips would come on top of that wave's tiles and
-  // lengthen the whole launch (by 1.5 us of 23 for eight sources).
-  const uint32_t tile_waves = gridDim.x - a.elem_wave;
-  if (blockIdx.x < a.elem_wave) {
-    // one element per lane: the head before the pointers (indices -head .. -1, fewer than 64
-    // bytes), then the tail after the last whole vector (fewer than 16 bytes): at most 31 + 7 lanes
-    const int64_t lane = threadIdx.x, head = a.head;
-    const int64_t i = lane < head ? lane - head : (int64_t)(a.nvec * per_vec<T>()) + (lane - head);
-    if (i < (int64_t)a.numel) {
-      reduce_one_elem<T, F>(a, nsrc, i);
-    }
+  // The head and tail elements have a workgroup of their own, workgroup 0 of every launch
+  // (which finds nothing to do when there are none): folded by a workgroup that also has
+  // tiles, their round trips would come on top of that wave's tiles and lengthen the whole
+  // launch (by 1.5 us of 23 for eight sources).  That it is ALWAYS workgroup 0 lets the tile
+  // workgroups know what they are from blockIdx alone: a test that needed a kernel argument
+  // held their first loads up behind one more scalar round trip (0.4 us of 23).
+  if (blockIdx.x == 0) {
+    // ReduceArgs is the kernel's only argument, so it sits at the start of the argument segment:
+    // the function reads it from there.  (The address of the kernel's own parameter would make
+    // every wave of the launch copy the struct to its stack first; and the segment's address has
+    // to be taken here, in the kernel -- inside a called function the builtin yields null.)
+    reduce_head_and_tail<T, F>((const ReduceArgs*)__builtin_amdgcn_kernarg_segment_ptr(), threadIdx.x);
     return;
   }
-  // The tile waves never outnumber the tiles (a launch with no whole vector has one, whose
+  // The tile workgroups never outnumber the tiles (a launch with no whole vector has one, whose
   // descriptors are then empty), so the first tile needs no test and the scalar loads of the
   // arguments are not held up behind a load-and-branch.
-  uint64_t tile = blockIdx.x - a.elem_wave;
+  const uint32_t tile_waves = gridDim.x - 1;
+  uint64_t tile = blockIdx.x - 1;
   do {
     const uint64_t tile_byte = tile * tile_bytes;
     const uint64_t left = body_bytes - tile_byte;
@@ -479,9 +493,8 @@ template<typename T, int F, bool PREMUL>
 int launch_one(const ReduceArgs& a0, hipStream_t stream) {
   const Tuning& t = tuning();
   const LaunchShape shape = choose_shape<T, PREMUL>(a0);
-  ReduceArgs a = a0;
-  a.elem_wave = (a.head != 0 || a.numel > a.nvec * (16 / sizeof(typename Traits<T>::elem_t))) ? 1u : 0u;
-  dim3 g((unsigned)shape.waves + a.elem_wave), b(kWave);
+  const ReduceArgs& a = a0;
+  dim3 g((unsigned)shape.waves + 1), b(kWave); // workgroup 0 takes the head and tail elements
   // reduce_wg_per_cu (measurement only): an unused LDS allocation caps the waves resident on a CU
   const int cap = t.reduce_wg_per_cu >= 2 && t.reduce_wg_per_cu <= 8 ? t.reduce_wg_per_cu : 0;
   const size_t lds = kLdsForCap[cap];
