@@ -26,17 +26,17 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 CLOCK_WARMUP_S = 0.3   # untimed launches before the first timed window
 TIMED_WINDOWS = 11     # windows of `steps` launches; the median window is reported
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch), each
-# scaled by what the same counter reads for the flat copy of exactly 256 MiB (FETCH_SIZE x 1.99982,
+# scaled by what the same counter reads for the flat copy of exactly 256 MiB (FETCH_SIZE x 1.99991,
 # WRITE_SIZE x 1.00000): profiles/hbm_traffic_pmc_reduce_and_copy_kernels.md.  E.g. the headline:
-# 65,557.89 x 1.99982 + 16,384.00 KiB = 147,488.2 KiB.  Workloads without an entry were not measured.
+# 65,557.74 x 1.99991 + 16,384.00 KiB = 147,493.5 KiB.  Workloads without an entry were not measured.
 MEASURED_TRAFFIC_BYTES = {
-    "reduce_fp32_p8": 151027962,
-    "reduce_bf16_p16": 1140846489,
-    "reduce_fp32_p64_sum": 272661054,
+    "reduce_fp32_p8": 151033315,
+    "reduce_bf16_p16": 1140899332,
+    "reduce_fp32_p64_sum": 272677851,
     "allgather_bf16_p8": 536870912,
-    "allgather_bf16_p8_strided": 536886304,
-    "redistribute_fp32_8192": 67145620,
-    "redistribute_bf16_3d": 16814970,
+    "allgather_bf16_p8_strided": 536907828,
+    "redistribute_fp32_8192": 67157194,
+    "redistribute_bf16_3d": 16825569,
 }
 
 def build_workload(name, torch, abi, dev, rotation_bytes):
