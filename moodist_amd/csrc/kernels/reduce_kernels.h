@@ -168,9 +168,10 @@ constexpr int kWave = 64;
 // buffer descriptor whose base is the tile's first byte (wave-uniform, in
 // SGPRs) and whose size is the bytes left in the tile: the lane offset is one
 // VGPR, and vectors past the end read as zero instead of needing a predicate.
-template<typename T, int F, int CNT, int U, int MODE, bool FIRST>
-__device__ __forceinline__ void fold_chunk(const ReduceArgs& a, int j0, uint64_t tile_byte, uint32_t tile_bytes,
-    uint32_t lane_byte, typename Traits<T>::acc_t (&acc)[U][per_vec<T>()]) {
+template<typename T, int F, int CNT, int U, int MODE, bool FIRST, int NP>
+__device__ __forceinline__ void fold_chunk(const ReduceArgs& a, const char* const (&src)[NP], uint64_t tile_byte,
+    uint32_t tile_bytes, uint32_t lane_byte, typename Traits<T>::acc_t (&acc)[U][per_vec<T>()]) {
+  static_assert(CNT <= NP, "a chunk has at most NP sources");
   using Tr = Traits<T>;
   using elem_t = typename Tr::elem_t;
   using acc_t = typename Tr::acc_t;
@@ -178,7 +179,7 @@ __device__ __forceinline__ void fold_chunk(const ReduceArgs& a, int j0, uint64_t
   u32x4 v[CNT][U];
 #pragma unroll
   for (int k = 0; k < CNT; ++k) {
-    const __amdgpu_buffer_rsrc_t rs = tile_rsrc((const char*)a.src[j0 + k] + tile_byte, tile_bytes);
+    const __amdgpu_buffer_rsrc_t rs = tile_rsrc(src[k] + tile_byte, tile_bytes);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       v[k][u] = tile_load(rs, lane_byte + (uint32_t)u * (kWave * 16));
@@ -260,13 +261,13 @@ __device__ __attribute__((noinline)) void reduce_head_and_tail(const ReduceArgs*
 
 // The sources left over when the count is not a multiple of CH (1 .. CH-1 of them).
 template<typename T, int F, int U, int CH, int MODE, bool FIRST, int R = CH - 1>
-__device__ __forceinline__ void fold_rest(const ReduceArgs& a, int rest, int j0, uint64_t tile_byte,
+__device__ __forceinline__ void fold_rest(const ReduceArgs& a, int rest, const char* const (&src)[CH], uint64_t tile_byte,
     uint32_t tile_bytes, uint32_t lane_byte, typename Traits<T>::acc_t (&acc)[U][per_vec<T>()]) {
   if constexpr (R >= 1) {
     if (rest == R) {
-      fold_chunk<T, F, R, U, MODE, FIRST>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
+      fold_chunk<T, F, R, U, MODE, FIRST>(a, src, tile_byte, tile_bytes, lane_byte, acc);
     } else {
-      fold_rest<T, F, U, CH, MODE, FIRST, R - 1>(a, rest, j0, tile_byte, tile_bytes, lane_byte, acc);
+      fold_rest<T, F, U, CH, MODE, FIRST, R - 1>(a, rest, src, tile_byte, tile_bytes, lane_byte, acc);
     }
   }
 }
@@ -281,16 +282,35 @@ __device__ __forceinline__ void reduce_tile(const ReduceArgs& a, int nsrc, uint6
   constexpr int N = per_vec<T>();
   const uint32_t lane_byte = threadIdx.x * 16;
   acc_t acc[U][N];
+  // The pointers of a group are read from the argument table one group AHEAD of their use: read
+  // when needed, every group would start with a scalar round trip during which the wave has no
+  // load in flight.  (Slots past the last source are never used; 63 is the table's last index.)
+  auto pointers = [&](int first, const char* (&p)[CH]) {
+#pragma unroll
+    for (int k = 0; k < CH; ++k) {
+      const int j = first + k;
+      p[k] = (const char*)a.src[j < MDH_MAX_SOURCES ? j : MDH_MAX_SOURCES - 1];
+    }
+  };
+  const char* cur[CH];
+  const char* nxt[CH];
+  pointers(0, cur);
+  pointers(CH, nxt);
   // the first group is peeled so that "initialise or fold" is decided at compile time
   if (nsrc >= CH) {
-    fold_chunk<T, F, CH, U, MODE, true>(a, 0, tile_byte, tile_bytes, lane_byte, acc);
+    fold_chunk<T, F, CH, U, MODE, true>(a, cur, tile_byte, tile_bytes, lane_byte, acc);
     int j0 = CH;
     for (; nsrc - j0 >= CH; j0 += CH) {
-      fold_chunk<T, F, CH, U, MODE, false>(a, j0, tile_byte, tile_bytes, lane_byte, acc);
+#pragma unroll
+      for (int k = 0; k < CH; ++k) {
+        cur[k] = nxt[k];
+      }
+      pointers(j0 + CH, nxt);
+      fold_chunk<T, F, CH, U, MODE, false>(a, cur, tile_byte, tile_bytes, lane_byte, acc);
     }
-    fold_rest<T, F, U, CH, MODE, false>(a, nsrc - j0, j0, tile_byte, tile_bytes, lane_byte, acc);
+    fold_rest<T, F, U, CH, MODE, false>(a, nsrc - j0, nxt, tile_byte, tile_bytes, lane_byte, acc);
   } else {
-    fold_rest<T, F, U, CH, MODE, true>(a, nsrc, 0, tile_byte, tile_bytes, lane_byte, acc);
+    fold_rest<T, F, U, CH, MODE, true>(a, nsrc, cur, tile_byte, tile_bytes, lane_byte, acc);
   }
   const __amdgpu_buffer_rsrc_t rd = tile_rsrc((const char*)a.dst + tile_byte, tile_bytes);
   u32x4 out[U];
