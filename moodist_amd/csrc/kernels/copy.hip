@@ -195,6 +195,17 @@ __global__ __launch_bounds__(kBlock) void copy_boxes_kernel(CopyArgs a) {
 // of columns out of every row: 3.92 / 4.60, 6.92 / 7.79 and 10.91 / 12.85 -- plain loads may then
 // hit in that cache, nt loads go past it.  A caller that knows its sources to be freshly
 // written and small can ask for them with the knob.
+// A box's descriptor, read from the argument table in ONE batch of scalar loads: every field the
+// common case needs passes through an empty asm statement, which the compiler has to have all of
+// them ready for at once.  Left to itself it reads each field where it is first used, behind the
+// branches of the index arithmetic: four scalar round trips in a row before the first vector
+// load, in launches that last 5 us.
+__device__ __forceinline__ void read_at_once(const BoxDesc& B) {
+  asm volatile("" ::"s"((uint64_t)(uintptr_t)B.src), "s"((uint64_t)(uintptr_t)B.dst), "s"((uint64_t)B.src_stride[0]),
+               "s"((uint64_t)B.dst_stride[0]), "s"(B.nouter), "s"(B.rows), "s"(B.cols), "s"(B.nct), "s"(B.log2tc),
+               "s"(B.src_span), "s"(B.dst_span));
+}
+
 template<int U, bool EQUAL, bool PLAIN>
 __global__ __launch_bounds__(kBlock) void copy_boxes16_kernel(CopyArgs a) {
   constexpr int kLoad = PLAIN ? 0 : 2;
@@ -204,6 +215,7 @@ __global__ __launch_bounds__(kBlock) void copy_boxes16_kernel(CopyArgs a) {
   do {
     TileLoc t;
     if (EQUAL) {
+      read_at_once(a.box[blockIdx.y]);
       const uint32_t nct = a.box[blockIdx.y].nct;
       const uint32_t rt = blockIdx.x / nct;
       t = TileLoc{blockIdx.y, rt, blockIdx.x - rt * nct};
