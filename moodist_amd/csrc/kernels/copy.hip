@@ -37,6 +37,11 @@ struct BoxDesc {
   uint32_t log2tc;
   uint32_t src_span; // bytes from src to the end of the box, when both spans fit 32 bits (else 0)
   uint32_t dst_span;
+  // Byte offset of a row's LAST vector.  (cols - 1) * vector width when the row is a whole number
+  // of vectors; a row of the 16-byte kernel that is not has one vector more, and that last one
+  // ends where the row ends: it overlaps the one before it, and the bytes they share are
+  // copied twice, to the same effect.
+  uint32_t last_off;
 };
 
 struct CopyArgs {
@@ -136,8 +141,9 @@ MDH_HD bool slot_offsets(const BoxDesc& B, const TileLoc& t, uint32_t slot, uint
     s += (Off)row * (Off)B.src_stride[B.nouter - 1];
     d += (Off)row * (Off)B.dst_stride[B.nouter - 1];
   }
-  *so = s + (Off)col * (Off)vec;
-  *dof = d + (Off)col * (Off)vec;
+  const uint32_t in_row = col * vec < B.last_off ? col * vec : B.last_off;
+  *so = s + (Off)in_row;
+  *dof = d + (Off)in_row;
   return ok;
 }
 
@@ -203,7 +209,7 @@ __global__ __launch_bounds__(kBlock) void copy_boxes_kernel(CopyArgs a) {
 __device__ __forceinline__ void read_at_once(const BoxDesc& B) {
   asm volatile("" ::"s"((uint64_t)(uintptr_t)B.src), "s"((uint64_t)(uintptr_t)B.dst), "s"((uint64_t)B.src_stride[0]),
                "s"((uint64_t)B.dst_stride[0]), "s"(B.nouter), "s"(B.rows), "s"(B.cols), "s"(B.nct), "s"(B.log2tc),
-               "s"(B.src_span), "s"(B.dst_span));
+               "s"(B.src_span), "s"(B.dst_span), "s"(B.last_off));
 }
 
 template<int U, bool EQUAL, bool PLAIN>
@@ -571,9 +577,18 @@ struct Launcher {
       bool equal = true;
       while (i < list.size() && a.nboxes < (uint32_t)kMaxBoxes) {
         BoxDesc d = list[i];
+        // Tile width: the power of two that covers the row, or the tile -- unless the column
+        // tiles of that width would be more than a sixteenth empty (a row of 513 vectors in tiles
+        // of 512 columns is two tiles, the second with one column in use: a gather of rows of
+        // 8200 bytes took 114 us, against 80 us for rows of 8192); then the widest that is not,
+        // down to 16 columns (256 bytes of a row per wave instruction) if the rows are many.
         uint32_t tc = 1, log2tc = 0;
         while (tc < d.cols && tc < slots) {
           tc <<= 1, ++log2tc;
+        }
+        while (tc > 16 && (slots >> (log2tc - 1)) <= d.rows &&
+               (uint64_t)((d.cols + tc - 1) / tc) * tc * 16 > (uint64_t)d.cols * 17) {
+          tc >>= 1, --log2tc;
         }
         const uint32_t tr = slots >> log2tc;
         d.log2tc = log2tc;
@@ -660,6 +675,7 @@ struct Launcher {
     }
     d.rows = (uint32_t)rows;
     d.cols = (uint32_t)(h.run / vec);
+    d.last_off = (d.cols - 1) * (uint32_t)vec;
     d.nct = d.log2tc = 0;
     d.src_span = d.dst_span = 0;
     uint64_t sspan = (uint64_t)h.run, dspan = (uint64_t)h.run;
@@ -668,8 +684,9 @@ struct Launcher {
       dspan += (uint64_t)(h.shape[k] - 1) * (uint64_t)h.dstride[k];
     }
     // (any byte alignment of bases and strides: the buffer path does not need it)
-    if ((h.run & 15) == 0 && sspan < 0xffffff00ull && dspan < 0xffffff00ull) {
-      d.cols = (uint32_t)(h.run / 16);
+    if (h.run >= 16 && sspan < 0xffffff00ull && dspan < 0xffffff00ull) {
+      d.cols = (uint32_t)((h.run + 15) / 16);
+      d.last_off = (uint32_t)(h.run - 16);
       d.src_span = (uint32_t)sspan;
       d.dst_span = (uint32_t)dspan;
       pending16.push_back(d);
@@ -737,19 +754,22 @@ struct Launcher {
       }
       return;
     }
-    if ((h.run & 15) && h.run >= 32) {
-      // Rows that are not a multiple of 16 bytes long would move as 1-, 2-, 4- or 8-byte vectors
-      // (0.6-1.7 TB/s on 4 KiB rows).  Their first run & ~15 bytes go as 16-byte vectors, which
-      // the buffer path takes at any alignment, and the last < 16 bytes of every row as a box
-      // of its own.
+    // Rows of 16 bytes and more that are not a whole number of 16-byte vectors go to the 16-byte
+    // kernel all the same, their last vector pulled back to end with the row (emit): 8 x 4096 rows
+    // of 8194 bytes 94 us, 8 x 1024 rows of 4098 bytes 15.7 us, against 97 and 16.4 us with the
+    // tails split off into a box for the narrow kernel.  Only tails that the narrow kernel moves
+    // as 8-byte vectors are still split off: rows of 8200 bytes 85.6 us split, 91.8 us not.
+    if (h.run >= 32 && (h.run & 15) == 8) {
       HostBox body = h, tail = h;
-      body.run = h.run & ~(int64_t)15;
+      body.run = h.run - 8;
       tail.src = h.src + body.run;
       tail.dst = h.dst + body.run;
-      tail.run = h.run & 15;
-      emit(body);
-      emit(tail);
-      return;
+      tail.run = 8;
+      if (vec_width(tail) == 8) {
+        emit(body);
+        emit(tail);
+        return;
+      }
     }
     emit(h);
   }
@@ -1066,6 +1086,7 @@ extern "C" int mdh_copy_plan_verify(const mdh_copy_plan* plan, const uint64_t* b
   }
   // For every destination byte: 1 + (source slot << 40 | source byte), 0 = not written.
   std::vector<std::vector<uint64_t>> expect((size_t)nbases), got((size_t)nbases);
+  std::vector<std::vector<uint8_t>> repeatable((size_t)nbases); // bytes a ragged row's last vector has written
   auto dest = [&](std::vector<std::vector<uint64_t>>& m, int slot) -> std::vector<uint64_t>& {
     if (m[(size_t)slot].empty()) {
       m[(size_t)slot].assign((size_t)base_bytes[slot], 0);
@@ -1113,7 +1134,9 @@ extern "C" int mdh_copy_plan_verify(const mdh_copy_plan* plan, const uint64_t* b
     *slot = (int)(v >> kSlotShift) - 1;
     *off = v & kOffsetMask;
   };
-  auto move = [&](int ss, uint64_t so, int ds, uint64_t dof, uint32_t n, size_t step) -> bool {
+  // may_repeat: a ragged row's last vector, which overlaps the one before it -- a byte may then
+  // be written a second time, with the same source byte
+  auto move = [&](int ss, uint64_t so, int ds, uint64_t dof, uint32_t n, size_t step, bool may_repeat = false) -> bool {
     if (ss < 0 || ss >= nbases || ds < 0 || ds >= nbases || so + n > base_bytes[ss] || dof + n > base_bytes[ds]) {
       set_error("mdh_copy_plan_verify: step %zu moves %u bytes from base %d + %llu to base %d + %llu: outside the bases", step, n,
           ss, (unsigned long long)so, ds, (unsigned long long)dof);
@@ -1121,11 +1144,18 @@ extern "C" int mdh_copy_plan_verify(const mdh_copy_plan* plan, const uint64_t* b
     }
     std::vector<uint64_t>& m = dest(got, ds);
     for (uint32_t k = 0; k < n; ++k) {
-      if (m[dof + k]) {
+      const uint64_t what = 1 + (((uint64_t)ss << 40) | (so + k));
+      if (m[dof + k] && !(m[dof + k] == what && (may_repeat || repeatable[(size_t)ds][dof + k]))) {
         set_error("mdh_copy_plan_verify: step %zu writes base %d byte %llu a second time", step, ds, (unsigned long long)(dof + k));
         return false;
       }
-      m[dof + k] = 1 + (((uint64_t)ss << 40) | (so + k));
+      m[dof + k] = what;
+      if (may_repeat) {
+        if (repeatable[(size_t)ds].empty()) {
+          repeatable[(size_t)ds].assign((size_t)base_bytes[ds], 0);
+        }
+        repeatable[(size_t)ds][dof + k] = 1;
+      }
     }
     return true;
   };
@@ -1247,7 +1277,10 @@ extern "C" int mdh_copy_plan_verify(const mdh_copy_plan* plan, const uint64_t* b
           }
           so = (uint64_t)so64, dof = (uint64_t)dof64;
         }
-        if (!move(ss, sbase + so, ds, dbase + dof, buffer16 ? 16u : (uint32_t)st.vec, s)) {
+        // the last vector of a row that is not a whole number of vectors overlaps the one before
+        const uint32_t col = (t.ct << B.log2tc) + (slot & ((1u << B.log2tc) - 1u));
+        const bool pulled_back = buffer16 && (B.last_off & 15) != 0 && col == B.cols - 1;
+        if (!move(ss, sbase + so, ds, dbase + dof, buffer16 ? 16u : (uint32_t)st.vec, s, pulled_back)) {
           return MDH_EINVAL;
         }
       }
