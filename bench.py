@@ -30,13 +30,13 @@ TIMED_WINDOWS = 11     # windows of `steps` launches; the median window is repor
 # WRITE_SIZE x 1.00000): profiles/hbm_traffic_pmc_reduce_and_copy_kernels.md.  E.g. the headline:
 # 65,557.74 x 1.99991 + 16,384.00 KiB = 147,493.5 KiB.  Workloads without an entry were not measured.
 MEASURED_TRAFFIC_BYTES = {
-    "reduce_fp32_p8": 151035242,
-    "reduce_bf16_p16": 1140900006,
-    "reduce_fp32_p64_sum": 272677757,
+    "reduce_fp32_p8": 151035164,
+    "reduce_bf16_p16": 1140899908,
+    "reduce_fp32_p64_sum": 272677707,
     "allgather_bf16_p8": 536870912,
-    "allgather_bf16_p8_strided": 536906807,
-    "redistribute_fp32_8192": 67156080,
-    "redistribute_bf16_3d": 16824549,
+    "allgather_bf16_p8_strided": 536907740,
+    "redistribute_fp32_8192": 67157159,
+    "redistribute_bf16_3d": 16825558,
 }
 
 def build_workload(name, torch, abi, dev, rotation_bytes):
