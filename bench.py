@@ -28,7 +28,7 @@ TIMED_WINDOWS = 11     # windows of `steps` launches; the median window is repor
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch), each
 # scaled by what the same counter reads for the flat copy of exactly 256 MiB (FETCH_SIZE x 1.99991,
 # WRITE_SIZE x 1.00000): profiles/hbm_traffic_pmc_reduce_and_copy_kernels.md.  E.g. the headline:
-# 65,557.74 x 1.99991 + 16,384.00 KiB = 147,493.5 KiB.  Workloads without an entry were not measured.
+# 65,558.66 x 1.99991 + 16,384.00 KiB = 147,495.3 KiB.  Workloads without an entry were not measured.
 MEASURED_TRAFFIC_BYTES = {
     "reduce_fp32_p8": 151035164,
     "reduce_bf16_p16": 1140899908,
