@@ -28,15 +28,15 @@ TIMED_WINDOWS = 11     # windows of `steps` launches; the median window is repor
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch), each
 # scaled by what the same counter reads for the flat copy of exactly 256 MiB (FETCH_SIZE x 1.99991,
 # WRITE_SIZE x 1.00000): profiles/hbm_traffic_pmc_reduce_and_copy_kernels.md.  E.g. the headline:
-# 65,558.66 x 1.99991 + 16,384.00 KiB = 147,495.3 KiB.  Workloads without an entry were not measured.
+# 65,560.67 x 1.99991 + 16,384.00 KiB = 147,499.3 KiB.  Workloads without an entry were not measured.
 MEASURED_TRAFFIC_BYTES = {
-    "reduce_fp32_p8": 151035164,
-    "reduce_bf16_p16": 1140899908,
-    "reduce_fp32_p64_sum": 272677707,
+    "reduce_fp32_p8": 151039298,
+    "reduce_bf16_p16": 1140903999,
+    "reduce_fp32_p64_sum": 272678699,
     "allgather_bf16_p8": 536870912,
-    "allgather_bf16_p8_strided": 536907740,
-    "redistribute_fp32_8192": 67157159,
-    "redistribute_bf16_3d": 16825558,
+    "allgather_bf16_p8_strided": 536907804,
+    "redistribute_fp32_8192": 67156846,
+    "redistribute_bf16_3d": 16825561,
 }
 
 def build_workload(name, torch, abi, dev, rotation_bytes):

@@ -8,8 +8,11 @@ out="${1:-$here/../libmoodist_hip.so}"
 extra="${MDH_EXTRA_FLAGS:-}"
 tag="$(echo "$extra" | tr -c 'A-Za-z0-9\n' '_')"
 jobs="${MDH_BUILD_JOBS:-8}"
+# -amdgpu-kernarg-preload-count: a kernel's leading scalar arguments (14 dwords at most) are in
+# registers when a wave starts; reduce_vec_kernel's are laid out for it.
 flags=(-O3 -std=c++17 -fPIC --offload-arch=gfx950 -ffp-contract=off
        -Xclang -target-feature -Xclang -packed-fp32-ops
+       -mllvm -amdgpu-kernarg-preload-count=14
        -I"$root/include" -I"$here/kernels" -Wall -Wno-unused-function -Wno-unused-const-variable $extra)
 bdir="$here/build"
 mkdir -p "$bdir"

@@ -72,7 +72,7 @@ extern "C" int mdh_reduce(const void* const* srcs, int nsrc, int first, void* ds
     set_error("mdh_reduce: null pointer");
     return MDH_EINVAL;
   }
-  ReduceArgs a;
+  ReduceArgs a{}; // unused source slots stay null
   const uintptr_t bytes = (uintptr_t)numel * itemsize;
   for (int j = 0; j < nsrc; ++j) {
     const void* p = srcs[(first + j) % nsrc];

@@ -33,6 +33,14 @@ struct ReduceArgs {
   int mode;
 };
 
+// reduce_vec_kernel's leading arguments (see there): vector count, tile workgroups, source count
+// and mode, scale, then this many source pointers -- fourteen dwords with the padding in front
+// of the pointers; ReduceArgs follows them in the argument segment.
+constexpr int kEarlySources = 4;
+constexpr size_t kArgsOffset = 8 + 4 + 4 + 4 + 4 + 8 * kEarlySources;
+static_assert(alignof(ReduceArgs) == 8 && kArgsOffset % alignof(ReduceArgs) == 0, "ReduceArgs follows the leading arguments without padding");
+static_assert(MDH_MAX_SOURCES < 256, "the source count travels in one byte");
+
 struct bf16_t {
   uint16_t bits;
 };
@@ -169,7 +177,7 @@ constexpr int kWave = 64;
 // SGPRs) and whose size is the bytes left in the tile: the lane offset is one
 // VGPR, and vectors past the end read as zero instead of needing a predicate.
 template<typename T, int F, int CNT, int U, int MODE, bool FIRST, int NP>
-__device__ __forceinline__ void fold_chunk(const ReduceArgs& a, const char* const (&src)[NP], uint64_t tile_byte,
+__device__ __forceinline__ void fold_chunk(float scale, const char* const (&src)[NP], uint64_t tile_byte,
     uint32_t tile_bytes, uint32_t lane_byte, typename Traits<T>::acc_t (&acc)[U][per_vec<T>()]) {
   static_assert(CNT <= NP, "a chunk has at most NP sources");
   using Tr = Traits<T>;
@@ -198,7 +206,7 @@ __device__ __forceinline__ void fold_chunk(const ReduceArgs& a, const char* cons
       for (int i = 0; i < N; ++i) {
         acc_t x = Tr::widen(e[i]);
         if constexpr (MODE == kPremul) {
-          x = Tr::premul(x, a.scale);
+          x = Tr::premul(x, scale);
         }
         if (FIRST && k == 0) {
           acc[u][i] = x; // the first source initialises the accumulator (the reference's memcpy)
@@ -261,13 +269,13 @@ __device__ __attribute__((noinline)) void reduce_head_and_tail(const ReduceArgs*
 
 // The sources left over when the count is not a multiple of CH (1 .. CH-1 of them).
 template<typename T, int F, int U, int CH, int MODE, bool FIRST, int R = CH - 1>
-__device__ __forceinline__ void fold_rest(const ReduceArgs& a, int rest, const char* const (&src)[CH], uint64_t tile_byte,
+__device__ __forceinline__ void fold_rest(float scale, int rest, const char* const (&src)[CH], uint64_t tile_byte,
     uint32_t tile_bytes, uint32_t lane_byte, typename Traits<T>::acc_t (&acc)[U][per_vec<T>()]) {
   if constexpr (R >= 1) {
     if (rest == R) {
-      fold_chunk<T, F, R, U, MODE, FIRST>(a, src, tile_byte, tile_bytes, lane_byte, acc);
+      fold_chunk<T, F, R, U, MODE, FIRST>(scale, src, tile_byte, tile_bytes, lane_byte, acc);
     } else {
-      fold_rest<T, F, U, CH, MODE, FIRST, R - 1>(a, rest, src, tile_byte, tile_bytes, lane_byte, acc);
+      fold_rest<T, F, U, CH, MODE, FIRST, R - 1>(scale, rest, src, tile_byte, tile_bytes, lane_byte, acc);
     }
   }
 }
@@ -275,7 +283,8 @@ __device__ __forceinline__ void fold_rest(const ReduceArgs& a, int rest, const c
 // One tile: U KiB of every source (U sub-tiles of one wave-wide 16-byte load each), consumed CH
 // sources at a time in order, so the fold stays a left fold and CH*U loads are in flight.
 template<typename T, int F, int U, int CH, int MODE>
-__device__ __forceinline__ void reduce_tile(const ReduceArgs& a, int nsrc, uint64_t tile_byte, uint32_t tile_bytes) {
+__device__ __forceinline__ void reduce_tile(const ReduceArgs& a, const char* const (&early)[kEarlySources], int nsrc,
+    int mode_arg, float scale, uint64_t tile_byte, uint32_t tile_bytes) {
   using Tr = Traits<T>;
   using elem_t = typename Tr::elem_t;
   using acc_t = typename Tr::acc_t;
@@ -292,13 +301,24 @@ __device__ __forceinline__ void reduce_tile(const ReduceArgs& a, int nsrc, uint6
       p[k] = (const char*)a.src[j < MDH_MAX_SOURCES ? j : MDH_MAX_SOURCES - 1];
     }
   };
+  // The first two groups' indices are compile-time constants: those below kEarlySources are
+  // the kernel's leading arguments, in registers when the wave starts, so the first vector
+  // loads wait for no scalar load at all.
+  auto early_pointers = [&](auto first, const char* (&p)[CH]) {
+#pragma unroll
+    for (int k = 0; k < CH; ++k) {
+      constexpr int kFirst = decltype(first)::value;
+      const int j = kFirst + k;
+      p[k] = j < kEarlySources ? early[j < kEarlySources ? j : 0] : (const char*)a.src[j < MDH_MAX_SOURCES ? j : MDH_MAX_SOURCES - 1];
+    }
+  };
   const char* cur[CH];
   const char* nxt[CH];
-  pointers(0, cur);
-  pointers(CH, nxt);
+  early_pointers(std::integral_constant<int, 0>{}, cur);
+  early_pointers(std::integral_constant<int, CH>{}, nxt);
   // the first group is peeled so that "initialise or fold" is decided at compile time
   if (nsrc >= CH) {
-    fold_chunk<T, F, CH, U, MODE, true>(a, cur, tile_byte, tile_bytes, lane_byte, acc);
+    fold_chunk<T, F, CH, U, MODE, true>(scale, cur, tile_byte, tile_bytes, lane_byte, acc);
     int j0 = CH;
     for (; nsrc - j0 >= CH; j0 += CH) {
 #pragma unroll
@@ -306,23 +326,23 @@ __device__ __forceinline__ void reduce_tile(const ReduceArgs& a, int nsrc, uint6
         cur[k] = nxt[k];
       }
       pointers(j0 + CH, nxt);
-      fold_chunk<T, F, CH, U, MODE, false>(a, cur, tile_byte, tile_bytes, lane_byte, acc);
+      fold_chunk<T, F, CH, U, MODE, false>(scale, cur, tile_byte, tile_bytes, lane_byte, acc);
     }
-    fold_rest<T, F, U, CH, MODE, false>(a, nsrc - j0, nxt, tile_byte, tile_bytes, lane_byte, acc);
+    fold_rest<T, F, U, CH, MODE, false>(scale, nsrc - j0, nxt, tile_byte, tile_bytes, lane_byte, acc);
   } else {
-    fold_rest<T, F, U, CH, MODE, true>(a, nsrc, cur, tile_byte, tile_bytes, lane_byte, acc);
+    fold_rest<T, F, U, CH, MODE, true>(scale, nsrc, cur, tile_byte, tile_bytes, lane_byte, acc);
   }
   const __amdgpu_buffer_rsrc_t rd = tile_rsrc((const char*)a.dst + tile_byte, tile_bytes);
   u32x4 out[U];
   // AVG's extra multiply is decided once per tile (wave-uniform), not per element
-  const int mode = MODE == kPremul ? (int)kPremul : a.mode;
+  const int mode = MODE == kPremul ? (int)kPremul : mode_arg;
   if (mode == kAvg) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       elem_t e[N];
 #pragma unroll
       for (int i = 0; i < N; ++i) {
-        e[i] = Tr::template finish<F>(acc[u][i], kAvg, a.scale);
+        e[i] = Tr::template finish<F>(acc[u][i], kAvg, scale);
       }
       __builtin_memcpy(&out[u], e, 16);
     }
@@ -332,7 +352,7 @@ __device__ __forceinline__ void reduce_tile(const ReduceArgs& a, int nsrc, uint6
       elem_t e[N];
 #pragma unroll
       for (int i = 0; i < N; ++i) {
-        e[i] = Tr::template finish<F>(acc[u][i], kPlain, a.scale);
+        e[i] = Tr::template finish<F>(acc[u][i], kPlain, scale);
       }
       __builtin_memcpy(&out[u], e, 16);
     }
@@ -352,10 +372,21 @@ __device__ __forceinline__ void reduce_tile(const ReduceArgs& a, int nsrc, uint6
 // than 64 bytes) and past the last whole vector (fewer than 16 bytes) are folded by workgroup 0,
 // which has no tiles.
 template<typename T, int F, int U, int CH, bool PREMUL>
-__global__ __launch_bounds__(kWave) void reduce_vec_kernel(ReduceArgs a) {
-  const int nsrc = a.nsrc;
+__global__ __launch_bounds__(kWave) void reduce_vec_kernel(uint64_t nvec, uint32_t tile_waves, uint32_t nsrc_and_mode,
+    float scale, const char* s0, const char* s1, const char* s2, const char* s3, ReduceArgs a) {
+  // The leading arguments repeat what a tile workgroup needs before its first vector load and
+  // to find its next tile -- vector count, number of tile workgroups, source count (low byte)
+  // and mode, the scale, the first four source pointers: compiled with
+  // -amdgpu-kernarg-preload-count they arrive in registers with the wave (fourteen dwords, all
+  // that the hardware preloads), where a read from the argument segment is a scalar round trip
+  // to memory the host has just written: 0.3-0.5 us of a launch that lasts 3-9 us.  (The scale
+  // is not needed early, but a scalar load of it, once the compiler chose to copy its result
+  // before the loop over the tiles, made the wave wait there for every load issued so far.)
+  const char* const early[kEarlySources] = {s0, s1, s2, s3};
+  const int nsrc = (int)(nsrc_and_mode & 0xff);
+  const int mode = (int)(nsrc_and_mode >> 8);
   constexpr uint64_t tile_bytes = (uint64_t)kWave * U * 16;
-  const uint64_t body_bytes = a.nvec * 16;
+  const uint64_t body_bytes = nvec * 16;
   const uint64_t ntiles = (body_bytes + tile_bytes - 1) / tile_bytes;
   // The head and tail elements have a workgroup of their own, workgroup 0 of every launch
   // (which finds nothing to do when there are none): folded by a workgroup that also has
@@ -364,17 +395,17 @@ __global__ __launch_bounds__(kWave) void reduce_vec_kernel(ReduceArgs a) {
   // workgroups know what they are from blockIdx alone: a test that needed a kernel argument
   // held their first loads up behind one more scalar round trip (0.4 us of 23).
   if (blockIdx.x == 0) {
-    // ReduceArgs is the kernel's only argument, so it sits at the start of the argument segment:
-    // the function reads it from there.  (The address of the kernel's own parameter would make
+    // ReduceArgs follows the leading arguments (kArgsOffset bytes) in the argument segment: the
+    // function reads it from there.  (The address of the kernel's own parameter would make
     // every wave of the launch copy the struct to its stack first; and the segment's address has
     // to be taken here, in the kernel -- inside a called function the builtin yields null.)
-    reduce_head_and_tail<T, F>((const ReduceArgs*)__builtin_amdgcn_kernarg_segment_ptr(), threadIdx.x);
+    const char* segment = (const char*)__builtin_amdgcn_kernarg_segment_ptr();
+    reduce_head_and_tail<T, F>((const ReduceArgs*)(segment + kArgsOffset), threadIdx.x);
     return;
   }
   // The tile workgroups never outnumber the tiles (a launch with no whole vector has one, whose
   // descriptors are then empty), so the first tile needs no test and the scalar loads of the
   // arguments are not held up behind a load-and-branch.
-  const uint32_t tile_waves = gridDim.x - 1;
   uint64_t tile = blockIdx.x - 1;
   do {
     const uint64_t tile_byte = tile * tile_bytes;
@@ -384,7 +415,7 @@ __global__ __launch_bounds__(kWave) void reduce_vec_kernel(ReduceArgs a) {
     // for 16-bit types, the rounding of every source element to the element type after it.  AVG
     // is the plain fold with one more multiply when the result is written (a wave-uniform test
     // there).
-    reduce_tile<T, F, U, CH, PREMUL ? kPremul : kPlain>(a, nsrc, tile_byte, n);
+    reduce_tile<T, F, U, CH, PREMUL ? kPremul : kPlain>(a, early, nsrc, mode, scale, tile_byte, n);
     tile += tile_waves;
   } while (tile < ntiles);
 }
@@ -518,9 +549,15 @@ int launch_one(const ReduceArgs& a0, hipStream_t stream) {
   // reduce_wg_per_cu (measurement only): an unused LDS allocation caps the waves resident on a CU
   const int cap = t.reduce_wg_per_cu >= 2 && t.reduce_wg_per_cu <= 8 ? t.reduce_wg_per_cu : 0;
   const size_t lds = kLdsForCap[cap];
+  const uint32_t lead = (uint32_t)a.nsrc | (uint32_t)a.mode << 8;
+  const char* e[kEarlySources];
+  for (int j = 0; j < kEarlySources; ++j) {
+    e[j] = (const char*)a.src[j]; // slots past the last source hold null and are never read
+  }
 #define MDH_LAUNCH_REDUCE(UU, CC)                                                  \
   if (shape.unroll == UU && shape.chunk == CC) {                                   \
-    hipLaunchKernelGGL((reduce_vec_kernel<T, F, UU, CC, PREMUL>), g, b, lds, stream, a); \
+    hipLaunchKernelGGL((reduce_vec_kernel<T, F, UU, CC, PREMUL>), g, b, lds, stream, a.nvec, (uint32_t)shape.waves, lead, a.scale, \
+        e[0], e[1], e[2], e[3], a);                                                \
     return check_launch("reduce_vec_kernel");                                      \
   }
   MDH_LAUNCH_REDUCE(16, 1)
