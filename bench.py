@@ -28,16 +28,29 @@ TIMED_WINDOWS = 11     # windows of `steps` launches; the median window is repor
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch), each
 # scaled by what the same counter reads for the flat copy of exactly 256 MiB (FETCH_SIZE x 1.99991,
 # WRITE_SIZE x 1.00000): profiles/hbm_traffic_pmc_reduce_and_copy_kernels.md.  E.g. the headline:
-# 65,560.67 x 1.99991 + 16,384.00 KiB = 147,499.3 KiB.  Workloads without an entry were not measured.
+# 65,552.31 x 1.99991 + 16,384.00 KiB = 147,482.6 KiB.  Workloads without an entry were not measured.
 MEASURED_TRAFFIC_BYTES = {
-    "reduce_fp32_p8": 151039298,
-    "reduce_bf16_p16": 1140903999,
-    "reduce_fp32_p64_sum": 272678699,
+    "reduce_fp32_p8": 151022184,
+    "reduce_bf16_p16": 1140903271,
+    "reduce_fp32_p64_sum": 272676106,
     "allgather_bf16_p8": 536870912,
-    "allgather_bf16_p8_strided": 536907804,
-    "redistribute_fp32_8192": 67156846,
-    "redistribute_bf16_3d": 16825561,
+    "allgather_bf16_p8_strided": 536907866,
+    "redistribute_fp32_8192": 67156871,
+    "redistribute_bf16_3d": 16825557,
 }
+
+def box_kernel(abi):
+    """The strided-box kernel the benchmark's shapes run: equal boxes of full tiles are started from
+    preloaded arguments (copy_rows16_kernel) unless the knob box_preload=1 asks for the table form."""
+    return "copy_boxes16_kernel" if abi.get_tuning("box_preload") == 1 else "copy_rows16_kernel"
+
+
+def flat_kernel(abi, sources, shard_bytes):
+    """The dense-gather kernel: up to eight equal shards on the 64-byte grid start from preloaded
+    arguments (copy_flat8_kernel), anything else from the segment table."""
+    early = 1 < sources <= 8 and shard_bytes % 64 == 0 and abi.get_tuning("box_preload") != 1
+    return "copy_flat8_kernel" if early else "copy_flat_kernel"
+
 
 def build_workload(name, torch, abi, dev, rotation_bytes):
     """Returns (describe, algorithmic_bytes, launch(i), check(), kernel name) for a named workload.
@@ -143,7 +156,7 @@ def build_workload(name, torch, abi, dev, rotation_bytes):
 
         desc = {"workload": name, "op": "all_gather_into_tensor chunk assembly", "sources": P, "shard_bytes": shard,
                 "dtype": "uint8", "buffer_sets": nsets}
-        return desc, set_bytes, launch, check, "copy_flat_kernel"
+        return desc, set_bytes, launch, check, flat_kernel(abi, P, shard)
 
     if name == "allgather_bf16_p8" or name == "allgather_bf16_p8_strided":
         P, n = 8, 16777216
@@ -177,7 +190,7 @@ def build_workload(name, torch, abi, dev, rotation_bytes):
 
         desc = {"workload": name, "op": "all_gather_into_tensor chunk assembly", "sources": P, "numel": n,
                 "dtype": "bfloat16", "buffer_sets": nsets}
-        return desc, set_bytes, launch, check, "copy_boxes16_kernel" if pad else "copy_flat_kernel"
+        return desc, set_bytes, launch, check, box_kernel(abi) if pad else flat_kernel(abi, P, n * 2)
 
     if name.startswith("redistribute"):
         # redistribute_fp32_8192, redistribute_bf16_8192, redistribute_bf16_3d
@@ -229,7 +242,7 @@ def build_workload(name, torch, abi, dev, rotation_bytes):
                 # these kernels are shorter than the host's launch call: the timed launches are
                 # enqueued behind a long blocker kernel so that the GPU runs them back to back
                 "queue_prefilled": True}
-        return desc, set_bytes, launch, check, "copy_boxes16_kernel"
+        return desc, set_bytes, launch, check, box_kernel(abi)
 
     raise SystemExit("bench: unknown workload %r" % name)
 

@@ -183,12 +183,15 @@ int mdh_copy_plan_verify(const mdh_copy_plan* plan, const uint64_t* base_bytes, 
 /*
  * Introspection, no reference counterpart: the kernel-argument block and the launch shape
  * that launch number `step` (0 .. mdh_copy_plan_launches-1) passes for these 16-byte aligned
- * bases.  `*size` receives the block's size; `out` may be NULL to ask for the size only.
- * Enqueues nothing.  For checks of what a stream capture recorded against what an eager
+ * bases.  `*size` receives the block's size; `out` may be NULL to ask for the size only.  The
+ * block begins with `*leading_scalars` 4-byte scalars, each a kernel parameter of its own
+ * (0 for most launches, 14 for one started from preloaded arguments); the rest is one struct
+ * parameter.  Enqueues nothing.  For checks of what a stream capture recorded against what an eager
  * launch passes.
  */
 int mdh_copy_plan_step_arguments(const mdh_copy_plan* plan, const void* const* bases, int nbases, int step, void* out,
-    size_t capacity, size_t* size, uint32_t* grid_x, uint32_t* grid_y, uint32_t* block, uint32_t* lds);
+    size_t capacity, size_t* size, uint32_t* leading_scalars, uint32_t* grid_x, uint32_t* grid_y, uint32_t* block,
+    uint32_t* lds);
 void mdh_copy_plan_destroy(mdh_copy_plan* plan);
 
 /*
@@ -215,7 +218,8 @@ int mdh_static_workspace(void** address, size_t* bytes);
  * 4, 8; contiguous segments), "box_unroll" (1, 2, 4, 8; strided boxes),
  * "copy_max_blocks", "copy_wg_per_cu" (2..8, 9 = never cap), "box_policy" (loads of the
  * strided-box kernel: 1 = plain, which pays when the sources are still in the Infinity Cache;
- * 0 or 2 = nt, the default).  Returns MDH_EINVAL for an unknown name or value.
+ * 0 or 2 = nt, the default), "box_preload" (1 = never start equal boxes of full tiles from
+ * preloaded kernel arguments).  Returns MDH_EINVAL for an unknown name or value.
  * No counterpart in the reference, whose grid is fixed at 4/16/64 blocks
  * (core/kernels.cc:547-556).
  */

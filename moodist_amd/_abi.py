@@ -77,6 +77,10 @@ def lib():
     L.mdh_copy_plan_verify.restype = ctypes.c_int
     L.mdh_copy_plan_destroy.argtypes = [ctypes.c_void_p]
     L.mdh_copy_plan_destroy.restype = None
+    u32p = ctypes.POINTER(ctypes.c_uint32)
+    L.mdh_copy_plan_step_arguments.argtypes = [ctypes.c_void_p, vpp, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                               ctypes.c_size_t, ctypes.POINTER(ctypes.c_size_t), u32p, u32p, u32p, u32p, u32p]
+    L.mdh_copy_plan_step_arguments.restype = ctypes.c_int
     L.mdh_set_tuning.argtypes = [ctypes.c_char_p, ctypes.c_int]
     L.mdh_set_tuning.restype = ctypes.c_int
     L.mdh_get_tuning.argtypes = [ctypes.c_char_p, ctypes.POINTER(ctypes.c_int)]
@@ -147,6 +151,17 @@ class CopyPlan:
     @property
     def launches(self):
         return lib().mdh_copy_plan_launches(self._plan)
+
+    def step_arguments(self, bases, step):
+        """What launch number `step` passes for these bases, without enqueuing anything: (argument
+        bytes, leading 4-byte scalar parameters among them, grid x, grid y, block, LDS bytes)."""
+        buf = ctypes.create_string_buffer(4096)
+        size = ctypes.c_size_t()
+        lead, gx, gy, block, lds = (ctypes.c_uint32() for _ in range(5))
+        check(lib().mdh_copy_plan_step_arguments(self._plan, ptr_table(bases), len(bases), step, buf, len(buf),
+                                                 ctypes.byref(size), ctypes.byref(lead), ctypes.byref(gx),
+                                                 ctypes.byref(gy), ctypes.byref(block), ctypes.byref(lds)))
+        return buf.raw[:size.value], lead.value, gx.value, gy.value, block.value, lds.value
 
     def __del__(self):
         if getattr(self, "_plan", None):

@@ -92,6 +92,9 @@ int* knob(const char* name) {
   if (!std::strcmp(name, "box_policy")) {
     return &t.box_policy;
   }
+  if (!std::strcmp(name, "box_preload")) {
+    return &t.box_preload;
+  }
   if (!std::strcmp(name, "copy_max_blocks")) {
     return &t.copy_max_blocks;
   }
@@ -112,7 +115,8 @@ extern "C" int mdh_set_tuning(const char* name, int value) {
       mdh::set_error("mdh_set_tuning: %s does not take %d", name, value);
       return MDH_EINVAL;
     }
-  } else if (value < 0 || (std::strstr(name, "wg_per_cu") && value > 9) || (!std::strcmp(name, "box_policy") && value > 2)) {
+  } else if (value < 0 || (std::strstr(name, "wg_per_cu") && value > 9) || (!std::strcmp(name, "box_policy") && value > 2) ||
+             (!std::strcmp(name, "box_preload") && value > 1)) {
     mdh::set_error("mdh_set_tuning: %s does not take %d", name, value);
     return MDH_EINVAL;
   }

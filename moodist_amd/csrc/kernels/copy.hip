@@ -252,6 +252,101 @@ __global__ __launch_bounds__(kBlock) void copy_boxes16_kernel(CopyArgs a) {
   } while (tile < a.total_tiles);
 }
 
+// ---- the same copy for equal boxes of full tiles, started from preloaded arguments ----
+//
+// In the form above a wave's first vector load waits for a scalar round trip to the argument
+// table, which the host has just written (0.3-0.5 us of launches that last 4-13 us).  When the
+// boxes of a launch are at most eight, have the same two-dimensional shape on the source side
+// and consist of full tiles only -- the shards of a redistribution or of a padded gather --
+// everything the loads need fits the fourteen dwords that the hardware hands a wave in registers
+// when it starts (kernels compiled with -amdgpu-kernarg-preload-count): the source row pitch,
+// the tile shape, and the eight source addresses as 48 bits each.  The destination side still
+// comes from the table, read while the vector loads are in flight.
+constexpr int kEarlyBoxes = 8;
+
+struct PackedSources {
+  uint32_t lo[kEarlyBoxes];     // source addresses, low halves
+  uint32_t hi[kEarlyBoxes / 2]; // bits 32..47 of two addresses each: box 2k low, box 2k+1 high
+};
+
+struct RowsLead {
+  uint32_t src_stride; // bytes between rows of the source
+  uint32_t shape;      // log2tc | column tiles per row << 5
+  PackedSources from;
+};
+static_assert(sizeof(RowsLead) == 14 * 4, "fourteen dwords are preloaded");
+
+// The same for copy_flat_kernel's equal segments (below).
+struct FlatLead {
+  uint32_t bytes; // of every segment
+  uint32_t reserved;
+  PackedSources from;
+};
+static_assert(sizeof(FlatLead) == 14 * 4, "fourteen dwords are preloaded");
+
+MDH_HD uint32_t pick8(uint32_t i, uint32_t a0, uint32_t a1, uint32_t a2, uint32_t a3, uint32_t a4, uint32_t a5, uint32_t a6,
+    uint32_t a7) {
+  uint32_t r = a0;
+  r = i == 1 ? a1 : r;
+  r = i == 2 ? a2 : r;
+  r = i == 3 ? a3 : r;
+  r = i == 4 ? a4 : r;
+  r = i == 5 ? a5 : r;
+  r = i == 6 ? a6 : r;
+  r = i == 7 ? a7 : r;
+  return r;
+}
+
+// Source address of box y out of the packed halves (selects of scalars: y is wave-uniform).
+MDH_HD uint64_t packed_source_address(uint32_t y, uint32_t l0, uint32_t l1, uint32_t l2, uint32_t l3, uint32_t l4, uint32_t l5,
+    uint32_t l6, uint32_t l7, uint32_t h0, uint32_t h1, uint32_t h2, uint32_t h3) {
+  const uint32_t lo = pick8(y, l0, l1, l2, l3, l4, l5, l6, l7);
+  const uint32_t pair = pick8(y >> 1, h0, h1, h2, h3, 0, 0, 0, 0);
+  const uint32_t hi = (y & 1u) ? pair >> 16 : pair & 0xffffu;
+  return (uint64_t)hi << 32 | lo;
+}
+
+// Offset of a slot of a full tile on one side of the box: what slot_offsets computes for a box
+// of one strided extent whose rows are a whole number of vectors.
+MDH_HD uint32_t rows_offset(uint32_t stride, uint32_t log2tc, uint32_t log2slots, uint32_t rt, uint32_t ct, uint32_t slot) {
+  const uint32_t col = (ct << log2tc) + (slot & ((1u << log2tc) - 1u));
+  const uint32_t row = (rt << (log2slots - log2tc)) + (slot >> log2tc);
+  return row * stride + col * 16u;
+}
+
+template<int U, bool PLAIN>
+__global__ __launch_bounds__(kBlock) void copy_rows16_kernel(uint32_t src_stride, uint32_t shape, uint32_t l0, uint32_t l1,
+    uint32_t l2, uint32_t l3, uint32_t l4, uint32_t l5, uint32_t l6, uint32_t l7, uint32_t h0, uint32_t h1, uint32_t h2,
+    uint32_t h3, CopyArgs a) {
+  constexpr int kLoad = PLAIN ? 0 : 2;
+  constexpr int kStore = 18;
+  constexpr uint32_t log2slots = ilog2(kBlock * U);
+  const uint32_t y = blockIdx.y;
+  const uint32_t log2tc = shape & 31u, nct = shape >> 5;
+  const uint32_t rt = blockIdx.x / nct;
+  const TileLoc t{y, rt, blockIdx.x - rt * nct};
+  // every slot of every tile lies inside the box (the host launches this form for nothing
+  // else), so the descriptor needs no end
+  const char* src = (const char*)(uintptr_t)packed_source_address(y, l0, l1, l2, l3, l4, l5, l6, l7, h0, h1, h2, h3);
+  const __amdgpu_buffer_rsrc_t rs = tile_rsrc(src, 0xffffffffu);
+  u32x4 v[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    v[u] = tile_load<kLoad>(rs, rows_offset(src_stride, log2tc, log2slots, t.rt, t.ct, (uint32_t)u * kBlock + threadIdx.x));
+  }
+  // The loads are out before anything of the table is waited for.  (The destination side is
+  // straight-line code on purpose: with branches between the loads and the stores the compiler
+  // sinks the loads below them, behind the wait for the table.)
+  __builtin_amdgcn_sched_barrier(0);
+  const BoxDesc& B = a.box[y];
+  const __amdgpu_buffer_rsrc_t rd = tile_rsrc(B.dst, B.dst_span);
+  const uint32_t dst_stride = (uint32_t)B.dst_stride[0];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    tile_store<kStore>(rd, rows_offset(dst_stride, log2tc, log2slots, t.rt, t.ct, (uint32_t)u * kBlock + threadIdx.x), v[u]);
+  }
+}
+
 // Contiguous segments (the shards of a dense all-gather, or any box that
 // collapses to one run): no per-lane index arithmetic at all.  A tile is
 // kBlock*U consecutive 16-byte vectors of one segment, addressed through a
@@ -377,6 +472,35 @@ __global__ __launch_bounds__(kBlock) void copy_flat_kernel(FlatArgs a) {
   } while (tile < a.total_tiles);
 }
 
+// Equal segments again -- at most eight, all of one length (the dense all-gather of up to eight
+// shards) -- started from preloaded arguments like copy_rows16_kernel: the segments' length and
+// their source addresses arrive in registers, the destination's address is read from the table
+// while the vector loads are in flight.
+template<int U>
+__global__ __launch_bounds__(kBlock) void copy_flat8_kernel(uint32_t bytes, uint32_t, uint32_t l0, uint32_t l1, uint32_t l2,
+    uint32_t l3, uint32_t l4, uint32_t l5, uint32_t l6, uint32_t l7, uint32_t h0, uint32_t h1, uint32_t h2, uint32_t h3,
+    FlatArgs a) {
+  constexpr uint32_t tile_bytes = kBlock * U * 16;
+  const uint32_t lane_byte = threadIdx.x * 16;
+  const uint32_t seg = blockIdx.y;
+  const uint32_t off = blockIdx.x * tile_bytes; // below the segment's length, which fits 32 bits
+  const uint32_t left = bytes - off;
+  const uint32_t n = left < tile_bytes ? left : tile_bytes;
+  const char* src = (const char*)(uintptr_t)packed_source_address(seg, l0, l1, l2, l3, l4, l5, l6, l7, h0, h1, h2, h3);
+  const __amdgpu_buffer_rsrc_t rs = tile_rsrc(src + off, n);
+  u32x4 v[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    v[u] = tile_load(rs, lane_byte + (uint32_t)u * (kBlock * 16));
+  }
+  __builtin_amdgcn_sched_barrier(0); // the loads are out before the table is waited for
+  const __amdgpu_buffer_rsrc_t rd = tile_rsrc(a.dst[seg] + off, n);
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    tile_store(rd, lane_byte + (uint32_t)u * (kBlock * 16), v[u]);
+  }
+}
+
 // ---- host side: reduce a box to the kernel's form ----
 
 struct HostBox {
@@ -406,12 +530,110 @@ struct Step {
   uint32_t grid;
   uint32_t grid_y; // > 0: the two-dimensional form for equal boxes / segments (grid x grid_y workgroups)
   bool plain_loads; // kBoxes16: plain instead of nt loads (tuning knob)
+  bool preloaded = false; // equal boxes of full tiles / equal segments of one length: started from preloaded arguments
   size_t lds;
   FlatArgs flat;   // kFlat
   CopyArgs boxes;  // kBoxes16, kBoxes
 };
 
 int launch_step(const Step& st, const FlatArgs* flat, const CopyArgs* boxes, hipStream_t stream);
+
+// Whether a launch of equal boxes qualifies for copy_rows16_kernel: at most eight boxes, one
+// strided extent, the same shape on the source side, rows a whole number of vectors, and no
+// tile with a slot outside its box.
+inline bool uniform_full_rows(const CopyArgs& a, int unroll) {
+  if (a.nboxes == 0 || a.nboxes > (uint32_t)kEarlyBoxes || a.tiles_per_box == 0) {
+    return false;
+  }
+  const BoxDesc& f = a.box[0];
+  const uint32_t slots = (uint32_t)kBlock * (uint32_t)unroll;
+  if (f.nouter > 1 || (slots >> f.log2tc) == 0 || f.cols == 0 || f.rows == 0) {
+    return false;
+  }
+  const uint32_t tr = slots >> f.log2tc;
+  if ((uint64_t)f.nct << f.log2tc != f.cols || f.rows % tr != 0 || f.nct >= (1u << 27) ||
+      (uint64_t)f.last_off != ((uint64_t)f.cols - 1) * 16) {
+    return false;
+  }
+  if (f.src_stride[0] < 0 || f.src_stride[0] > 0xffffffffll) {
+    return false;
+  }
+  // the end of the last vector of the last row: the largest offset the kernel forms, plus 16
+  const uint64_t reach = (uint64_t)(f.rows - 1) * (uint64_t)f.src_stride[0] + (uint64_t)f.cols * 16;
+  if (f.src_span == 0 || reach > f.src_span) {
+    return false;
+  }
+  for (uint32_t k = 0; k < a.nboxes; ++k) {
+    // the destination side may differ from box to box, but is addressed the same way
+    const BoxDesc& b = a.box[k];
+    if (b.dst_stride[0] < 0 || b.dst_stride[0] > 0xffffffffll || b.dst_span == 0 ||
+        (uint64_t)(f.rows - 1) * (uint64_t)b.dst_stride[0] + (uint64_t)f.cols * 16 > b.dst_span) {
+      return false;
+    }
+  }
+  for (uint32_t k = 1; k < a.nboxes; ++k) {
+    const BoxDesc& b = a.box[k];
+    if (b.nouter > 1 || b.rows != f.rows || b.cols != f.cols || b.nct != f.nct || b.log2tc != f.log2tc ||
+        b.last_off != f.last_off || b.src_stride[0] != f.src_stride[0] || b.src_span != f.src_span) {
+      return false;
+    }
+  }
+  return true;
+}
+
+// Packs up to eight source addresses as 48 bits each; false when one does not fit, and the
+// launch then takes the table form.
+inline bool pack_sources(const char* const* src, uint32_t n, PackedSources* out) {
+  PackedSources P{};
+  for (uint32_t k = 0; k < n; ++k) {
+    const uint64_t addr = (uint64_t)(uintptr_t)src[k];
+    if (addr >> 48) {
+      return false;
+    }
+    P.lo[k] = (uint32_t)addr;
+    P.hi[k / 2] |= (uint32_t)(addr >> 32) << (16 * (k & 1));
+  }
+  for (uint32_t k = 0; k < n; ++k) {
+    // through the function the kernels unpack them with
+    if (packed_source_address(k, P.lo[0], P.lo[1], P.lo[2], P.lo[3], P.lo[4], P.lo[5], P.lo[6], P.lo[7], P.hi[0], P.hi[1],
+            P.hi[2], P.hi[3]) != (uint64_t)(uintptr_t)src[k]) {
+      return false;
+    }
+  }
+  *out = P;
+  return true;
+}
+
+// The leading arguments of copy_rows16_kernel for these (patched) boxes.
+inline bool make_rows_lead(const CopyArgs& a, RowsLead* lead) {
+  const char* src[kEarlyBoxes];
+  for (uint32_t k = 0; k < a.nboxes; ++k) {
+    src[k] = a.box[k].src;
+  }
+  lead->src_stride = (uint32_t)a.box[0].src_stride[0];
+  lead->shape = a.box[0].log2tc | a.box[0].nct << 5;
+  return pack_sources(src, a.nboxes, &lead->from);
+}
+
+// Whether a two-dimensional launch of flat segments qualifies for copy_flat8_kernel: at most
+// eight segments, all of the same length.
+inline bool uniform_segments(const FlatArgs& a) {
+  if (a.nsegs == 0 || a.nsegs > (uint32_t)kEarlyBoxes || a.tiles_per_seg == 0 || a.edge_wgs != 0) {
+    return false;
+  }
+  for (uint32_t k = 0; k < a.nsegs; ++k) {
+    if (a.bytes[k] != a.bytes[0] || a.bytes[k] > 0xffffffffull) {
+      return false;
+    }
+  }
+  return true;
+}
+
+inline bool make_flat_lead(const FlatArgs& a, FlatLead* lead) {
+  lead->bytes = (uint32_t)a.bytes[0];
+  lead->reserved = 0;
+  return pack_sources(a.src, a.nsegs, &lead->from);
+}
 
 // The grid a step is launched with: st.grid (x st.grid_y) tile workgroups, and in the
 // one-dimensional form of a flat step the edge workgroups in front of them.
@@ -514,6 +736,7 @@ struct Launcher {
       st.plain_loads = false;
       if (a.tiles_per_seg && grid == a.total_tiles && a.nsegs > 1 && !edges) {
         st.grid = a.tiles_per_seg, st.grid_y = a.nsegs;
+        st.preloaded = t.box_preload != 1 && uniform_segments(a);
       }
       submit(st, &a, nullptr);
     }
@@ -552,6 +775,7 @@ struct Launcher {
     st.plain_loads = plain_loads;
     if (buffer16 && a.tiles_per_box && grid == a.total_tiles) {
       st.grid = a.tiles_per_box, st.grid_y = a.nboxes;
+      st.preloaded = t.box_preload != 1 && uniform_full_rows(a, unroll);
     }
     submit(st, nullptr, &a);
   }
@@ -846,6 +1070,8 @@ int launch_step(const Step& st, const FlatArgs* flat, const CopyArgs* boxes, hip
   launch_dims(st, &gx, &gy);
   dim3 g(gx, gy), b(kBlock);
 #define MDH_COMMA ,
+#define MDH_PACKED(P) \
+  P.lo[0], P.lo[1], P.lo[2], P.lo[3], P.lo[4], P.lo[5], P.lo[6], P.lo[7], P.hi[0], P.hi[1], P.hi[2], P.hi[3]
 #define MDH_LAUNCH_COPY(kernel, more, args)                                                  \
   switch (st.unroll) {                                                                 \
   case 1:                                                                              \
@@ -878,17 +1104,75 @@ int launch_step(const Step& st, const FlatArgs* flat, const CopyArgs* boxes, hip
     break;                                                                             \
   }
   switch (st.kind) {
-  case Step::kFlat:
+  case Step::kFlat: {
+    FlatLead L;
+    if (st.preloaded && make_flat_lead(*flat, &L)) {
+      switch (st.unroll) {
+      case 1:
+        hipLaunchKernelGGL((copy_flat8_kernel<1>), g, b, st.lds, stream, L.bytes, L.reserved, MDH_PACKED(L.from), *flat);
+        break;
+      case 2:
+        hipLaunchKernelGGL((copy_flat8_kernel<2>), g, b, st.lds, stream, L.bytes, L.reserved, MDH_PACKED(L.from), *flat);
+        break;
+      case 4:
+        hipLaunchKernelGGL((copy_flat8_kernel<4>), g, b, st.lds, stream, L.bytes, L.reserved, MDH_PACKED(L.from), *flat);
+        break;
+      default:
+        hipLaunchKernelGGL((copy_flat8_kernel<8>), g, b, st.lds, stream, L.bytes, L.reserved, MDH_PACKED(L.from), *flat);
+        break;
+      }
+      return check_launch("copy_flat8_kernel");
+    }
     MDH_LAUNCH_COPY(copy_flat_kernel, , *flat)
     return check_launch("copy_flat_kernel");
-  case Step::kBoxes16:
+  }
+  case Step::kBoxes16: {
+    RowsLead L;
+    if (st.preloaded && make_rows_lead(*boxes, &L)) {
+#define MDH_LAUNCH_ROWS(UU, PP)                                                                                  \
+  hipLaunchKernelGGL((copy_rows16_kernel<UU, PP>), g, b, st.lds, stream, L.src_stride, L.shape, MDH_PACKED(L.from), *boxes)
+      switch (st.unroll) {
+      case 1:
+        if (st.plain_loads) {
+          MDH_LAUNCH_ROWS(1, true);
+        } else {
+          MDH_LAUNCH_ROWS(1, false);
+        }
+        break;
+      case 2:
+        if (st.plain_loads) {
+          MDH_LAUNCH_ROWS(2, true);
+        } else {
+          MDH_LAUNCH_ROWS(2, false);
+        }
+        break;
+      case 4:
+        if (st.plain_loads) {
+          MDH_LAUNCH_ROWS(4, true);
+        } else {
+          MDH_LAUNCH_ROWS(4, false);
+        }
+        break;
+      default:
+        if (st.plain_loads) {
+          MDH_LAUNCH_ROWS(8, true);
+        } else {
+          MDH_LAUNCH_ROWS(8, false);
+        }
+        break;
+      }
+#undef MDH_LAUNCH_ROWS
+      return check_launch("copy_rows16_kernel");
+    }
     if (st.plain_loads) {
       MDH_LAUNCH_COPY(copy_boxes16_kernel, MDH_COMMA true, *boxes)
     } else {
       MDH_LAUNCH_COPY(copy_boxes16_kernel, MDH_COMMA false, *boxes)
     }
     return check_launch("copy_boxes16_kernel");
+  }
 #undef MDH_LAUNCH_COPY
+#undef MDH_PACKED
 #undef MDH_COMMA
   default:
     switch (st.vec) {
@@ -1206,6 +1490,11 @@ extern "C" int mdh_copy_plan_verify(const mdh_copy_plan* plan, const uint64_t* b
         set_error("mdh_copy_plan_verify: step %zu: the two-dimensional form has no edge workgroups", s);
         return MDH_EINVAL;
       }
+      // copy_flat8_kernel takes every segment's length from one leading argument
+      if (st.preloaded && (!st.grid_y || !uniform_segments(a))) {
+        set_error("mdh_copy_plan_verify: step %zu: the preloaded form does not fit this launch", s);
+        return MDH_EINVAL;
+      }
       // the edge workgroups: every slot of every segment, through the kernel's own mapping
       if ((a.edge_wgs != 0) != [&] {
             for (uint32_t seg = 0; seg < a.nsegs; ++seg) {
@@ -1261,7 +1550,19 @@ extern "C" int mdh_copy_plan_verify(const mdh_copy_plan* plan, const uint64_t* b
         uint64_t so, dof;
         if (buffer16) {
           uint32_t so32, dof32;
-          if (!slot_offsets<uint32_t>(B, t, slot, log2slots, 16u, &so32, &dof32)) {
+          const bool inside = slot_offsets<uint32_t>(B, t, slot, log2slots, 16u, &so32, &dof32);
+          if (st.preloaded) {
+            // copy_rows16_kernel: no slot may lie outside the box, and its own arithmetic --
+            // from the leading arguments alone -- must name the same source vector
+            const BoxDesc& f = a.box[0];
+            const uint32_t early = rows_offset((uint32_t)f.src_stride[0], f.log2tc, log2slots, t.rt, t.ct, slot);
+            const uint32_t early_dst = rows_offset((uint32_t)B.dst_stride[0], f.log2tc, log2slots, t.rt, t.ct, slot);
+            if (!inside || early != so32 || early_dst != dof32 || !uniform_full_rows(a, st.unroll)) {
+              set_error("mdh_copy_plan_verify: step %zu box %u: the preloaded form does not fit this launch", s, t.box);
+              return MDH_EINVAL;
+            }
+          }
+          if (!inside) {
             continue; // the kernel gives this slot the offset just past the descriptor
           }
           // an access the descriptor would clip is an access the kernel silently loses
@@ -1375,7 +1676,8 @@ extern "C" int mdh_copy_plan_launch(const mdh_copy_plan* plan, const void* const
 }
 
 extern "C" int mdh_copy_plan_step_arguments(const mdh_copy_plan* plan, const void* const* bases, int nbases, int step,
-    void* out, size_t capacity, size_t* size, uint32_t* grid_x, uint32_t* grid_y, uint32_t* block, uint32_t* lds) {
+    void* out, size_t capacity, size_t* size, uint32_t* leading_scalars, uint32_t* grid_x, uint32_t* grid_y,
+    uint32_t* block, uint32_t* lds) {
   using namespace mdh;
   if (!plan || nbases != plan->nbases || (nbases > 0 && !bases) || step < 0 || (size_t)step >= plan->steps.size() ||
       !size) {
@@ -1396,17 +1698,34 @@ extern "C" int mdh_copy_plan_step_arguments(const mdh_copy_plan* plan, const voi
   }
   FlatArgs flat;
   CopyArgs boxes;
+  union {
+    RowsLead rows;
+    FlatLead flat;
+  } lead;
+  static_assert(sizeof(RowsLead) == sizeof(FlatLead), "one size of leading arguments");
+  size_t lead_bytes = 0;
   const void* from;
   if (st.kind == Step::kFlat) {
     flat = st.flat;
     patch_step(*plan, (size_t)step, at, bases, &flat, nullptr);
     from = &flat;
     *size = sizeof(FlatArgs);
+    if (st.preloaded && make_flat_lead(flat, &lead.flat)) {
+      lead_bytes = sizeof(FlatLead);
+      *size += lead_bytes;
+    }
   } else {
     boxes = st.boxes;
     patch_step(*plan, (size_t)step, at, bases, nullptr, &boxes);
     from = &boxes;
     *size = sizeof(CopyArgs);
+    if (st.kind == Step::kBoxes16 && st.preloaded && make_rows_lead(boxes, &lead.rows)) {
+      lead_bytes = sizeof(RowsLead);
+      *size += lead_bytes;
+    }
+  }
+  if (leading_scalars) {
+    *leading_scalars = (uint32_t)(lead_bytes / 4);
   }
   uint32_t gx, gy;
   launch_dims(st, &gx, &gy);
@@ -1419,7 +1738,8 @@ extern "C" int mdh_copy_plan_step_arguments(const mdh_copy_plan* plan, const voi
       set_error("mdh_copy_plan_step_arguments: the block is %zu bytes", *size);
       return MDH_EINVAL;
     }
-    std::memcpy(out, from, *size);
+    std::memcpy(out, &lead, lead_bytes);
+    std::memcpy((char*)out + lead_bytes, from, *size - lead_bytes);
   }
   return MDH_OK;
 }

@@ -92,6 +92,7 @@ struct Tuning {
   int copy_max_blocks = 0;
   int copy_wg_per_cu = 0; // as reduce_wg_per_cu, for the copy kernels
   int box_policy = 0;     // loads of the strided-box kernel: 1 plain, 0 or 2 nt
+  int box_preload = 0;    // 1: never launch equal boxes of full tiles from preloaded arguments
 };
 Tuning& tuning();
 

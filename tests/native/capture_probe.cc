@@ -175,9 +175,9 @@ int main(int argc, char** argv) {
       CK(hipGraphKernelNodeGetParams(kernels[i], &kp));
       std::vector<unsigned char> want(4096);
       size_t size = 0;
-      uint32_t gx = 0, gy = 0, block = 0, lds = 0;
-      if (plan_args(plan, bases.data(), P + 1, position[i], want.data(), want.size(), &size, &gx, &gy, &block, &lds) !=
-          MDH_OK) {
+      uint32_t gx = 0, gy = 0, block = 0, lds = 0, leading = 0;
+      if (plan_args(plan, bases.data(), P + 1, position[i], want.data(), want.size(), &size, &leading, &gx, &gy, &block,
+              &lds) != MDH_OK) {
         std::printf("%s: step_arguments: %s\n", c.name, last_error());
         return 1;
       }
@@ -195,7 +195,26 @@ int main(int argc, char** argv) {
         ok = false;
         continue;
       }
-      const unsigned char* got = (const unsigned char*)kp.kernelParams[0];
+      // the passed block: `leading` 4-byte scalars, each a parameter of its own, then one struct
+      std::vector<unsigned char> recorded(size);
+      bool complete = true;
+      for (uint32_t k = 0; k <= leading; ++k) {
+        if (!kp.kernelParams[k]) {
+          complete = false;
+          break;
+        }
+        if (k < leading) {
+          std::memcpy(recorded.data() + 4 * k, kp.kernelParams[k], 4);
+        } else {
+          std::memcpy(recorded.data() + 4 * leading, kp.kernelParams[k], size - 4 * leading);
+        }
+      }
+      if (!complete) {
+        std::printf("%s: launch %d: the node holds fewer than %u parameters\n", c.name, position[i], leading + 1);
+        ok = false;
+        continue;
+      }
+      const unsigned char* got = recorded.data();
       size_t first = size;
       for (size_t k = 0; k < size; ++k) {
         if (got[k] != want[k]) {

@@ -36,6 +36,66 @@ def test_the_three_compiled_redistributions_of_the_benchmark():
         p.verify([8 * 512 * 1024 * 2] * 8 + [64 * 512 * 128 * 2])
 
 
+def test_equal_boxes_of_full_tiles_start_from_leading_scalar_arguments():
+    # The shards of a redistribution (at most eight boxes of one shape, full tiles only) are launched
+    # with fourteen leading 4-byte arguments -- source row pitch, tile shape, eight 48-bit source
+    # addresses -- in front of the table; anything else with the table alone.
+    import struct
+
+    specs = [(1024 * 8192 * 4, 1024 * 3, s * 1024 * 1024, [1024, 1024], [8192, 1], [1024, 1]) for s in range(8)]
+    p = plan_for(specs, 4)
+    bases = [0x7F12_3456_0000 + (s << 33) + 16 * s for s in range(8)] + [0x7E00_0000_1000]
+    args, lead, gx, gy, block, lds = p.step_arguments(bases, 0)
+    assert lead == 14 and gy == 8 and block == 256
+    words = struct.unpack("<14I", args[:56])
+    assert words[0] == 8192 * 4                       # source row pitch in bytes
+    log2tc, nct = words[1] & 31, words[1] >> 5
+    assert (1 << log2tc) == 4096 // 16 and nct == 1   # a row of 4 KiB is one tile's width
+    assert gx * (512 >> log2tc) == 1024               # every row of tiles is full (two sub-tiles: 512 slots)
+    for s in range(8):
+        pair = words[10 + s // 2]
+        address = ((pair >> 16 if s & 1 else pair & 0xFFFF) << 32) | words[2 + s]
+        assert address == bases[s] + 1024 * 3 * 4
+    # the table that follows holds the same boxes: source and destination address lead each entry
+    src0, dst0 = struct.unpack("<QQ", args[56:72])
+    assert src0 == bases[0] + 1024 * 3 * 4 and dst0 == bases[8]
+    # nine boxes, rows that are not whole vectors, or a ragged last row of tiles: the table form
+    for other in (
+        [(1024 * 8192 * 4, 0, s * 1024 * 1024, [1024, 1024], [8192, 1], [1024, 1]) for s in range(9)],
+        [(1024 * 8192 * 2, 0, s * 1024 * 1021, [1024, 1021], [8192, 1], [1021, 1]) for s in range(8)],
+        [(1023 * 8192 * 4, 0, s * 1023 * 1024, [1023, 1024], [8192, 1], [1024, 1]) for s in range(8)],
+    ):
+        q = plan_for(other, 4 if other[0][3][1] == 1024 else 2)
+        n = len(other)
+        b = [0x7F00_0000_0000 + (s << 33) for s in range(n + 1)]
+        for step in range(q.launches):
+            assert q.step_arguments(b, step)[1] == 0
+    # an address beyond 48 bits cannot be packed: the same plan then takes the table form
+    assert p.step_arguments([1 << 50] + bases[1:], 0)[1] == 0
+    # a dense gather of eight equal shards: the segments' length and the packed source addresses
+    shard = 1 << 20
+    g = plan_for([(shard, 0, r * shard, [shard], [1], [1]) for r in range(8)], 1)
+    assert g.launches == 1
+    g.verify([shard] * 8 + [8 * shard])
+    args, lead, gx, gy, block, lds = g.step_arguments(bases, 0)
+    assert lead == 14 and gy == 8
+    words = struct.unpack("<14I", args[:56])
+    assert words[0] == shard and gx * 256 * 16 * 4 == shard   # four sub-tiles of 4 KiB per workgroup
+    for r in range(8):
+        pair = words[10 + r // 2]
+        assert (((pair >> 16 if r & 1 else pair & 0xFFFF) << 32) | words[2 + r]) == bases[r]
+    # unequal shards, or shards off the 16-byte grid (heads and tails): the table form
+    lens = [shard, shard, shard - 16, shard]
+    at, specs = 0, []
+    for n in lens:
+        specs.append((n, 0, at, [n], [1], [1]))
+        at += n
+    u = plan_for(specs, 1)
+    assert all(u.step_arguments(bases[:4] + [bases[8]], k)[1] == 0 for k in range(u.launches))
+    r = plan_for([(shard + 2, 0, k * (shard + 2), [shard + 2], [1], [1]) for k in range(8)], 1)
+    assert all(r.step_arguments(bases, k)[1] == 0 for k in range(r.launches))
+
+
 def test_strided_gather_and_dense_gather_shapes():
     # [8, rows, cols] bf16 gather into a padded row pitch, scaled down 4x per side from the benchmark's
     rows, cols, pad = 1024, 1024, 64
