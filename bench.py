@@ -26,17 +26,17 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 CLOCK_WARMUP_S = 0.3   # untimed launches before the first timed window
 TIMED_WINDOWS = 11     # windows of `steps` launches; the median window is reported
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch), each
-# scaled by what the same counter reads for the flat copy of exactly 256 MiB (FETCH_SIZE x 1.99991,
+# scaled by what the same counter reads for the flat copy of exactly 256 MiB (FETCH_SIZE x 1.99982,
 # WRITE_SIZE x 1.00000): profiles/hbm_traffic_pmc_reduce_and_copy_kernels.md.  E.g. the headline:
-# 65,552.31 x 1.99991 + 16,384.00 KiB = 147,482.6 KiB.  Workloads without an entry were not measured.
+# 65,552.38 x 1.99982 + 16,384.00 KiB = 147,477.2 KiB.  Workloads without an entry were not measured.
 MEASURED_TRAFFIC_BYTES = {
-    "reduce_fp32_p8": 151022184,
-    "reduce_bf16_p16": 1140903271,
-    "reduce_fp32_p64_sum": 272676106,
+    "reduce_fp32_p8": 151016678,
+    "reduce_bf16_p16": 1140857916,
+    "reduce_fp32_p64_sum": 272664743,
     "allgather_bf16_p8": 536870912,
-    "allgather_bf16_p8_strided": 536907866,
-    "redistribute_fp32_8192": 67156871,
-    "redistribute_bf16_3d": 16825557,
+    "allgather_bf16_p8_strided": 536887363,
+    "redistribute_fp32_8192": 67146416,
+    "redistribute_bf16_3d": 16815987,
 }
 
 def box_kernel(abi):

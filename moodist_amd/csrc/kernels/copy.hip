@@ -51,7 +51,9 @@ struct CopyArgs {
   uint32_t total_tiles;
   uint32_t tiles_per_box; // non-zero when every box has the same tile count
 };
-static_assert(sizeof(CopyArgs) <= 4096, "kernel arguments are limited to 4 KiB");
+// with fourteen leading scalars in front (copy_rows16_kernel) and the compiler's 256 bytes of
+// hidden arguments behind
+static_assert(sizeof(CopyArgs) + 56 + 256 <= 4096, "kernel arguments are limited to 4 KiB");
 
 template<int VEC>
 struct VecType;
@@ -369,7 +371,7 @@ struct FlatArgs {
   uint32_t tiles_per_seg; // non-zero when every segment has the same tile count
   uint32_t edge_wgs;      // non-zero: some segment has a head or a tail
 };
-static_assert(sizeof(FlatArgs) <= 4096, "kernel arguments are limited to 4 KiB");
+static_assert(sizeof(FlatArgs) + 56 + 256 <= 4096, "kernel arguments are limited to 4 KiB");
 
 // Edge bytes are numbered per segment: slots 0..63 are the head's bytes, 64..79 the tail's.
 constexpr uint32_t kEdgeSlots = 80;
