@@ -429,6 +429,71 @@ def test_plan_random_boxes_against_copy_boxes(dev):
         _plan_vs_boxes(dev, specs, itemsize)
 
 
+@pytest.mark.parametrize("preload", [0, 1])
+def test_equal_shards_started_from_preloaded_arguments(dev, preload):
+    # Up to eight equal boxes of full tiles (copy_rows16_kernel) and up to eight equal dense shards
+    # (copy_flat8_kernel) take their source addresses from leading scalar arguments; with the knob
+    # box_preload=1 the same calls run the table kernels.  Expected bytes come from torch slicing.
+    stream = torch.cuda.current_stream().cuda_stream
+    g = torch.Generator().manual_seed(11)
+    abi.set_tuning("box_preload", preload)
+    try:
+        for P, rows, row_bytes, src_pitch, dst_pitch, src_off, full_tiles in (
+            (8, 64, 4096, 32768, 4096, 8192, True),     # the redistribution's shape, scaled down
+            (8, 512, 256, 2048, 256, 1280, True),       # 256-byte runs
+            (5, 32, 8192, 8192, 8192 + 128, 0, True),   # a gather into a padded pitch
+            (3, 8, 1024, 4096, 2048, 48, True),
+            (3, 2, 1024, 4096, 2048, 48, False),        # two rows in tiles of four: the table form
+            (1, 128, 512, 1024, 512, 512, True),
+            (8, 4, 16384, 65536, 16384, 32768, True),   # rows longer than a tile is wide
+        ):
+            srcs = [torch.randint(0, 256, (rows * src_pitch + 64,), dtype=torch.uint8, generator=g) for _ in range(P)]
+            dsrc = [x.to(dev) for x in srcs]
+            out = torch.full((P * rows * dst_pitch + 64,), 0xA5, dtype=torch.uint8, device=dev)
+            want = torch.full((P * rows * dst_pitch + 64,), 0xA5, dtype=torch.uint8)
+            for s in range(P):
+                for r in range(rows):
+                    a = src_off + r * src_pitch
+                    d = (s * rows + r) * dst_pitch
+                    want[d:d + row_bytes] = srcs[s][a:a + row_bytes]
+            offs = [abi.make_box(src_off, s * rows * dst_pitch, [rows, row_bytes], [src_pitch, 1], [dst_pitch, 1])
+                    for s in range(P)]
+            plan = abi.CopyPlan(offs, list(range(P)), [P] * P, 1, P + 1)
+            bases = [x.data_ptr() for x in dsrc] + [out.data_ptr()]
+            assert plan.launches == 1
+            assert plan.step_arguments(bases, 0)[1] == (14 if full_tiles and not preload else 0), (P, rows, row_bytes)
+            plan.launch(bases, stream)
+            sync()
+            assert torch.equal(out.cpu(), want), (P, rows, row_bytes)
+            # the general entry point, with sources off the 16-byte grid
+            out.fill_(0xA5)
+            shifted = [torch.cat([torch.zeros(6, dtype=torch.uint8), x]).to(dev) for x in srcs]
+            boxes = [abi.make_box(shifted[s].data_ptr() + 6 + src_off, out.data_ptr() + s * rows * dst_pitch,
+                                  [rows, row_bytes], [src_pitch, 1], [dst_pitch, 1]) for s in range(P)]
+            abi.copy_boxes(boxes, 1, stream)
+            sync()
+            assert torch.equal(out.cpu(), want), (P, rows, row_bytes, "unaligned sources")
+        for P, shard in ((2, 64), (5, 4096), (8, 65536 + 64), (8, 1 << 20), (7, 12288)):
+            srcs = [torch.randint(0, 256, (shard,), dtype=torch.uint8, generator=g) for _ in range(P)]
+            dsrc = [x.to(dev) for x in srcs]
+            out = torch.full((P * shard + 64,), 0x5A, dtype=torch.uint8, device=dev)
+            want = torch.cat(srcs + [torch.full((64,), 0x5A, dtype=torch.uint8)])
+            offs = [abi.make_box(0, s * shard, [shard], [1], [1]) for s in range(P)]
+            plan = abi.CopyPlan(offs, list(range(P)), [P] * P, 1, P + 1)
+            bases = [x.data_ptr() for x in dsrc] + [out.data_ptr()]
+            assert plan.launches == 1
+            assert plan.step_arguments(bases, 0)[1] == (0 if preload else 14), (P, shard)
+            plan.launch(bases, stream)
+            sync()
+            assert torch.equal(out.cpu(), want), (P, shard)
+            out.fill_(0x5A)
+            abi.gather([x.data_ptr() for x in dsrc], out.data_ptr(), shard, 1, shard, shard, shard, stream)
+            sync()
+            assert torch.equal(out.cpu(), want), (P, shard, "mdh_gather")
+    finally:
+        abi.set_tuning("box_preload", 0)
+
+
 def test_host_cost_of_a_compiled_redistribution_from_cpp(dev):
     # the C++ loop: enqueuing a prepared plan must cost the host less than the fp32 8192 x 8192 kernel
     # takes (about 12 us) and no more than the general entry point does -- both are mostly the
