@@ -664,19 +664,40 @@ struct Launcher {
   int rc = MDH_OK;
   int unroll = 2; // sub-tiles of the box launch being assembled
 
-  // Copies of 128 MiB and more run long enough to settle into a steady state in which reads
-  // and writes interleave at the DRAM; two sub-tiles with four workgroups per CU (an unused LDS
-  // allocation holds the others back) then move 4-10 % more than the shape that is best for
-  // short launches.  Measured on 8 x 32 MiB: 6.58 against 6.29 TB/s dense, 6.15 against 5.61 TB/s
-  // with a padded row pitch; at 64 MiB and below a cap gains nothing or costs.
-  static constexpr uint64_t kLongCopyBytes = (uint64_t)128 << 20;
+  // Launch shapes, measured with every operand coming from HBM (the launches rotate over 4 GiB):
+  // sub-tiles per lane x workgroups resident per CU (an unused LDS allocation holds the others
+  // back; "-" = no cap), us per launch.
+  //   dense, 8 shards of    1 MiB   4 MiB   8 MiB  16 MiB  32 MiB  64 MiB
+  //     1 x -                4.06   11.72   21.61   41.70   81.87
+  //     2 x -                4.18   12.30   22.35   43.02   85.67
+  //     4 x -                4.20   12.12   22.53   43.40   86.46
+  //     2 x 4                4.03   11.82   21.48   40.72   80.62  162.33
+  //     2 x 3                4.29   11.43   20.97   40.10   78.74  154.97
+  //     4 x 2                4.09   11.90   21.64   41.34   81.18  165.87
+  //   strided, 8 boxes     256 B x 4096   2 KiB x 1024   4 KiB x 1024   4 KiB x 4096   8 KiB x 4096 (padded pitch)
+  //     1 x -                  4.41           7.40          11.57          40.83          79.14
+  //     2 x -                  4.37           7.55          12.23          42.77          84.43
+  //     2 x 4                  4.34           7.64          11.76          41.06          80.24
+  //     2 x 3                  4.81           7.56          11.68          40.48          79.60
+  // Dense copies of equal segments (the two-dimensional form of the grid), 32 MiB and more: two
+  // sub-tiles, three workgroups per CU (24 KiB in flight per CU; the same bytes as six workgroups
+  // of one sub-tile, which take 41.5 us where these take 40.1); shorter ones: one sub-tile, every
+  // workgroup resident.  Unequal or ragged segments (the one-dimensional form, whose workgroups
+  // scan the segment table for every tile they take and do better with longer tiles): four
+  // sub-tiles, from 128 MiB on two with four workgroups per CU (8 shards of 1 MiB + 2 bytes 5.8
+  // against 6.2 us with the shape of the equal form, of 32 MiB + 2 bytes 86.7 against 90.2).
+  // Strided boxes: one sub-tile and no cap throughout, except launches of 8 MiB and less, which
+  // are over in 4 us and do better with half as many workgroups to dispatch.
+  static constexpr uint64_t kCappedCopyBytes = (uint64_t)32 << 20;
+  static constexpr uint64_t kLongRaggedBytes = (uint64_t)128 << 20;
+  static constexpr uint64_t kShortBoxBytes = (uint64_t)8 << 20;
   size_t lds = 0; // of the launch being assembled
   bool plain_loads = false;
 
-  void choose_cap(uint64_t bytes) {
-    int cap = tuning().copy_wg_per_cu;
-    if (cap == 0 && bytes >= kLongCopyBytes) {
-      cap = 4;
+  // `cap` is the library's own choice (0 = none), which the knob overrides
+  void choose_cap(int cap) {
+    if (tuning().copy_wg_per_cu) {
+      cap = tuning().copy_wg_per_cu;
     }
     lds = cap >= 2 && cap <= 8 ? kLdsForCap[cap] : 0; // one per CU would need the LDS limit raised
   }
@@ -687,8 +708,23 @@ struct Launcher {
     for (const Segment& g : flat) {
       all_vectors += g.bytes / 16;
     }
-    const int U = t.copy_unroll ? t.copy_unroll : all_vectors * 16 >= kLongCopyBytes ? 2 : auto_unroll(all_vectors, 4);
-    choose_cap(all_vectors * 16);
+    bool even = flat.size() > 1;
+    for (const Segment& g : flat) {
+      even = even && g.bytes == flat[0].bytes && !g.head && !g.tail;
+    }
+    const uint64_t all_bytes = all_vectors * 16;
+    int U, cap;
+    if (even) {
+      U = all_bytes >= kCappedCopyBytes ? 2 : 1;
+      cap = all_bytes >= kCappedCopyBytes ? 3 : 0;
+    } else {
+      U = all_bytes >= kLongRaggedBytes ? 2 : auto_unroll(all_vectors, 4);
+      cap = all_bytes >= kLongRaggedBytes ? 4 : 0;
+    }
+    if (t.copy_unroll) {
+      U = t.copy_unroll;
+    }
+    choose_cap(cap);
     const uint64_t tile_bytes = (uint64_t)kBlock * U * 16;
     size_t i = 0;
     while (i < flat.size()) {
@@ -788,10 +824,10 @@ struct Launcher {
     for (const BoxDesc& d : list) {
       all_vectors += (uint64_t)d.rows * d.cols;
     }
-    choose_cap(lg == 5 ? all_vectors * 16 : 0); // the 16-byte buffer kernel only
+    const uint64_t all_bytes = all_vectors * (lg == 5 ? 16u : 1u << lg);
+    choose_cap(0); // (a cap exists for the 16-byte buffer kernel only, and only by the knob)
     plain_loads = tuning().box_policy == 1;
-    // strided boxes: two sub-tiles measured best on large gathers (6.1 against 5.9 TB/s with four)
-    const int U = tuning().box_unroll ? tuning().box_unroll : auto_unroll(all_vectors, 2);
+    const int U = tuning().box_unroll ? tuning().box_unroll : all_bytes <= kShortBoxBytes ? auto_unroll(all_vectors, 2) : 1;
     unroll = U;
     const uint32_t slots = (uint32_t)kBlock * (uint32_t)U;
     size_t i = 0;

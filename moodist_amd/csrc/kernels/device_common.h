@@ -100,10 +100,9 @@ Tuning& tuning();
 // (index n): the only handle a launch has on how many workgroups a CU holds at once.
 constexpr size_t kLdsForCap[9] = {0, 98304, 65536, 49152, 40960, 32768, 27136, 23296, 20480};
 
-// Sub-tiles per lane.  More sub-tiles mean more loads in flight per lane and longer contiguous
-// pieces per workgroup (faster once the chip is full: 23.6 us with four against 28.5 us with one
-// on 8 x 16 MiB), but fewer workgroups; below about one workgroup per CU the smaller tile wins
-// (1 MiB per source: 3.6 us with one against 4.8 us with four).
+// Sub-tiles per lane, where longer tiles are wanted (short strided launches, dense copies of
+// unequal segments): the widest that still leaves a workgroup for every CU -- below one per CU
+// the smaller tile wins (1 MiB per source took 3.6 us with one sub-tile against 4.8 us with four).
 inline int auto_unroll(uint64_t vectors, int widest) {
   int u = widest;
   while (u > 1 && vectors / ((uint64_t)kBlock * u) < 256) {

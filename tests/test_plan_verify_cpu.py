@@ -51,7 +51,7 @@ def test_equal_boxes_of_full_tiles_start_from_leading_scalar_arguments():
     assert words[0] == 8192 * 4                       # source row pitch in bytes
     log2tc, nct = words[1] & 31, words[1] >> 5
     assert (1 << log2tc) == 4096 // 16 and nct == 1   # a row of 4 KiB is one tile's width
-    assert gx * (512 >> log2tc) == 1024               # every row of tiles is full (two sub-tiles: 512 slots)
+    assert gx % nct == 0 and 1024 % (gx // nct) == 0  # whole rows of tiles, each of the same number of rows
     for s in range(8):
         pair = words[10 + s // 2]
         address = ((pair >> 16 if s & 1 else pair & 0xFFFF) << 32) | words[2 + s]
@@ -63,9 +63,9 @@ def test_equal_boxes_of_full_tiles_start_from_leading_scalar_arguments():
     for other in (
         [(1024 * 8192 * 4, 0, s * 1024 * 1024, [1024, 1024], [8192, 1], [1024, 1]) for s in range(9)],
         [(1024 * 8192 * 2, 0, s * 1024 * 1021, [1024, 1021], [8192, 1], [1021, 1]) for s in range(8)],
-        [(1023 * 8192 * 4, 0, s * 1023 * 1024, [1023, 1024], [8192, 1], [1024, 1]) for s in range(8)],
+        [(1023 * 8192 * 4, 0, s * 1023 * 512, [1023, 512], [8192, 1], [512, 1]) for s in range(8)],
     ):
-        q = plan_for(other, 4 if other[0][3][1] == 1024 else 2)
+        q = plan_for(other, 2 if other[0][3][1] == 1021 else 4)
         n = len(other)
         b = [0x7F00_0000_0000 + (s << 33) for s in range(n + 1)]
         for step in range(q.launches):
@@ -80,7 +80,7 @@ def test_equal_boxes_of_full_tiles_start_from_leading_scalar_arguments():
     args, lead, gx, gy, block, lds = g.step_arguments(bases, 0)
     assert lead == 14 and gy == 8
     words = struct.unpack("<14I", args[:56])
-    assert words[0] == shard and gx * 256 * 16 * 4 == shard   # four sub-tiles of 4 KiB per workgroup
+    assert words[0] == shard and shard % gx == 0 and (shard // gx) % 4096 == 0   # whole sub-tiles of 4 KiB
     for r in range(8):
         pair = words[10 + r // 2]
         assert (((pair >> 16 if r & 1 else pair & 0xFFFF) << 32) | words[2 + r]) == bases[r]
