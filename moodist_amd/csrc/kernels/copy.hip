@@ -666,7 +666,8 @@ struct Launcher {
 
   // Launch shapes, measured with every operand coming from HBM (the launches rotate over 4 GiB):
   // sub-tiles per lane x workgroups resident per CU (an unused LDS allocation holds the others
-  // back; "-" = no cap), us per launch.
+  // back; "-" = no cap), us per launch.  (Zero-filled buffers, which copy 2-3 % faster than any
+  // other data; the order of the shapes is the same with random data.)
   //   dense, 8 shards of    1 MiB   4 MiB   8 MiB  16 MiB  32 MiB  64 MiB
   //     1 x -                4.06   11.72   21.61   41.70   81.87
   //     2 x -                4.18   12.30   22.35   43.02   85.67
