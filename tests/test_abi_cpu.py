@@ -68,6 +68,7 @@ def test_box_struct_layout_matches_header():
     (lambda: abi.set_tuning("reduce_wg_per_cu", 10), "does not take 10"),
     (lambda: abi.set_tuning("no_such_knob", 1), "unknown knob"),
     (lambda: abi.set_tuning("reduce_unroll", 3), "does not take 3"),
+    (lambda: abi.set_tuning("box_preload", 2), "does not take 2"),
 ])
 def test_bad_arguments_are_refused_before_launch(call, match):
     with pytest.raises(abi.MoodistError, match=match):
@@ -87,6 +88,10 @@ def test_tuning_round_trip():
     abi.set_tuning("copy_unroll", 2)
     assert abi.get_tuning("copy_unroll") == 2
     abi.set_tuning("copy_unroll", old)
+    assert abi.get_tuning("box_preload") == 0
+    abi.set_tuning("box_preload", 1)
+    assert abi.get_tuning("box_preload") == 1
+    abi.set_tuning("box_preload", 0)
 
 
 def test_missing_kernel_library_fails_loudly(monkeypatch, tmp_path):
