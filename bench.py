@@ -46,9 +46,9 @@ def box_kernel(abi):
 
 
 def flat_kernel(abi, sources, shard_bytes):
-    """The dense-gather kernel: up to eight equal shards on the 64-byte grid start from preloaded
-    arguments (copy_flat8_kernel), anything else from the segment table."""
-    early = 1 < sources <= 8 and shard_bytes % 64 == 0 and abi.get_tuning("box_preload") != 1
+    """The dense-gather kernel: up to eight equal shards start from preloaded arguments
+    (copy_flat8_kernel), anything else from the segment table."""
+    early = 1 < sources <= 8 and shard_bytes >= 32 and abi.get_tuning("box_preload") != 1
     return "copy_flat8_kernel" if early else "copy_flat_kernel"
 
 

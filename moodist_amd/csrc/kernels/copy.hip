@@ -362,21 +362,27 @@ struct FlatArgs {
   uint32_t tile_end[kMaxSegments]; // cumulative tiles; unused entries are ~0
   uint64_t bytes[kMaxSegments];    // of whole vectors: multiples of 16
   // The segment's first bytes, up to its destination's next 64-byte boundary, and its last
-  // < 16 bytes: they sit before src/dst and after src/dst + bytes, and are copied byte by byte
-  // by workgroups of their own, in front of the tile workgroups.
+  // bytes (fewer than 16, or fewer than 80 when equal segments were given one common length of
+  // whole vectors): they sit before src/dst and after src/dst + bytes, and are copied byte by
+  // byte by workgroups of their own, in front of the tile workgroups.
   uint8_t head[kMaxSegments]; // 0..63
-  uint8_t tail[kMaxSegments]; // 0..15
+  uint8_t tail[kMaxSegments]; // 0..79
   uint32_t nsegs;
   uint32_t total_tiles;
   uint32_t tiles_per_seg; // non-zero when every segment has the same tile count
-  uint32_t edge_wgs;      // non-zero: some segment has a head or a tail
+  // 0: no segment has a head or a tail.  1: some have, and the first kEdgeWgs workgroups of the
+  // one-dimensional grid copy them.  2: some have, and workgroup 0 of every row of the
+  // two-dimensional grid copies its segment's (the tiles are then workgroups 1, 2, ...).
+  uint32_t edge_wgs;
 };
 static_assert(sizeof(FlatArgs) + 56 + 256 <= 4096, "kernel arguments are limited to 4 KiB");
 
-// Edge bytes are numbered per segment: slots 0..63 are the head's bytes, 64..79 the tail's.
-constexpr uint32_t kEdgeSlots = 80;
-// Workgroups that copy them (the one-dimensional form of the grid; segments with edges are never
-// launched in the two-dimensional form): one lane per slot of a full table.
+// Edge bytes are numbered per segment: slots 0..63 are the head's bytes, 64..143 the tail's.
+constexpr uint32_t kMaxTail = 80;
+constexpr uint32_t kEdgeSlots = 64 + kMaxTail;
+static_assert(kEdgeSlots <= (uint32_t)kBlock, "one workgroup has a lane for every edge byte of a segment");
+// Workgroups that copy them in the one-dimensional form of the grid: one lane per slot of a
+// full table.
 constexpr uint32_t kEdgeWgs = (kMaxSegments * kEdgeSlots + 255) / 256;
 
 // The byte a slot stands for, as an offset from the segment's src/dst (negative in the head);
@@ -430,13 +436,25 @@ __device__ __attribute__((noinline)) void copy_edges(const FlatArgs* args, uint3
   }
 }
 
-// EQUAL: as for the boxes -- segments of equal tile count and without heads or tails,
-// blockIdx.y the segment, blockIdx.x the tile.  Otherwise the first kEdgeWgs workgroups of the
+// The two-dimensional form: the edge bytes of one segment, one per lane, by workgroup 0 of the
+// segment's row.  Out of line for the same reason.
+__device__ __attribute__((noinline)) void copy_segment_edges(const FlatArgs* args, uint32_t seg, uint32_t lane) {
+  const FlatArgs& a = *args;
+  int64_t off;
+  if (lane < kEdgeSlots && edge_offset(a, seg, lane, &off)) {
+    a.dst[seg][off] = a.src[seg][off];
+  }
+}
+
+// EQUAL: as for the boxes -- segments of equal tile count, blockIdx.y the segment, blockIdx.x the
+// tile; when they have heads or tails (edge_wgs == 2) workgroup 0 of every row copies those and
+// the tiles are workgroups 1, 2, ...  Otherwise the first kEdgeWgs workgroups of the
 // grid are the edge workgroups -- ALWAYS, finding nothing to do when no segment has a head or a
 // tail: a tile workgroup then knows what it is from blockIdx alone, and its first loads do not
 // wait for a kernel argument to decide it.
-template<int U, bool EQUAL>
+template<int U, bool EQUAL, bool EDGES = false>
 __global__ __launch_bounds__(kBlock) void copy_flat_kernel(FlatArgs a) {
+  static_assert(EQUAL || !EDGES, "the edge column belongs to the two-dimensional form");
   constexpr uint32_t tile_bytes = kBlock * U * 16;
   const uint32_t lane_byte = threadIdx.x * 16;
   uint32_t first_tile = blockIdx.x, tile_wgs = 0;
@@ -452,7 +470,14 @@ __global__ __launch_bounds__(kBlock) void copy_flat_kernel(FlatArgs a) {
   uint32_t tile = first_tile; // untested, as in the box kernels
   do {
     uint32_t local;
-    const uint32_t seg = EQUAL ? (local = blockIdx.x, row) : locate_segment(a, tile, &local);
+    if (EDGES) { // (a template argument: read from the table, it would cost the tiles a scalar round trip)
+      if (blockIdx.x == 0) {
+        copy_segment_edges((const FlatArgs*)__builtin_amdgcn_kernarg_segment_ptr(), row, threadIdx.x);
+        return;
+      }
+      tile = blockIdx.x - 1;
+    }
+    const uint32_t seg = EQUAL ? (local = tile, row) : locate_segment(a, tile, &local);
     const uint64_t off = (uint64_t)local * tile_bytes;
     const uint64_t left = a.bytes[seg] - off;
     const uint32_t n = left < tile_bytes ? (uint32_t)left : tile_bytes;
@@ -478,14 +503,25 @@ __global__ __launch_bounds__(kBlock) void copy_flat_kernel(FlatArgs a) {
 // shards) -- started from preloaded arguments like copy_rows16_kernel: the segments' length and
 // their source addresses arrive in registers, the destination's address is read from the table
 // while the vector loads are in flight.
-template<int U>
+//
+// EDGES: the segments have heads or tails -- shards whose length is not a whole number of
+// vectors, or whose destinations are off the 64-byte grid, cut to one common length of whole
+// vectors.  Workgroup 0 of every row copies its segment's edge bytes and the tiles are
+// workgroups 1, 2, ...: a workgroup knows which it is from blockIdx alone.
+template<int U, bool EDGES>
 __global__ __launch_bounds__(kBlock) void copy_flat8_kernel(uint32_t bytes, uint32_t, uint32_t l0, uint32_t l1, uint32_t l2,
     uint32_t l3, uint32_t l4, uint32_t l5, uint32_t l6, uint32_t l7, uint32_t h0, uint32_t h1, uint32_t h2, uint32_t h3,
     FlatArgs a) {
   constexpr uint32_t tile_bytes = kBlock * U * 16;
   const uint32_t lane_byte = threadIdx.x * 16;
   const uint32_t seg = blockIdx.y;
-  const uint32_t off = blockIdx.x * tile_bytes; // below the segment's length, which fits 32 bits
+  if (EDGES && blockIdx.x == 0) {
+    // FlatArgs follows the fourteen leading dwords in the argument segment
+    const char* segment = (const char*)__builtin_amdgcn_kernarg_segment_ptr();
+    copy_segment_edges((const FlatArgs*)(segment + sizeof(FlatLead)), seg, threadIdx.x);
+    return;
+  }
+  const uint32_t off = (blockIdx.x - (EDGES ? 1u : 0u)) * tile_bytes; // below the segment's length, which fits 32 bits
   const uint32_t left = bytes - off;
   const uint32_t n = left < tile_bytes ? left : tile_bytes;
   const char* src = (const char*)(uintptr_t)packed_source_address(seg, l0, l1, l2, l3, l4, l5, l6, l7, h0, h1, h2, h3);
@@ -533,6 +569,7 @@ struct Step {
   uint32_t grid_y; // > 0: the two-dimensional form for equal boxes / segments (grid x grid_y workgroups)
   bool plain_loads; // kBoxes16: plain instead of nt loads (tuning knob)
   bool preloaded = false; // equal boxes of full tiles / equal segments of one length: started from preloaded arguments
+  bool edge_column = false; // kFlat, two-dimensional form: workgroup 0 of every row copies its segment's edge bytes
   size_t lds;
   FlatArgs flat;   // kFlat
   CopyArgs boxes;  // kBoxes16, kBoxes
@@ -620,7 +657,7 @@ inline bool make_rows_lead(const CopyArgs& a, RowsLead* lead) {
 // Whether a two-dimensional launch of flat segments qualifies for copy_flat8_kernel: at most
 // eight segments, all of the same length.
 inline bool uniform_segments(const FlatArgs& a) {
-  if (a.nsegs == 0 || a.nsegs > (uint32_t)kEarlyBoxes || a.tiles_per_seg == 0 || a.edge_wgs != 0) {
+  if (a.nsegs == 0 || a.nsegs > (uint32_t)kEarlyBoxes || a.tiles_per_seg == 0 || a.edge_wgs == 1) {
     return false;
   }
   for (uint32_t k = 0; k < a.nsegs; ++k) {
@@ -641,7 +678,7 @@ inline bool make_flat_lead(const FlatArgs& a, FlatLead* lead) {
 // one-dimensional form of a flat step the edge workgroups in front of them.
 inline void launch_dims(const Step& st, uint32_t* x, uint32_t* y) {
   if (st.grid_y > 0) {
-    *x = st.grid;
+    *x = st.grid + (st.edge_column ? 1u : 0u);
     *y = st.grid_y;
   } else {
     *x = st.grid + (st.kind == Step::kFlat ? kEdgeWgs : 0u);
@@ -683,10 +720,9 @@ struct Launcher {
   // Dense copies of equal segments (the two-dimensional form of the grid), 32 MiB and more: two
   // sub-tiles, three workgroups per CU (24 KiB in flight per CU; the same bytes as six workgroups
   // of one sub-tile, which take 41.5 us where these take 40.1); shorter ones: one sub-tile, every
-  // workgroup resident.  Unequal or ragged segments (the one-dimensional form, whose workgroups
-  // scan the segment table for every tile they take and do better with longer tiles): four
-  // sub-tiles, from 128 MiB on two with four workgroups per CU (8 shards of 1 MiB + 2 bytes 5.8
-  // against 6.2 us with the shape of the equal form, of 32 MiB + 2 bytes 86.7 against 90.2).
+  // workgroup resident.  Unequal segments (the one-dimensional form, whose workgroups scan the
+  // segment table for every tile they take and do better with longer tiles): four sub-tiles,
+  // from 128 MiB on two with four workgroups per CU.
   // Strided boxes: one sub-tile and no cap throughout, except launches of 8 MiB and less, which
   // are over in 4 us and do better with half as many workgroups to dispatch.
   static constexpr uint64_t kCappedCopyBytes = (uint64_t)32 << 20;
@@ -709,13 +745,40 @@ struct Launcher {
     for (const Segment& g : flat) {
       all_vectors += g.bytes / 16;
     }
-    bool even = flat.size() > 1;
+    bool even = flat.size() > 1, same_total = flat.size() > 1;
+    uint64_t shortest = flat.empty() ? 0 : flat[0].bytes;
     for (const Segment& g : flat) {
       even = even && g.bytes == flat[0].bytes && !g.head && !g.tail;
+      same_total = same_total && g.head + g.bytes + g.tail == flat[0].head + flat[0].bytes + flat[0].tail;
+      shortest = g.bytes < shortest ? g.bytes : shortest;
+    }
+    // Segments of one total length whose heads differ (shards that are not a whole number of
+    // vectors, or land off the 64-byte grid): all get the shortest one's whole vectors, and the
+    // longer tails (fewer than 80 bytes) go with the edge bytes.  They are then equal segments
+    // and take the two-dimensional form.
+    bool cut = false;
+    if (!even && same_total && shortest > 0) {
+      for (Segment& g : flat) {
+        const uint64_t tail = g.bytes - shortest + g.tail;
+        if (tail >= kMaxTail) {
+          same_total = false;
+        }
+      }
+      if (same_total) {
+        for (Segment& g : flat) {
+          g.tail = (uint8_t)(g.bytes - shortest + g.tail);
+          g.bytes = shortest;
+        }
+        even = cut = true;
+      }
     }
     const uint64_t all_bytes = all_vectors * 16;
     int U, cap;
-    if (even) {
+    if (cut) {
+      // sources off the 16-byte grid: one sub-tile and no cap at every size (8 x (32 MiB + 2)
+      // 83.7 us, against 87.5 with the shape of aligned segments and 84.9 with 2 x 4)
+      U = 1, cap = 0;
+    } else if (even) {
       U = all_bytes >= kCappedCopyBytes ? 2 : 1;
       cap = all_bytes >= kCappedCopyBytes ? 3 : 0;
     } else {
@@ -773,8 +836,10 @@ struct Launcher {
       Step st;
       st.kind = Step::kFlat, st.vec = 16, st.unroll = U, st.grid = grid, st.grid_y = 0, st.lds = lds;
       st.plain_loads = false;
-      if (a.tiles_per_seg && grid == a.total_tiles && a.nsegs > 1 && !edges) {
+      if (a.tiles_per_seg && grid == a.total_tiles && a.nsegs > 1) {
         st.grid = a.tiles_per_seg, st.grid_y = a.nsegs;
+        st.edge_column = edges;
+        a.edge_wgs = edges ? 2 : 0;
         st.preloaded = t.box_preload != 1 && uniform_segments(a);
       }
       submit(st, &a, nullptr);
@@ -1146,21 +1211,45 @@ int launch_step(const Step& st, const FlatArgs* flat, const CopyArgs* boxes, hip
   case Step::kFlat: {
     FlatLead L;
     if (st.preloaded && make_flat_lead(*flat, &L)) {
+#define MDH_LAUNCH_FLAT8(UU)                                                                                          \
+  if (st.edge_column) {                                                                                               \
+    hipLaunchKernelGGL((copy_flat8_kernel<UU, true>), g, b, st.lds, stream, L.bytes, L.reserved, MDH_PACKED(L.from), *flat);  \
+  } else {                                                                                                            \
+    hipLaunchKernelGGL((copy_flat8_kernel<UU, false>), g, b, st.lds, stream, L.bytes, L.reserved, MDH_PACKED(L.from), *flat); \
+  }
       switch (st.unroll) {
       case 1:
-        hipLaunchKernelGGL((copy_flat8_kernel<1>), g, b, st.lds, stream, L.bytes, L.reserved, MDH_PACKED(L.from), *flat);
+        MDH_LAUNCH_FLAT8(1)
         break;
       case 2:
-        hipLaunchKernelGGL((copy_flat8_kernel<2>), g, b, st.lds, stream, L.bytes, L.reserved, MDH_PACKED(L.from), *flat);
+        MDH_LAUNCH_FLAT8(2)
         break;
       case 4:
-        hipLaunchKernelGGL((copy_flat8_kernel<4>), g, b, st.lds, stream, L.bytes, L.reserved, MDH_PACKED(L.from), *flat);
+        MDH_LAUNCH_FLAT8(4)
         break;
       default:
-        hipLaunchKernelGGL((copy_flat8_kernel<8>), g, b, st.lds, stream, L.bytes, L.reserved, MDH_PACKED(L.from), *flat);
+        MDH_LAUNCH_FLAT8(8)
         break;
       }
+#undef MDH_LAUNCH_FLAT8
       return check_launch("copy_flat8_kernel");
+    }
+    if (st.edge_column) {
+      switch (st.unroll) {
+      case 1:
+        hipLaunchKernelGGL((copy_flat_kernel<1, true, true>), g, b, st.lds, stream, *flat);
+        break;
+      case 2:
+        hipLaunchKernelGGL((copy_flat_kernel<2, true, true>), g, b, st.lds, stream, *flat);
+        break;
+      case 4:
+        hipLaunchKernelGGL((copy_flat_kernel<4, true, true>), g, b, st.lds, stream, *flat);
+        break;
+      default:
+        hipLaunchKernelGGL((copy_flat_kernel<8, true, true>), g, b, st.lds, stream, *flat);
+        break;
+      }
+      return check_launch("copy_flat_kernel");
     }
     MDH_LAUNCH_COPY(copy_flat_kernel, , *flat)
     return check_launch("copy_flat_kernel");
@@ -1525,8 +1614,9 @@ extern "C" int mdh_copy_plan_verify(const mdh_copy_plan* plan, const uint64_t* b
           return MDH_EINVAL;
         }
       }
-      if (st.grid_y && a.edge_wgs) {
-        set_error("mdh_copy_plan_verify: step %zu: the two-dimensional form has no edge workgroups", s);
+      if ((st.grid_y != 0 && a.edge_wgs == 1) || (st.grid_y == 0 && a.edge_wgs == 2) ||
+          st.edge_column != (a.edge_wgs == 2)) {
+        set_error("mdh_copy_plan_verify: step %zu: edge workgroups of the other form of the grid", s);
         return MDH_EINVAL;
       }
       // copy_flat8_kernel takes every segment's length from one leading argument

@@ -84,7 +84,7 @@ def test_equal_boxes_of_full_tiles_start_from_leading_scalar_arguments():
     for r in range(8):
         pair = words[10 + r // 2]
         assert (((pair >> 16 if r & 1 else pair & 0xFFFF) << 32) | words[2 + r]) == bases[r]
-    # unequal shards, or shards off the 16-byte grid (heads and tails): the table form
+    # unequal shards: the table form
     lens = [shard, shard, shard - 16, shard]
     at, specs = 0, []
     for n in lens:
@@ -92,8 +92,16 @@ def test_equal_boxes_of_full_tiles_start_from_leading_scalar_arguments():
         at += n
     u = plan_for(specs, 1)
     assert all(u.step_arguments(bases[:4] + [bases[8]], k)[1] == 0 for k in range(u.launches))
+    # equal shards that are not a whole number of vectors: cut to one common length of whole
+    # vectors, their heads and tails copied by workgroup 0 of every row of the grid
     r = plan_for([(shard + 2, 0, k * (shard + 2), [shard + 2], [1], [1]) for k in range(8)], 1)
-    assert all(r.step_arguments(bases, k)[1] == 0 for k in range(r.launches))
+    assert r.launches == 1
+    r.verify([shard + 2] * 8 + [8 * (shard + 2)])
+    args, lead, gx, gy, block, lds = r.step_arguments(bases, 0)
+    assert lead == 14 and gy == 8
+    common = struct.unpack("<I", args[:4])[0]
+    assert common % 16 == 0 and shard + 2 - 64 - 16 < common <= shard + 2
+    assert (gx - 1) * 4096 >= common > (gx - 2) * 4096   # one workgroup more than the tiles of 4 KiB
 
 
 def test_strided_gather_and_dense_gather_shapes():
