@@ -24,7 +24,7 @@ from util import ALL_DTYPES, TORCH_TO_CODE, bits, same_bits
 pytestmark = pytest.mark.gpu
 OPS = [oracle.OP_SUM, oracle.OP_MIN, oracle.OP_MAX, oracle.OP_AVG, oracle.OP_PREMUL_SUM]
 KNOBS = ("reduce_unroll", "reduce_max_blocks", "reduce_wg_per_cu", "box_unroll", "copy_unroll", "copy_max_blocks",
-         "copy_wg_per_cu")
+         "copy_wg_per_cu", "box_preload")
 
 
 @pytest.fixture()
@@ -136,14 +136,15 @@ def test_copy_random_boxes_match_torch_slicing(dev, knobs, seed):
 
 @pytest.mark.parametrize("seed", [1, 2])
 def test_gather_random_shapes_match_numpy(dev, knobs, seed):
-    # 1..70 shards, 1..300 rows, widths with and without a 16-byte body, independent row pitches,
-    # byte misalignment of every shard and of the output, guard bytes between and after shards
+    # 1..70 shards, 1..300 rows, widths with and without a 16-byte body (among them the powers of
+    # two whose tiles are all full: the forms started from preloaded arguments), independent row
+    # pitches, byte misalignment of every shard and of the output, guard bytes between and after shards
     st = torch.cuda.current_stream().cuda_stream
     rng = random.Random(seed)
     for case in range(200):
         P = rng.choice([1, 2, 3, 8, 9, 33, 70])
-        rows = rng.choice([1, 1, 2, 5, 64, 300])
-        width = rng.choice([1, 3, 15, 16, 17, 100, 1000, 4096, 4100, rng.randint(1, 20000)])
+        rows = rng.choice([1, 1, 2, 5, 32, 64, 128, 300])
+        width = rng.choice([1, 3, 15, 16, 17, 100, 256, 1000, 2048, 4096, 4100, 8192, rng.randint(1, 20000)])
         if rows * width * P > 10_000_000:
             rows = max(1, 10_000_000 // (width * P))
         sp = width + rng.choice([0, 0, 1, 16, 100])
@@ -153,6 +154,8 @@ def test_gather_random_shapes_match_numpy(dev, knobs, seed):
         stride = rows * dp + rng.choice([0, 0, 5, 256])
         soff = [rng.randrange(0, 17) for _ in range(P)]
         doff = rng.randrange(0, 17)
+        if rng.random() < 0.3:  # everything on the 16-byte grid
+            soff, doff = [0] * P, 0
         g = torch.Generator().manual_seed(seed * 100000 + case)
         shards = [torch.randint(0, 255, (rows * sp + 32,), generator=g, dtype=torch.uint8) for _ in range(P)]
         d = [s.to(dev) for s in shards]
@@ -161,6 +164,7 @@ def test_gather_random_shapes_match_numpy(dev, knobs, seed):
             abi.set_tuning(k, rng.choice([0, 0, 1, 2, 4, 8]))
         abi.set_tuning("copy_max_blocks", rng.choice([0, 0, 1, 11]))
         abi.set_tuning("copy_wg_per_cu", rng.choice([0, 0, 2, 5, 9]))
+        abi.set_tuning("box_preload", rng.choice([0, 0, 0, 1]))
         abi.gather([d[s].data_ptr() + soff[s] for s in range(P)], out.data_ptr() + doff, width, rows, sp, dp, stride, st)
         torch.cuda.synchronize()
         want = np.full(P * stride + 64, 7, dtype=np.uint8)
