@@ -337,10 +337,13 @@ def main():
     # clocks, far longer than `warmup` launches of 25 us; keep launching until CLOCK_WARMUP_S of
     # wall time have passed.  These launches are not timed.
     clock_launches = 0
+    enqueue_us = []  # the host's launch call, per batch of 50: sizes the spin in front of a pre-filled window
     t_warm = time.perf_counter()
-    while time.perf_counter() - t_warm < args.clock_warmup:
+    while time.perf_counter() - t_warm < args.clock_warmup or not enqueue_us:
+        t_batch = time.perf_counter()
         for i in range(50):
             launch(clock_launches + i)
+        enqueue_us.append((time.perf_counter() - t_batch) * 1e6 / 50)
         clock_launches += 50
         torch.cuda.synchronize()
     # TIMED_WINDOWS windows of exactly `steps` launches each, every one bracketed by a
@@ -358,7 +361,9 @@ def main():
     # The work in front is a spin kernel that touches no memory (torch.cuda._sleep): a kernel
     # that streams through HBM would leave the caches full of its dirty lines, and writing those
     # back would be charged to the launches that follow.  Long enough to outlast the host's
-    # enqueuing of one window (up to 12 us per launch).
+    # enqueuing of one window: 12 us per launch, or three times what the launch call took during
+    # the clock warm-up when that is more (under a profiler it takes 10 us there and 25-65 us
+    # into a queue that is held up).
     def spin_ms(cycles):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
@@ -370,8 +375,8 @@ def main():
 
     spin_ms(100_000)
     cycles_per_ms = 4_000_000 / max(spin_ms(4_000_000), 1e-3)
-    spin_cycles = int(cycles_per_ms * (0.2 + args.steps * 12e-3))
-    desc["prefill_spin_ms"] = round(spin_cycles / cycles_per_ms, 3)
+    per_launch_ms = max(12e-3, 3e-3 * sorted(enqueue_us)[len(enqueue_us) // 2])
+    spin_cycles = int(cycles_per_ms * (0.2 + args.steps * per_launch_ms))
     done = 0
 
     def median(v):
@@ -379,9 +384,10 @@ def main():
         return v[len(v) // 2]
 
     def timed_windows(prefilled):
-        nonlocal done
+        nonlocal done, spin_cycles
         window_ms, enqueue_ms, wall_ms = [], [], []
-        for w in range(TIMED_WINDOWS):
+        lengthened = 0
+        while len(window_ms) < TIMED_WINDOWS:
             torch.cuda.synchronize()
             if prefilled:
                 torch.cuda._sleep(spin_cycles)
@@ -391,15 +397,24 @@ def main():
             e0.record()  # on torch's current stream, the stream every launch above and below uses
             for i in range(args.steps):
                 launch(done + i)
-            enqueue_ms.append((time.perf_counter() - t0) * 1e3)
+            enqueued = (time.perf_counter() - t0) * 1e3
             e1.record()
             torch.cuda.synchronize()
-            wall_ms.append((time.perf_counter() - t0) * 1e3)
-            window_ms.append(e0.elapsed_time(e1))
+            wall = (time.perf_counter() - t0) * 1e3
             done += args.steps
+            if prefilled and enqueued > 0.9 * spin_cycles / cycles_per_ms and lengthened < 6:
+                # the host was still enqueuing when the spin ended (a profiler slows the launch
+                # call several times over): this window measured the host; again behind a longer spin
+                spin_cycles = int(spin_cycles * 1.6)
+                lengthened += 1
+                continue
+            enqueue_ms.append(enqueued)
+            wall_ms.append(wall)
+            window_ms.append(e0.elapsed_time(e1))
         return window_ms, median(enqueue_ms), median(wall_ms)
 
     prefilled_ms, enqueue_ms, wall_ms = timed_windows(True)
+    desc["prefill_spin_ms"] = round(spin_cycles / cycles_per_ms, 3)
     kernel_ms = median(prefilled_ms) / args.steps
     desc["timed_windows"] = TIMED_WINDOWS
     if desc.get("queue_prefilled"):
