@@ -28,15 +28,15 @@ TIMED_WINDOWS = 11     # windows of `steps` launches; the median window is repor
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch), each
 # scaled by what the same counter reads for the flat copy of exactly 256 MiB (FETCH_SIZE x 1.99982,
 # WRITE_SIZE x 1.00000): profiles/hbm_traffic_pmc_reduce_and_copy_kernels.md.  E.g. the headline:
-# 65,552.31 x 1.99982 + 16,384.00 KiB = 147,477.1 KiB.  Workloads without an entry were not measured.
+# 65,552.29 x 1.99982 + 16,384.00 KiB = 147,476.6 KiB.  Workloads without an entry were not measured.
 MEASURED_TRAFFIC_BYTES = {
-    "reduce_fp32_p8": 151016523,
-    "reduce_bf16_p16": 1140857996,
-    "reduce_fp32_p64_sum": 272664628,
+    "reduce_fp32_p8": 151016081,
+    "reduce_bf16_p16": 1140854653,
+    "reduce_fp32_p64_sum": 272663625,
     "allgather_bf16_p8": 536870912,
-    "allgather_bf16_p8_strided": 536885292,
-    "redistribute_fp32_8192": 67146261,
-    "redistribute_bf16_3d": 16815972,
+    "allgather_bf16_p8_strided": 536884313,
+    "redistribute_fp32_8192": 67144034,
+    "redistribute_bf16_3d": 16799525,
 }
 
 def box_kernel(abi):
