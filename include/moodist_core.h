@@ -93,6 +93,14 @@ int moodist_pg_all_gather(moodist_pg* pg, const moodist_tensor* output, const mo
  * dense, of the input's dtype and size; n_outputs must equal the group size. */
 int moodist_pg_all_gather_list(moodist_pg* pg, const moodist_tensor* outputs, size_t n_outputs,
     const moodist_tensor* input, void* stream, moodist_work** work);
+/* c10d's allgather_into_tensor_coalesced (wrapper/processgroup_wrapper.cc:139-148), which the
+ * reference serves with one all_gather per tensor: here the n tensors are ONE collective --
+ * outputs[t] (group size times inputs[t]'s bytes) receives every rank's inputs[t] -- and its
+ * copies go out in as few launches as the segment table of the copy kernel allows.  Every
+ * rank must bring lists of the same length and sizes.  `outputs` may be NULL for a rank that
+ * only contributes. */
+int moodist_pg_all_gather_many(moodist_pg* pg, const moodist_tensor* outputs, const moodist_tensor* inputs, size_t n,
+    void* stream, moodist_work** work);
 /* processGroupReduceScatter (api/processgroup_api.h:45-46; core/processgroup.cc:1290-1668).
  * reduce_op is a c10d RedOpType number; premul_value is used by PREMUL_SUM only. */
 int moodist_pg_reduce_scatter(moodist_pg* pg, const moodist_tensor* output, const moodist_tensor* input,

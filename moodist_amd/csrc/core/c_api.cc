@@ -135,6 +135,16 @@ int moodist_pg_all_gather_list(moodist_pg* pg, const moodist_tensor* outputs, si
   });
 }
 
+int moodist_pg_all_gather_many(moodist_pg* pg, const moodist_tensor* outputs, const moodist_tensor* inputs, size_t n,
+    void* stream, moodist_work** work) {
+  return guarded([&] {
+    if (!inputs) {
+      throw std::runtime_error("moodist: null tensor");
+    }
+    give(work, as_pg(pg)->all_gather_many(outputs, inputs, n, stream));
+  });
+}
+
 int moodist_pg_reduce_scatter(moodist_pg* pg, const moodist_tensor* output, const moodist_tensor* input,
     int reduce_op, void* stream, float premul_value, moodist_work** work) {
   return guarded([&] {

@@ -259,6 +259,40 @@ std::shared_ptr<Collective> ProcessGroup::all_gather_list(const moodist_tensor* 
   return last = world->post(Kind::all_gather, next_seq++, rank, std::move(p), 0, 1.0f, bytes, input.dtype, 0, nullptr);
 }
 
+// allgather_into_tensor_coalesced (wrapper/processgroup_wrapper.cc:139-148).  The reference loops
+// over the tensors, one collective each; here the list is one collective, and its copies --
+// one contiguous segment per tensor and source rank -- go out in as few launches as the kernel's
+// segment table allows (64 segments each) instead of one launch per tensor.
+std::shared_ptr<Collective> ProcessGroup::all_gather_many(const moodist_tensor* outputs, const moodist_tensor* inputs,
+    size_t n, void* stream, Keep keep) {
+  Busy guard(*this);
+  if (n == 0 || n > 0xffffu) {
+    throw std::runtime_error("moodist: a coalesced all_gather takes 1..65535 tensors, not " + std::to_string(n));
+  }
+  Posting p;
+  size_t total = 0;
+  for (size_t t = 0; t < n; ++t) {
+    check_device_tensor(inputs[t], world->device, "all_gather input");
+    const size_t bytes = bytes_of(inputs[t]);
+    MD_CHECK(bytes > 0); // core/processgroup.cc:1078
+    moodist_tensor in = inputs[t];
+    snapshot(in, stream, keep);
+    p.inputs.push_back(in);
+    total += bytes;
+    if (outputs) {
+      check_device_tensor(outputs[t], world->device, "all_gather output");
+      MD_CHECK(bytes_of(outputs[t]) == bytes * (size_t)size); // :1079
+      p.outputs.push_back(outputs[t]);
+    }
+  }
+  p.wants_output = outputs != nullptr;
+  p.keep = std::move(keep);
+  p.stream = stream;
+  p.kernel_less = options.forceKernelLess || options.preferKernelLess;
+  return last = world->post(Kind::all_gather_many, next_seq++, rank, std::move(p), 0, 1.0f, total, inputs[0].dtype,
+             (uint32_t)n, nullptr);
+}
+
 std::shared_ptr<Collective> ProcessGroup::reduce_scatter(const moodist_tensor* output, const moodist_tensor& input,
     int reduce_op, void* stream, float premul, Keep keep) {
   Busy guard(*this);
@@ -687,6 +721,21 @@ void World::order_streams_after(Collective& c) {
 }
 
 void World::launch(Collective& c, const std::shared_ptr<CompiledOp>& op) {
+  if (c.kind == Kind::all_gather_many) {
+    // the ranks agreed on the number of tensors and their total size (post); now tensor by tensor
+    const size_t n = c.post[0].inputs.size();
+    for (int j = 0; j < size; ++j) {
+      const Posting& pj = c.post[(size_t)j];
+      bool same = pj.inputs.size() == n;
+      for (size_t t = 0; same && t < n; ++t) {
+        same = bytes_of(pj.inputs[t]) == bytes_of(c.post[0].inputs[t]);
+      }
+      if (!same) {
+        throw std::runtime_error("moodist: rank " + std::to_string(j) + " brought a different list of tensors to "
+                                 "collective #" + std::to_string(c.seq) + " than rank 0 did");
+      }
+    }
+  }
   const HipRuntime& h = hip();
   int current = -1;
   check_hip(h.GetDevice(&current), "hipGetDevice");
@@ -696,7 +745,10 @@ void World::launch(Collective& c, const std::shared_ptr<CompiledOp>& op) {
   order_streams_before(c);
   std::vector<const void*> srcs((size_t)size);
   log_debug("collective #%llu: launching %s for %d ranks, %zu bytes per rank, dtype %d", (unsigned long long)c.seq,
-      c.kind == Kind::reduce_scatter ? "reduce_scatter" : c.kind == Kind::all_gather ? "all_gather" : "custom op",
+      c.kind == Kind::reduce_scatter    ? "reduce_scatter"
+      : c.kind == Kind::all_gather      ? "all_gather"
+      : c.kind == Kind::all_gather_many ? "all_gather of a list"
+                                        : "custom op",
       size, c.bytes, c.dtype);
 
   if (c.kind == Kind::reduce_scatter) {
@@ -787,6 +839,42 @@ void World::launch(Collective& c, const std::shared_ptr<CompiledOp>& op) {
         check_hip(h.MemcpyAsync(back.data, pq.output.data, (size_t)back.numel * (size_t)back.itemsize,
                       kHipMemcpyDeviceToDevice, pq.stream),
             "hipMemcpyAsync");
+      }
+    }
+  } else if (c.kind == Kind::all_gather_many) {
+    // out_q[t][bytes_t*j .. +bytes_t] = in_j[t] for every tensor t and rank j: one table of
+    // contiguous copies per destination rank
+    const size_t n = c.post[0].inputs.size();
+    std::vector<mdh_box> boxes;
+    for (int q = 0; q < size; ++q) {
+      const Posting& pq = c.post[(size_t)q];
+      if (!pq.wants_output) {
+        continue;
+      }
+      boxes.clear();
+      boxes.reserve(n * (size_t)size);
+      for (size_t t = 0; t < n; ++t) {
+        const size_t bytes = bytes_of(pq.inputs[t]);
+        for (int j = 0; j < size; ++j) {
+          mdh_box b{};
+          b.src = c.post[(size_t)j].inputs[t].data;
+          b.dst = (char*)pq.outputs[t].data + bytes * (size_t)j;
+          if (b.src == b.dst) {
+            continue; // already in place
+          }
+          if (pq.kernel_less) { // the copy-engine form: one copy per tensor and source rank
+            check_hip(h.MemcpyAsync(b.dst, b.src, bytes, kHipMemcpyDeviceToDevice, pq.stream), "hipMemcpyAsync");
+            ++kernel_less_copies_1d;
+            continue;
+          }
+          b.ndim = 1;
+          b.shape[0] = (int64_t)bytes;
+          b.src_strides[0] = b.dst_strides[0] = 1;
+          boxes.push_back(b);
+        }
+      }
+      if (!boxes.empty()) {
+        check_mdh(h.copy_boxes(boxes.data(), (int)boxes.size(), 1, pq.stream));
       }
     }
   } else {

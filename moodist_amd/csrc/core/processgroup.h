@@ -22,7 +22,7 @@ namespace moodist {
 
 class World;
 
-enum class Kind : int { all_gather = 0, reduce_scatter = 1, custom = 2 };
+enum class Kind : int { all_gather = 0, reduce_scatter = 1, custom = 2, all_gather_many = 3 };
 
 // What one rank brought to a collective.
 struct Posting {
@@ -30,8 +30,8 @@ struct Posting {
   bool wants_output = false;
   moodist_tensor input{};
   moodist_tensor output{};
-  std::vector<moodist_tensor> inputs;  // custom op
-  std::vector<moodist_tensor> outputs; // custom op; all_gather into one tensor per rank
+  std::vector<moodist_tensor> inputs;  // custom op; all_gather of a list of tensors
+  std::vector<moodist_tensor> outputs; // custom op; all_gather into one tensor per rank, or of a list of tensors
   bool kernel_less = false;   // this rank asked for the copy-engine form of all_gather
   bool has_copy_back = false; // allreduce through a padded temporary
   moodist_tensor copy_back{};
@@ -109,6 +109,10 @@ public:
       Keep keep = {});
   std::shared_ptr<Collective> all_gather_list(const moodist_tensor* outputs, size_t n_outputs,
       const moodist_tensor& input, void* stream, Keep keep = {});
+  // n all_gathers as one collective: outputs[t] receives every rank's inputs[t] (outputs may be
+  // null for a rank that only contributes)
+  std::shared_ptr<Collective> all_gather_many(const moodist_tensor* outputs, const moodist_tensor* inputs, size_t n,
+      void* stream, Keep keep = {});
   std::shared_ptr<Collective> reduce_scatter(const moodist_tensor* output, const moodist_tensor& input, int reduce_op,
       void* stream, float premul, Keep keep = {});
   std::shared_ptr<Collective> allreduce(const moodist_tensor& tensor, const moodist_tensor* scratch, int reduce_op,

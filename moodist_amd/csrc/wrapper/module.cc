@@ -62,6 +62,7 @@ struct CoreExtras {
   MOODIST_EXTRA(moodistOpCHandle)
   MOODIST_EXTRA(moodist_last_error)
   MOODIST_EXTRA(moodist_pg_all_gather_list)
+  MOODIST_EXTRA(moodist_pg_all_gather_many)
   MOODIST_EXTRA(moodist_pg_stage_input)
   MOODIST_EXTRA(moodist_pg_last_work)
   MOODIST_EXTRA(moodist_pg_keep_alive)
@@ -232,6 +233,7 @@ void load_core() {
   MOODIST_EXTRA(moodistOpCHandle)
   MOODIST_EXTRA(moodist_last_error)
   MOODIST_EXTRA(moodist_pg_all_gather_list)
+  MOODIST_EXTRA(moodist_pg_all_gather_many)
   MOODIST_EXTRA(moodist_pg_stage_input)
   MOODIST_EXTRA(moodist_pg_last_work)
   MOODIST_EXTRA(moodist_pg_keep_alive)
@@ -404,16 +406,33 @@ public:
     return work({output});
   }
 
-  // wrapper/processgroup_wrapper.cc:139-148
+  // wrapper/processgroup_wrapper.cc:139-148 loops over the tensors; here a list of two or more
+  // is one collective whose copies share launches (moodist_pg_all_gather_many)
   c10::intrusive_ptr<c10d::Work> allgather_into_tensor_coalesced(std::vector<at::Tensor>& outputs,
       std::vector<at::Tensor>& inputs, const c10d::AllgatherOptions& = c10d::AllgatherOptions()) override {
     TORCH_CHECK(outputs.size() == inputs.size());
     auto result = c10::make_intrusive<WorkImpl>();
-    for (size_t k = 0; k < inputs.size(); ++k) {
-      Wrapped o(outputs[k]), i(inputs[k]);
-      core->processGroupAllGather(handle_.get(), o.ptr, i.ptr, stream_of(inputs[k]));
-      add_last(*result);
+    if (inputs.size() < 2) {
+      for (size_t k = 0; k < inputs.size(); ++k) {
+        Wrapped o(outputs[k]), i(inputs[k]);
+        core->processGroupAllGather(handle_.get(), o.ptr, i.ptr, stream_of(inputs[k]));
+        add_last(*result);
+      }
+      result->tensors = outputs;
+      return result;
     }
+    std::vector<moodist_tensor> outs, ins;
+    for (size_t k = 0; k < inputs.size(); ++k) {
+      outs.push_back(describe(outputs[k]));
+      ins.push_back(describe(inputs[k]));
+    }
+    moodist_work* w = nullptr;
+    check(extra.moodist_pg_all_gather_many(c_, outs.data(), ins.data(), ins.size(), stream_of(inputs[0]), &w));
+    result->parts.push_back(w);
+    auto held = new std::vector<at::Tensor>(outputs);
+    held->insert(held->end(), inputs.begin(), inputs.end());
+    // the core owns `held` from the call on and releases it exactly once, also when it fails
+    check(extra.moodist_pg_keep_alive(c_, held, release_tensors));
     result->tensors = outputs;
     return result;
   }

@@ -46,6 +46,8 @@ def core():
                                         ctypes.c_void_p]
     L.moodist_pg_all_gather_list.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p,
                                              ctypes.c_void_p, ctypes.c_void_p]
+    L.moodist_pg_all_gather_many.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
+                                             ctypes.c_void_p, ctypes.c_void_p]
     L.moodist_pg_allreduce.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
                                        ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p]
     L.moodist_work_wait.argtypes = [ctypes.c_void_p]
@@ -141,6 +143,42 @@ def test_argument_checks_use_the_reference_messages(core):
     four[2] = fake(4, contiguous=0)
     assert core.moodist_pg_all_gather_list(pg, four, 4, ctypes.byref(fake(4)), None, ctypes.byref(work)) != 0
     assert b"must be contiguous" in core.moodist_last_error()
+    # a list of all_gathers as one collective: outputs[t] is group size times inputs[t]
+    T = type(fake(4))
+    ins = (T * 2)(fake(4), fake(6))
+    outs = (T * 2)(fake(16), fake(24))
+    assert core.moodist_pg_all_gather_many(pg, outs, ins, 0, None, ctypes.byref(work)) != 0
+    assert b"1..65535 tensors" in core.moodist_last_error()
+    assert core.moodist_pg_all_gather_many(pg, outs, None, 2, None, ctypes.byref(work)) != 0
+    outs[1] = fake(23)
+    assert core.moodist_pg_all_gather_many(pg, outs, ins, 2, None, ctypes.byref(work)) != 0
+    outs[1] = fake(24, contiguous=0)
+    assert core.moodist_pg_all_gather_many(pg, outs, ins, 2, None, ctypes.byref(work)) != 0
+    assert b"must be contiguous" in core.moodist_last_error()
+    ins[0] = fake(4, device=-1)
+    assert core.moodist_pg_all_gather_many(pg, None, ins, 2, None, ctypes.byref(work)) != 0
+    assert b"no CPU fallback" in core.moodist_last_error()
+    core.moodist_world_destroy(w)
+
+
+def test_a_list_of_all_gathers_must_be_the_same_list_on_every_rank(core):
+    # lists of different lengths are different collectives (caught when the second rank posts);
+    # lists of the same length and total size but other tensor sizes are caught before the launch
+    T = type(fake(4))
+    w = make_world(core, 2)
+    work = ctypes.c_void_p()
+    a, b = core.moodist_world_group(w, 0), core.moodist_world_group(w, 1)
+    assert core.moodist_pg_all_gather_many(a, None, (T * 2)(fake(4), fake(6)), 2, None, ctypes.byref(work)) == 0
+    core.moodist_work_destroy(work)
+    assert core.moodist_pg_all_gather_many(b, None, (T * 1)(fake(10)), 1, None, ctypes.byref(work)) != 0
+    assert b"different operation, size, dtype or reduction" in core.moodist_last_error()
+    core.moodist_world_destroy(w)
+    w = make_world(core, 2)
+    a, b = core.moodist_world_group(w, 0), core.moodist_world_group(w, 1)
+    assert core.moodist_pg_all_gather_many(a, None, (T * 2)(fake(4), fake(6)), 2, None, ctypes.byref(work)) == 0
+    core.moodist_work_destroy(work)
+    assert core.moodist_pg_all_gather_many(b, None, (T * 2)(fake(5), fake(5)), 2, None, ctypes.byref(work)) != 0
+    assert b"a different list of tensors" in core.moodist_last_error()
     core.moodist_world_destroy(w)
 
 

@@ -231,6 +231,34 @@ def test_coalesced_variants(world, dev):
 
 
 @pytest.mark.parametrize("kernel_less", [False, True])
+def test_allgather_coalesced_many_tensors_of_awkward_sizes_and_types(world, dev, kernel_less):
+    # a list of tensors is ONE collective whose copies share launches (the reference loops,
+    # wrapper/processgroup_wrapper.cc:139-148): 40 tensors, sizes with and without whole vectors,
+    # three element types, one tensor already in place in its rank's output
+    for pg in world:
+        pg.options().force_kernel_less = kernel_less
+    try:
+        g = torch.Generator().manual_seed(4)
+        sizes = [1, 2, 3, 7, 8, 15, 16, 17, 31, 64, 100, 255, 1000, 1023, 4096, 4099, 65536, 70001, 5, 9] * 2
+        dtypes = [torch.float32, torch.bfloat16, torch.int64]
+        ins = [[(torch.randn(n, generator=g) * 100).to(dtypes[k % 3]).to(dev) for k, n in enumerate(sizes)]
+               for r in range(P)]
+        outs = [[torch.zeros(n * P, dtype=dtypes[k % 3], device=dev) for k, n in enumerate(sizes)] for _ in range(P)]
+        for r in range(P):  # tensor 14 of every rank already sits in its slot of that rank's output
+            outs[r][14][r * sizes[14]:(r + 1) * sizes[14]] = ins[r][14]
+            ins[r][14] = outs[r][14][r * sizes[14]:(r + 1) * sizes[14]]
+        each_rank(world, lambda r, pg: pg.allgather_into_tensor_coalesced(outs[r], ins[r]))
+        torch.cuda.synchronize()
+        for k in range(len(sizes)):
+            want = torch.cat([ins[j][k] for j in range(P)])
+            for r in range(P):
+                assert torch.equal(outs[r][k], want), (k, sizes[k], r)
+    finally:
+        for pg in world:
+            pg.options().force_kernel_less = False
+
+
+@pytest.mark.parametrize("kernel_less", [False, True])
 def test_allgather_into_a_list_of_tensors(world, dev, kernel_less):
     # c10d's list form (reference wrapper/processgroup_wrapper.cc:112-129): outputs[j] = rank j's input.
     # Sizes with and without a 16-byte body and tail; one output is the rank's own input (in place).
