@@ -511,11 +511,21 @@ def test_snapshot_inputs_with_allreduce_and_allgather(world, dev):
         pg.allreduce([ev[r]])
         pg._allgather_base(outs[r], ins[r])
         ins[r].fill_(-1.0)  # after the call: must not be seen
+    # a coalesced list is snapshotted tensor by tensor
+    cins = [[torch.full((k + 5,), float(10 * r + k), device=dev) for k in range(3)] for r in range(P)]
+    couts = [[torch.zeros(P * (k + 5), device=dev) for k in range(3)] for _ in range(P)]
+    for r, pg in enumerate(world):
+        pg.allgather_into_tensor_coalesced(couts[r], cins[r])
+        for t in cins[r]:
+            t.fill_(-1.0)
     torch.cuda.synchronize()
     for r in range(P):
         assert torch.equal(ts[r], torch.full((n,), P * (P + 1) / 2, device=dev))
         assert torch.equal(ev[r], torch.full((P * 64,), P * (P + 1) / 2, device=dev))
         assert torch.equal(outs[r], torch.arange(P, device=dev, dtype=torch.float32).repeat_interleave(100))
+        for k in range(3):
+            want = torch.cat([torch.full((k + 5,), float(10 * j + k), device=dev) for j in range(P)])
+            assert torch.equal(couts[r][k], want), (r, k)
 
 
 def test_kernel_less_gather_from_padded_staging_equals_the_kernel_path(world, dev):
