@@ -24,6 +24,24 @@ int main() {
       if (wk) works.push_back(wk);
     }
     for (auto* wk : works) { int rc = moodist_work_wait(wk); if (rc) std::printf("wait: %s\n", moodist_last_error()); std::printf("completed %d\n", moodist_work_is_completed(wk)); }
+    // a list of all_gathers as one collective: left incomplete in round 0, launched (and failing
+    // for want of a device) otherwise; a rank that brings another list; things kept alive for it
+    {
+      std::vector<moodist_work*> many;
+      static int released = 0;
+      for (int r = 0; r < (round == 0 ? 2 : 4); ++r) {
+        moodist_pg* pg = moodist_world_group(w, r);
+        moodist_tensor ins[3] = {fake(4), fake(6), fake(r == 3 && round == 2 ? 9 : 10)};
+        moodist_tensor outs[3] = {fake(16), fake(24), fake(r == 3 && round == 2 ? 36 : 40)};
+        moodist_work* wk = nullptr;
+        int rc = moodist_pg_all_gather_many(pg, r % 2 ? outs : nullptr, ins, 3, nullptr, &wk);
+        if (rc) std::printf("round %d rank %d many: %s\n", round, r, moodist_last_error());
+        if (wk) many.push_back(wk);
+        moodist_pg_keep_alive(pg, new int(r), [](void* p) { delete (int*)p; ++released; });
+      }
+      for (auto* wk : many) { moodist_work_wait(wk); moodist_work_destroy(wk); }
+      std::printf("round %d: %d kept objects released so far\n", round, released);
+    }
     // compile + plan accessors
     int shape[1] = {8};
     int in_ranks[1] = {0}, in_off[1] = {0}, in_shape[1] = {8};
