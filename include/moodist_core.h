@@ -112,6 +112,14 @@ int moodist_pg_reduce_scatter(moodist_pg* pg, const moodist_tensor* output, cons
  * elements, same dtype), or NULL when numel divides evenly. */
 int moodist_pg_allreduce(moodist_pg* pg, const moodist_tensor* tensor, const moodist_tensor* scratch, int reduce_op,
     void* stream, float premul_value, moodist_work** work);
+/* c10d's allreduce_coalesced (wrapper/processgroup_wrapper.cc:182-191), which the reference serves
+ * with one allreduce per tensor, for tensors whose element counts the group size divides (the
+ * others go through moodist_pg_allreduce one by one): a reduce_scatter per tensor into the
+ * rank's own chunk, in place, then ONE all_gather of every tensor's chunks
+ * (moodist_pg_all_gather_many).  `*work` is the last collective; the earlier ones have been
+ * launched when it has. */
+int moodist_pg_allreduce_many(moodist_pg* pg, const moodist_tensor* tensors, size_t n, int reduce_op, void* stream,
+    float premul_value, moodist_work** work);
 /* No counterpart in the reference.  moodist_pg_allreduce for callers that cannot allocate
  * device memory and have no temporary to pass (code under stream capture, tight serving
  * loops, harnesses that forbid hipMalloc): the padded temporary is this rank's slice of the

@@ -378,6 +378,40 @@ std::shared_ptr<Collective> ProcessGroup::allreduce(const moodist_tensor& tensor
   return all_gather_impl(&whole, chunk, stream, &tensor, std::move(keep));
 }
 
+// allreduce_coalesced (wrapper/processgroup_wrapper.cc:182-191), for the tensors of the list that
+// need no padding: the reference runs one allreduce -- a reduce_scatter and an all_gather -- per
+// tensor; here the reductions are followed by one gather of every tensor's chunks.
+std::shared_ptr<Collective> ProcessGroup::allreduce_many(const moodist_tensor* tensors, size_t n, int reduce_op,
+    void* stream, float premul, Keep keep) {
+  if (n == 0 || n > 0xffffu) {
+    throw std::runtime_error("moodist: a coalesced allreduce takes 1..65535 tensors, not " + std::to_string(n));
+  }
+  std::vector<moodist_tensor> chunks(n);
+  for (size_t t = 0; t < n; ++t) {
+    check_device_tensor(tensors[t], world->device, "allreduce tensor");
+    MD_CHECK(tensors[t].numel > 0 && tensors[t].numel % size == 0);
+    check_reduce_dtype(tensors[t].dtype); // before anything of the list is posted
+  }
+  for (size_t t = 0; t < n; ++t) {
+    moodist_tensor& chunk = chunks[t];
+    chunk = tensors[t];
+    chunk.numel = tensors[t].numel / size;
+    chunk.data = (char*)tensors[t].data + (size_t)rank * (size_t)chunk.numel * (size_t)tensors[t].itemsize;
+    chunk.ndim = 1;
+    chunk.shape[0] = chunk.numel;
+    reduce_scatter(&chunk, tensors[t], reduce_op, stream, premul, keep);
+  }
+  // the gather's inputs are what the reductions will have written by then: never snapshots
+  internal_input = true;
+  struct Reset {
+    bool& flag;
+    ~Reset() {
+      flag = false;
+    }
+  } reset{internal_input};
+  return all_gather_many(tensors, chunks.data(), n, stream, std::move(keep));
+}
+
 std::shared_ptr<Collective> ProcessGroup::allreduce_static(const moodist_tensor& tensor, int reduce_op, void* stream,
     float premul, Keep keep) {
   check_device_tensor(tensor, world->device, "allreduce tensor");

@@ -117,6 +117,10 @@ public:
       void* stream, float premul, Keep keep = {});
   std::shared_ptr<Collective> allreduce(const moodist_tensor& tensor, const moodist_tensor* scratch, int reduce_op,
       void* stream, float premul, Keep keep = {});
+  // n in-place allreduces whose element counts the group size divides: one reduce_scatter each,
+  // then ONE gather of all the chunks
+  std::shared_ptr<Collective> allreduce_many(const moodist_tensor* tensors, size_t n, int reduce_op, void* stream,
+      float premul, Keep keep = {});
   // allreduce whose padded temporary is this rank's slice of the kernel library's fixed
   // workspace (mdh_static_workspace) instead of a tensor from the caller
   std::shared_ptr<Collective> allreduce_static(const moodist_tensor& tensor, int reduce_op, void* stream, float premul,

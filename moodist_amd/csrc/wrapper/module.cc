@@ -63,6 +63,7 @@ struct CoreExtras {
   MOODIST_EXTRA(moodist_last_error)
   MOODIST_EXTRA(moodist_pg_all_gather_list)
   MOODIST_EXTRA(moodist_pg_all_gather_many)
+  MOODIST_EXTRA(moodist_pg_allreduce_many)
   MOODIST_EXTRA(moodist_pg_stage_input)
   MOODIST_EXTRA(moodist_pg_last_work)
   MOODIST_EXTRA(moodist_pg_keep_alive)
@@ -234,6 +235,7 @@ void load_core() {
   MOODIST_EXTRA(moodist_last_error)
   MOODIST_EXTRA(moodist_pg_all_gather_list)
   MOODIST_EXTRA(moodist_pg_all_gather_many)
+  MOODIST_EXTRA(moodist_pg_allreduce_many)
   MOODIST_EXTRA(moodist_pg_stage_input)
   MOODIST_EXTRA(moodist_pg_last_work)
   MOODIST_EXTRA(moodist_pg_keep_alive)
@@ -467,8 +469,40 @@ public:
   c10::intrusive_ptr<c10d::Work> allreduce_coalesced(std::vector<at::Tensor>& tensors,
       const c10d::AllreduceCoalescedOptions& opts = c10d::AllreduceCoalescedOptions()) override {
     auto result = c10::make_intrusive<WorkImpl>();
+    // The tensors that need no padded temporary -- same element type, element count a multiple
+    // of the group size -- are reduced one by one and gathered together
+    // (moodist_pg_allreduce_many); the others take one allreduce each, as in the reference.
+    // Every rank holds the same list, so every rank splits it the same way.
+    std::vector<at::Tensor> together;
     for (at::Tensor& t : tensors) {
-      allreduce_one(t, opts.reduceOp, *result);
+      if (t.is_cuda() && t.is_contiguous() && t.numel() > 0 && t.numel() % getSize() == 0 &&
+          (together.empty() || t.scalar_type() == together[0].scalar_type())) {
+        together.push_back(t);
+      }
+    }
+    if (together.size() < 2) {
+      together.clear();
+    }
+    if (!together.empty()) {
+      std::vector<moodist_tensor> descs;
+      for (at::Tensor& t : together) {
+        descs.push_back(describe(t));
+      }
+      moodist_work* w = nullptr;
+      check(extra.moodist_pg_allreduce_many(c_, descs.data(), descs.size(), static_cast<int>(reduce_op_code(opts.reduceOp)),
+          stream_of(together[0]), premul_value(opts.reduceOp, together[0].scalar_type()), &w));
+      result->parts.push_back(w);
+      // the core owns the list from the call on and releases it exactly once, also when it fails
+      check(extra.moodist_pg_keep_alive(c_, new std::vector<at::Tensor>(together), release_tensors));
+    }
+    for (at::Tensor& t : tensors) {
+      bool done = false;
+      for (const at::Tensor& u : together) {
+        done = done || u.is_same(t);
+      }
+      if (!done) {
+        allreduce_one(t, opts.reduceOp, *result);
+      }
     }
     result->tensors = tensors;
     return result;

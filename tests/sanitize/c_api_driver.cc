@@ -39,6 +39,13 @@ int main() {
         if (wk) many.push_back(wk);
         moodist_pg_keep_alive(pg, new int(r), [](void* p) { delete (int*)p; ++released; });
       }
+      for (int r = 0; r < (round == 0 ? 1 : 4); ++r) {
+        moodist_tensor ts[2] = {fake(16), fake(r == 2 && round == 1 ? 25 : 24)};
+        moodist_work* wk = nullptr;
+        int rc = moodist_pg_allreduce_many(moodist_world_group(w, r), ts, 2, 0, nullptr, 0.0f, &wk);
+        if (rc) std::printf("round %d rank %d allreduce list: %s\n", round, r, moodist_last_error());
+        if (wk) many.push_back(wk);
+      }
       for (auto* wk : many) { moodist_work_wait(wk); moodist_work_destroy(wk); }
       std::printf("round %d: %d kept objects released so far\n", round, released);
     }

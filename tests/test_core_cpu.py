@@ -48,6 +48,8 @@ def core():
                                              ctypes.c_void_p, ctypes.c_void_p]
     L.moodist_pg_all_gather_many.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
                                              ctypes.c_void_p, ctypes.c_void_p]
+    L.moodist_pg_allreduce_many.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int,
+                                            ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p]
     L.moodist_pg_allreduce.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
                                        ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p]
     L.moodist_work_wait.argtypes = [ctypes.c_void_p]
@@ -158,6 +160,19 @@ def test_argument_checks_use_the_reference_messages(core):
     ins[0] = fake(4, device=-1)
     assert core.moodist_pg_all_gather_many(pg, None, ins, 2, None, ctypes.byref(work)) != 0
     assert b"no CPU fallback" in core.moodist_last_error()
+    # a list of allreduces: every element count a multiple of the group size, a reduce dtype;
+    # nothing of the list is posted when one tensor is refused
+    ts = (T * 2)(fake(16), fake(24))
+    assert core.moodist_pg_allreduce_many(pg, ts, 0, 0, None, 0.0, ctypes.byref(work)) != 0
+    assert core.moodist_pg_allreduce_many(pg, None, 2, 0, None, 0.0, ctypes.byref(work)) != 0
+    ts[1] = fake(25)
+    assert core.moodist_pg_allreduce_many(pg, ts, 2, 0, None, 0.0, ctypes.byref(work)) != 0
+    ts[1] = fake(24, dtype=0, itemsize=1)
+    assert core.moodist_pg_allreduce_many(pg, ts, 2, 0, None, 0.0, ctypes.byref(work)) != 0
+    assert core.moodist_last_error() == b"Unsupported dtype for reduce operation"
+    ok = (T * 2)(fake(16), fake(24))
+    assert core.moodist_pg_allreduce_many(pg, ok, 2, 0, None, 0.0, ctypes.byref(work)) == 0  # first rank of four: posted
+    core.moodist_work_destroy(work)
     core.moodist_world_destroy(w)
 
 

@@ -296,6 +296,41 @@ def test_allreduce_coalesced(world, dev):
             assert torch.equal(ts[r][k], torch.arange(n, device=dev, dtype=torch.float32) * 36.0)
 
 
+@pytest.mark.parametrize("snapshot", [False, True])
+def test_allreduce_coalesced_divisible_tensors_share_one_gather(world, dev, snapshot):
+    # tensors whose sizes divide by the group size are reduced one by one and gathered together
+    # (moodist_pg_allreduce_many); the others, and a tensor of another element type, take one
+    # allreduce each.  Random values against the oracle's composition: chunk q of a tensor is
+    # folded starting at rank q (reference core/processgroup.cc:1674-1722).
+    for pg in world:
+        pg.options().snapshot_inputs = snapshot
+    g = torch.Generator().manual_seed(9)
+    sizes = [8, 16, 1001, 4096, 8 * 1000, 24, 7, 65536, 8 * 12345, 40]
+    dtypes = [torch.float32] * 9 + [torch.bfloat16]
+    for name, code, op in (("SUM", oracle.OP_SUM, dist.ReduceOp.SUM), ("MAX", oracle.OP_MAX, dist.ReduceOp.MAX),
+                           ("AVG", oracle.OP_AVG, dist.ReduceOp.AVG)):
+        host = [[(torch.randn(n, generator=g) * 3).to(dt) for n, dt in zip(sizes, dtypes)] for _ in range(P)]
+        ts = [[t.to(dev) for t in row] for row in host]
+        opts = dist.AllreduceCoalescedOptions()
+        opts.reduceOp = op
+        works = []
+        for r, pg in enumerate(world):
+            works.append(pg.allreduce_coalesced(ts[r], opts))
+        for w in works:
+            w.wait()
+        torch.cuda.synchronize()
+        for k, (n, dt) in enumerate(zip(sizes, dtypes)):
+            padded = (n + P - 1) // P * P
+            c = padded // P
+            pin = [torch.cat([host[r][k], torch.zeros(padded - n, dtype=dt)]) for r in range(P)]
+            want = np.concatenate([oracle.reduce([bits(t[q * c:(q + 1) * c]) for t in pin], q, TORCH_TO_CODE[dt], code,
+                                                 1.0 / P if code == oracle.OP_AVG else 1.0) for q in range(P)])[:n]
+            for r in range(P):
+                assert same_bits(bits(ts[r][k]), want), (name, k, n, r)
+    for pg in world:
+        pg.options().snapshot_inputs = False
+
+
 def test_ranks_on_different_streams(world, dev):
     # each rank posts on its own stream; the launches must still see every rank's input
     n = 1 << 20
