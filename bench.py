@@ -7,9 +7,17 @@ before the timed region; the launches rotate over 4 GiB of distinct buffers, so 
 not in the 256 MB Infinity Cache either.  Prints one JSON line.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
-                  [--tuning KNOB=VALUE ...]
-  NAME is one of the fixed workloads (the headline reduce_fp32_p8 by default) or, for size sweeps,
-  reduce:<fp32|bf16|fp16>:<sources>:<elements>[:<sum|avg|max>] and gather:<sources>:<bytes per shard>.
+                  [--headline-only] [--tuning KNOB=VALUE ...]
+  Without --workload the headline (reduce_fp32_p8) is measured and reported as the line's top-level
+  figures, and after it, in the same process, every other configuration of the benchmark --
+  reduce_bf16_p16, reduce_fp32_p64_{sum,avg,max}, allgather_bf16_p8[_strided],
+  redistribute_{fp32,bf16}_8192, redistribute_bf16_3d -- each with the same steps, warm-up, rotation
+  and result check; their kernel times go into "configs" of the same JSON line.
+  NAME is one of those or, for sweeps,
+    reduce:<fp32|bf16|fp16|fp64|int32|int64>:<sources>:<elements>[:<sum|avg|max>]
+    gather:<sources>:<bytes per shard>
+    rows:<boxes>:<rows per box>:<run bytes>:<source pitch bytes>    strided rows into a dense destination
+    transpose:<rows>:<cols>:<itemsize>                              2-D element transpose
 """
 
 import argparse
@@ -38,6 +46,15 @@ MEASURED_TRAFFIC_BYTES = {
     "redistribute_fp32_8192": 67144034,
     "redistribute_bf16_3d": 16799525,
 }
+
+DTYPE_NAMES = {"float32": "f32", "bfloat16": "bf16", "float16": "f16", "float64": "f64", "int32": "i32", "int64": "i64",
+               "uint8": "u8"}
+
+# every configuration of the benchmark; the first is the headline
+ALL_WORKLOADS = ("reduce_fp32_p8", "reduce_bf16_p16", "reduce_fp32_p64_sum", "reduce_fp32_p64_avg", "reduce_fp32_p64_max",
+                 "allgather_bf16_p8", "allgather_bf16_p8_strided", "redistribute_fp32_8192", "redistribute_bf16_8192",
+                 "redistribute_bf16_3d")
+
 
 def box_kernel(abi):
     """The strided-box kernel the benchmark's shapes run: equal boxes of full tiles are started from
@@ -86,7 +103,8 @@ def build_workload(name, torch, abi, dev, rotation_bytes):
             if parts[0] != "reduce" or len(parts) not in (4, 5):
                 raise SystemExit("bench.py: unknown workload " + name)
             tdt, code = {"fp32": (torch.float32, abi.DTYPE_FLOAT32), "bf16": (torch.bfloat16, abi.DTYPE_BFLOAT16),
-                         "fp16": (torch.float16, abi.DTYPE_FLOAT16)}[parts[1]]
+                         "fp16": (torch.float16, abi.DTYPE_FLOAT16), "fp64": (torch.float64, abi.DTYPE_FLOAT64),
+                         "int32": (torch.int32, abi.DTYPE_INT32), "int64": (torch.int64, abi.DTYPE_INT64)}[parts[1]]
             P, N = int(parts[2]), int(parts[3])
             op = {"sum": abi.OP_SUM, "avg": abi.OP_AVG, "max": abi.OP_MAX}[parts[4] if len(parts) == 5 else "sum"]
             spec = (P, N, tdt, code, op, "rand", 1.0 / P if op == abi.OP_AVG else 1.0)
@@ -101,8 +119,10 @@ def build_workload(name, torch, abi, dev, rotation_bytes):
                 x = torch.randn(N)  # first N draws of rank r's 8*N-element input = its chunk for rank 0
             elif dist == "randn1e-3":
                 x = (torch.randn(N) * 1e-3).to(tdt)
-            else:
+            elif tdt.is_floating_point:
                 x = (torch.rand(N) * 2 - 1).to(tdt)
+            else:
+                x = torch.randint(-2 ** 30, 2 ** 30, (N,)).to(tdt)
             base.append(x)
         on_device = [b.to(dev) for b in base]
         sets = [on_device] + [[b.clone() for b in on_device] for _ in range(nsets - 1)]
@@ -251,6 +271,72 @@ def build_workload(name, torch, abi, dev, rotation_bytes):
                 "queue_prefilled": True}
         return desc, set_bytes, launch, check, box_kernel(abi)
 
+    if name.startswith("rows:"):
+        # rows:<boxes>:<rows per box>:<run bytes>:<source pitch bytes> -- every box is `rows` runs of
+        # `run` bytes, `pitch` bytes apart in its source, packed densely into the destination: the
+        # shape of a last-dimension shard (run = row bytes / ranks) at any run length
+        P, rows, run, pitch = (int(x) for x in name.split(":")[1:5])
+        if run > pitch or run < 1:
+            raise SystemExit("bench.py: rows: the run must fit the pitch")
+        isz = 1
+        while isz < 16 and run % (isz * 2) == 0 and pitch % (isz * 2) == 0:
+            isz *= 2
+        set_bytes = 2 * P * rows * run
+        nsets = nsets_for(set_bytes)
+        g = torch.Generator().manual_seed(2)
+        # only the runs are read, so only they need distinct memory per set; the slabs are whole
+        base = [torch.randint(0, 256, (rows, pitch), dtype=torch.uint8, generator=g) for _ in range(P)]
+        on_device = [b.to(dev) for b in base]
+        sets = [on_device] + [[t.clone() for t in on_device] for _ in range(nsets - 1)]
+        outs = [torch.empty(P * rows * run, dtype=torch.uint8, device=dev) for _ in range(nsets)]
+        plan = abi.CopyPlan([abi.make_box(0, s_ * rows * run, [rows, run // isz], [pitch // isz, 1], [run // isz, 1])
+                             for s_ in range(P)], list(range(P)), [P] * P, isz, P + 1)
+        tabs = [abi.ptr_table([t.data_ptr() for t in sets[i]] + [outs[i].data_ptr()]) for i in range(nsets)]
+
+        def launch(i):
+            rc = L.mdh_copy_plan_launch(plan._plan, tabs[i % nsets], P + 1, current())
+            if rc:
+                abi.check(rc)
+
+        def check():
+            want = torch.cat([b[:, :run].reshape(-1) for b in base])
+            for o in outs:
+                if not torch.equal(o.cpu(), want):
+                    raise SystemExit("bench: result differs from the expected rows")
+
+        desc = {"workload": name, "op": "strided rows into a dense destination (prepared plan)", "sources": P,
+                "rows": rows, "run_bytes": run, "source_pitch_bytes": pitch, "vector_bytes": isz, "dtype": "uint8",
+                "buffer_sets": nsets, "queue_prefilled": True, "launches_per_step": plan.launches}
+        return desc, set_bytes, launch, check, "strided-box kernels"
+
+    if name.startswith("transpose:"):
+        # transpose:<rows>:<cols>:<itemsize> -- out[c, r] = in[r, c], both dense: through mdh_copy_boxes
+        R, C, isz = (int(x) for x in name.split(":")[1:4])
+        tdt = {1: torch.uint8, 2: torch.int16, 4: torch.int32, 8: torch.int64}[isz]
+        set_bytes = 2 * R * C * isz
+        nsets = nsets_for(set_bytes)
+        g = torch.Generator().manual_seed(3)
+        base = torch.randint(0, 127, (R, C), dtype=tdt, generator=g)
+        ins = [base.to(dev) for _ in range(nsets)]
+        outs = [torch.empty(C, R, dtype=tdt, device=dev) for _ in range(nsets)]
+        boxes = [(abi.Box * 1)(abi.make_box(ins[k].data_ptr(), outs[k].data_ptr(), [C, R], [1, C], [R, 1]))
+                 for k in range(nsets)]
+
+        def launch(i):
+            rc = L.mdh_copy_boxes(boxes[i % nsets], 1, isz, current())
+            if rc:
+                abi.check(rc)
+
+        def check():
+            want = base.t().contiguous()
+            for o in outs:
+                if not torch.equal(o.cpu(), want):
+                    raise SystemExit("bench: result differs from the expected transpose")
+
+        desc = {"workload": name, "op": "2-D element transpose (mdh_copy_boxes)", "rows": R, "cols": C, "itemsize": isz,
+                "dtype": "uint8", "buffer_sets": nsets}
+        return desc, set_bytes, launch, check, "strided-box kernels"
+
     raise SystemExit("bench: unknown workload %r" % name)
 
 
@@ -295,37 +381,10 @@ def cpu_baseline(seconds_budget=12.0):
     }
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=400)
-    ap.add_argument("--warmup", type=int, default=50)
-    ap.add_argument("--workload", default="reduce_fp32_p8")
-    ap.add_argument("--rotation-mib", type=int, default=4096,
-                    help="touched bytes of all buffer sets together (the launches rotate over them)")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-check", action="store_true")
-    ap.add_argument("--clock-warmup", type=float, default=CLOCK_WARMUP_S, metavar="SECONDS",
-                    help="untimed launches before the first timed window (0 under a counter-collecting profiler)")
-    ap.add_argument("--tuning", action="append", default=[], metavar="KNOB=VALUE",
-                    help="force a launch-shape knob of the kernel library (mdh_set_tuning), e.g. reduce_unroll=8")
-    args = ap.parse_args()
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        raise SystemExit("bench.py measures one GPU: the path is one rank's share with its peers staged in the "
-                         "same GPU's HBM; run it with --gpus 1")
-
-    import torch
-
-    from moodist_amd import _abi as abi
-
-    if not torch.cuda.is_available():
-        raise SystemExit("bench.py needs a GPU")
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    for item in args.tuning:  # before the workload is built: a prepared plan fixes its shape at create time
-        knob, _, value = item.partition("=")
-        abi.set_tuning(knob, int(value))
-    desc, alg_bytes, launch, check, kernel = build_workload(args.workload, torch, abi, dev, args.rotation_mib << 20)
+def measure(name, args, torch, abi, dev):
+    """Builds the workload, warms up, times it and checks its results; returns the JSON line's
+    fields for it.  Everything the workload allocated is released before returning."""
+    desc, alg_bytes, launch, check, kernel = build_workload(name, torch, abi, dev, args.rotation_mib << 20)
     desc["rotation_mib"] = args.rotation_mib
     if args.tuning:
         desc["tuning"] = dict(item.split("=") for item in args.tuning)
@@ -428,6 +487,7 @@ def main():
     desc["window_ms_min_median_max"] = [round(min(window_ms), 5), round(ms, 5), round(max(window_ms), 5)]
     desc["clock_warmup_s"] = args.clock_warmup
     desc["clock_warmup_launches"] = clock_launches
+    checked = False
     if not args.no_check:
         # every set's output is checked: make sure each has been written (a short run may not
         # have gone round the whole rotation)
@@ -435,11 +495,12 @@ def main():
             launch(i)
         torch.cuda.synchronize()
         check()
+        checked = True
     gbs = alg_bytes / (ms_per_step * 1e-3) / 1e9
     kernel_gbs = alg_bytes / (kernel_ms * 1e-3) / 1e9
     out = {
         "metric": "achieved HBM GB/s (% of peak) for 1-GPU local reduce-scatter, fp32 P=8"
-        if args.workload == "reduce_fp32_p8" else "achieved HBM GB/s (% of peak), " + args.workload,
+        if name == "reduce_fp32_p8" else "achieved HBM GB/s (% of peak), " + name,
         "value": round(gbs, 1),
         "unit": "GB/s",
         "n_gpus": 1,
@@ -449,12 +510,13 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": {"float32": "f32", "bfloat16": "bf16", "float16": "f16", "uint8": "u8"}[desc["dtype"]],
+        "dtype": DTYPE_NAMES[desc["dtype"]],
         "data": "synthetic",
         "config": desc,
         "percent_of_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),
         "host_wall_ms_per_step": round(wall_ms / args.steps, 6),
         "host_enqueue_ms_per_step": round(enqueue_ms / args.steps, 6),
+        "result_checked": checked,
         "roofline": {
             "bound": "hbm",
             "kernel": kernel,
@@ -467,11 +529,73 @@ def main():
             "algorithmic_bytes_per_launch": alg_bytes,
             # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by the
             # same counter's reading on a copy of known size; null for a workload not measured
-            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "traffic": MEASURED_TRAFFIC_BYTES.get(name),
         },
     }
-    if not args.no_cpu_baseline and args.workload == "reduce_fp32_p8":
+    # the closures hold every buffer of the workload: let go of them, then of the allocator's cache
+    del launch, check
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--workload", default=None,
+                    help="measure this workload alone (default: the headline, then every other configuration)")
+    ap.add_argument("--headline-only", action="store_true", help="measure reduce_fp32_p8 alone")
+    ap.add_argument("--rotation-mib", type=int, default=4096,
+                    help="touched bytes of all buffer sets together (the launches rotate over them)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-check", action="store_true")
+    ap.add_argument("--clock-warmup", type=float, default=CLOCK_WARMUP_S, metavar="SECONDS",
+                    help="untimed launches before the first timed window (0 under a counter-collecting profiler)")
+    ap.add_argument("--tuning", action="append", default=[], metavar="KNOB=VALUE",
+                    help="force a launch-shape knob of the kernel library (mdh_set_tuning), e.g. reduce_unroll=8")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        raise SystemExit("bench.py measures one GPU: the path is one rank's share with its peers staged in the "
+                         "same GPU's HBM; run it with --gpus 1")
+
+    import torch
+
+    from moodist_amd import _abi as abi
+
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    for item in args.tuning:  # before the workload is built: a prepared plan fixes its shape at create time
+        knob, _, value = item.partition("=")
+        abi.set_tuning(knob, int(value))
+    first = args.workload or ALL_WORKLOADS[0]
+    t_start = time.perf_counter()
+    out = measure(first, args, torch, abi, dev)
+    if not args.no_cpu_baseline and first == "reduce_fp32_p8":
         out["cpu_baseline"] = cpu_baseline()
+    if args.workload is None and not args.headline_only:
+        # every other configuration, same steps, warm-up, rotation and result check; the line's
+        # top-level figures stay the headline's
+        configs = {}
+        for name in ALL_WORKLOADS:
+            if name == first:
+                r = out
+            else:
+                sys.stderr.write("bench: %s (%.0f s so far)\n" % (name, time.perf_counter() - t_start))
+                sys.stderr.flush()
+                r = measure(name, args, torch, abi, dev)
+            rf = r["roofline"]
+            configs[name] = {
+                "kernel": rf["kernel"], "kernel_us": rf["kernel_us"], "frac": rf["frac"], "achieved": rf["achieved"],
+                "algorithmic_bytes": rf["algorithmic_bytes_per_launch"], "traffic": rf["traffic"],
+                "ms_per_step": r["ms_per_step"], "queue_prefilled": bool(r["config"].get("queue_prefilled")),
+                "buffer_sets": r["config"]["buffer_sets"], "result_checked": r["result_checked"],
+            }
+        out["configs"] = configs
+        out["bench_wall_s"] = round(time.perf_counter() - t_start, 1)
     print(json.dumps(out))
 
 

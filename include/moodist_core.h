@@ -29,6 +29,10 @@
  * ordering with later work is by stream, not by the host.
  *
  * Nothing here synchronises the host with the device.
+ *
+ * A stream that is being captured into a graph (hipStreamBeginCapture) is refused by every
+ * collective, with an error and nothing recorded: replaying a graph that holds this library's
+ * launches is not supported.
  */
 #ifndef MOODIST_CORE_H
 #define MOODIST_CORE_H
@@ -121,8 +125,8 @@ int moodist_pg_allreduce(moodist_pg* pg, const moodist_tensor* tensor, const moo
 int moodist_pg_allreduce_many(moodist_pg* pg, const moodist_tensor* tensors, size_t n, int reduce_op, void* stream,
     float premul_value, moodist_work** work);
 /* No counterpart in the reference.  moodist_pg_allreduce for callers that cannot allocate
- * device memory and have no temporary to pass (code under stream capture, tight serving
- * loops, harnesses that forbid hipMalloc): the padded temporary is this rank's slice of the
+ * device memory and have no temporary to pass (tight serving loops, harnesses that forbid
+ * hipMalloc): the padded temporary is this rank's slice of the
  * kernel library's fixed workspace (mdh_static_workspace in moodist_hip.h, 64 MiB per GPU,
  * split evenly over the group's ranks and rounded down to 256 bytes).  Allocates and frees no
  * device memory.  Same results as moodist_pg_allreduce.  Limits:
@@ -134,9 +138,10 @@ int moodist_pg_allreduce_many(moodist_pg* pg, const moodist_tensor* tensors, siz
  *  - the padding elements hold what the last call left there; they are reduced and thrown
  *    away, nothing needs to start at zero.
  * When numel is a multiple of the group size no temporary is used at all.  The first call on
- * a device looks the workspace's address up (and may load the kernel library's code there):
- * a caller that captures streams makes one call, or calls mdh_static_workspace, before it
- * starts capturing. */
+ * a device looks the workspace's address up (and may load the kernel library's code there).
+ * The group option snapshot_inputs, which copies a posted input into memory from an allocator,
+ * is not applied to this call: the tensor is read when the collective launches.
+ * Like every collective here it refuses a stream that is being captured into a graph. */
 int moodist_pg_allreduce_static(moodist_pg* pg, const moodist_tensor* tensor, int reduce_op, void* stream,
     float premul_value, moodist_work** work);
 /* No counterpart in the reference, where a peer's contribution is whatever that peer's own

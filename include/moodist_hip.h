@@ -19,6 +19,9 @@
  *     owns every buffer until that work has finished.  Long copies ask for
  *     40 KiB of dynamic LDS per workgroup that the kernels never touch: it
  *     limits how many workgroups a CU holds at once;
+ *   - `stream` must not be capturing (hipStreamBeginCapture): a launch function that finds it
+ *     capturing enqueues and records nothing and returns MDH_ECAPTURE.  Graph replay of these
+ *     launches is not supported;
  *   - all data pointers are device pointers on the current device; pointer
  *     TABLES (srcs, boxes) are host memory and are consumed before return;
  *   - dtype codes are torch ScalarType numbers and op codes are c10d RedOpType
@@ -44,6 +47,10 @@ extern "C" {
 #define MDH_EOP 3         /* "Unsupported reduce operation" (core/processgroup.cc:294) */
 #define MDH_ELAUNCH 4     /* the HIP runtime refused the launch; see mdh_last_error() */
 #define MDH_ENODEVICE 5   /* no usable gfx950 device */
+#define MDH_ECAPTURE 6    /* `stream` is being captured into a graph: nothing was enqueued or recorded.
+                             Replaying a graph that holds these launches is not supported (the one replay
+                             ever made of them raised an illegal-address fault whose cause was not found),
+                             so every launch function refuses a capturing stream. */
 
 /* api/moodist_api.h:30-42 */
 #define MDH_DTYPE_INT32 3
@@ -104,6 +111,32 @@ const char* mdh_last_error(void);
  */
 int mdh_reduce(const void* const* srcs, int nsrc, int first, void* dst, size_t numel, int dtype, int op,
     float scale, void* stream);
+
+/*
+ * A list of such reductions, all of one element type and operation, in as few launches as
+ * possible: job j is mdh_reduce(jobs[j].srcs, jobs[j].nsrc, jobs[j].first, jobs[j].dst,
+ * jobs[j].numel, dtype, op, scale, stream), with the same results bit for bit.
+ *
+ * Replaces: the loops of the coalesced collectives, which run one reduce_scatter (and so one
+ * kernel launch per rank) per tensor (wrapper/processgroup_wrapper.cc:159-170 for
+ * reduce_scatter_tensor_coalesced, :182-191 for allreduce_coalesced; the fold of each is
+ * core/reduce_scatter.cc:104-142).  Launches of a few KiB to a few MiB are bound by the launch
+ * itself, so the jobs share launches: up to 40 jobs and 320 source pointers per launch, their
+ * tiles numbered through.  A job of 8 MiB per source and more gets a launch of its own, shaped
+ * as mdh_reduce shapes it.  Jobs with numel == 0 are skipped.
+ *
+ * The jobs must be independent: no job's destination may overlap another job's sources or
+ * destination (within a job, dst may equal srcs[first], as for mdh_reduce).  Every job is
+ * checked before anything is enqueued: on an error nothing has been launched.
+ */
+typedef struct mdh_reduce_job {
+  const void* const* srcs; /* nsrc device pointers (the table itself is host memory) */
+  int32_t nsrc;            /* 1..MDH_MAX_SOURCES */
+  int32_t first;           /* the fold starts at srcs[first] */
+  void* dst;
+  size_t numel;
+} mdh_reduce_job;
+int mdh_reduce_many(const mdh_reduce_job* jobs, int njobs, int dtype, int op, float scale, void* stream);
 
 /*
  * All-gather chunk assembly: for every shard s < nsrc and row r < rows,
@@ -186,8 +219,8 @@ int mdh_copy_plan_verify(const mdh_copy_plan* plan, const uint64_t* base_bytes, 
  * bases.  `*size` receives the block's size; `out` may be NULL to ask for the size only.  The
  * block begins with `*leading_scalars` 4-byte scalars, each a kernel parameter of its own
  * (0 for most launches, 14 for one started from preloaded arguments); the rest is one struct
- * parameter.  Enqueues nothing.  For checks of what a stream capture recorded against what an eager
- * launch passes.
+ * parameter.  Enqueues nothing.  For host-side checks of a launch's argument block (for one, against
+ * the kernel node a stream capture recorded, read back and never replayed).
  */
 int mdh_copy_plan_step_arguments(const mdh_copy_plan* plan, const void* const* bases, int nbases, int step, void* out,
     size_t capacity, size_t* size, uint32_t* leading_scalars, uint32_t* grid_x, uint32_t* grid_y, uint32_t* block,
@@ -219,7 +252,16 @@ int mdh_static_workspace(void** address, size_t* bytes);
  * "copy_max_blocks", "copy_wg_per_cu" (2..8, 9 = never cap), "box_policy" (loads of the
  * strided-box kernel: 1 = plain, which pays when the sources are still in the Infinity Cache;
  * 0 or 2 = nt, the default), "box_preload" (1 = never start equal boxes of full tiles from
- * preloaded kernel arguments).  Returns MDH_EINVAL for an unknown name or value.
+ * preloaded kernel arguments), four variants of the dense copy of up to eight equal segments that
+ * exist for measurement and that the library never chooses by itself -- "copy_xcd_run" (2, 4, 8, ...:
+ * each of the eight XCDs takes runs of that many consecutive tiles, where by default adjacent tiles
+ * go to different XCDs), "copy_grid_order" (1: the segments advance together instead of one after
+ * the other), "copy_tail_tiles" (that many tiles at every segment's end are dealt as two halves
+ * each, so the launch ends on short workgroups), "copy_lds" (1: loads go straight to LDS and the
+ * stores are fed from there) --, "allow_capture" (1 = the launch functions accept a capturing
+ * stream; only for a host-side comparison of what a capture records with what an eager launch
+ * passes, by a program that destroys the graph without instantiating it).  Returns MDH_EINVAL
+ * for an unknown name or value.
  * No counterpart in the reference, whose grid is fixed at 4/16/64 blocks
  * (core/kernels.cc:547-556).
  */

@@ -19,7 +19,7 @@ MAX_DIMS = 10
 ABI_VERSION = 2
 
 SYMBOLS = (
-    "mdh_abi_version", "mdh_error_string", "mdh_last_error", "mdh_reduce", "mdh_gather", "mdh_copy_boxes",
+    "mdh_abi_version", "mdh_error_string", "mdh_last_error", "mdh_reduce", "mdh_reduce_many", "mdh_gather", "mdh_copy_boxes",
     "mdh_set_tuning", "mdh_get_tuning", "mdh_copy_plan_create", "mdh_copy_plan_launch", "mdh_copy_plan_launches",
     "mdh_copy_plan_verify", "mdh_copy_plan_destroy", "mdh_copy_plan_step_arguments", "mdh_static_workspace",
 )
@@ -38,6 +38,16 @@ class Box(ctypes.Structure):
         ("shape", ctypes.c_int64 * MAX_DIMS),
         ("src_strides", ctypes.c_int64 * MAX_DIMS),
         ("dst_strides", ctypes.c_int64 * MAX_DIMS),
+    ]
+
+
+class ReduceJob(ctypes.Structure):
+    _fields_ = [
+        ("srcs", ctypes.POINTER(ctypes.c_void_p)),
+        ("nsrc", ctypes.c_int32),
+        ("first", ctypes.c_int32),
+        ("dst", ctypes.c_void_p),
+        ("numel", ctypes.c_size_t),
     ]
 
 
@@ -62,6 +72,9 @@ def lib():
     L.mdh_reduce.argtypes = [vpp, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int,
                              ctypes.c_int, ctypes.c_float, ctypes.c_void_p]
     L.mdh_reduce.restype = ctypes.c_int
+    L.mdh_reduce_many.argtypes = [ctypes.POINTER(ReduceJob), ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_float,
+                                  ctypes.c_void_p]
+    L.mdh_reduce_many.restype = ctypes.c_int
     L.mdh_gather.argtypes = [vpp, ctypes.c_int, ctypes.c_void_p] + [ctypes.c_size_t] * 5 + [ctypes.c_void_p]
     L.mdh_gather.restype = ctypes.c_int
     L.mdh_copy_boxes.argtypes = [ctypes.POINTER(Box), ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
@@ -107,6 +120,26 @@ def ptr_table(ptrs):
 
 def reduce(src_ptrs, first, dst_ptr, numel, dtype, op, scale=1.0, stream=0):
     check(lib().mdh_reduce(ptr_table(src_ptrs), len(src_ptrs), first, dst_ptr, numel, dtype, op, scale, stream))
+
+
+def reduce_jobs(jobs):
+    """A ctypes job table for mdh_reduce_many from (src_ptrs, first, dst_ptr, numel) tuples; the
+    second value returned keeps the pointer tables alive."""
+    arr = (ReduceJob * max(len(jobs), 1))()
+    tables = []
+    for k, (src_ptrs, first, dst_ptr, numel) in enumerate(jobs):
+        tab = ptr_table(src_ptrs)
+        tables.append(tab)
+        arr[k].srcs = ctypes.cast(tab, ctypes.POINTER(ctypes.c_void_p))
+        arr[k].nsrc, arr[k].first, arr[k].dst, arr[k].numel = len(src_ptrs), first, dst_ptr, numel
+    return arr, tables
+
+
+def reduce_many(jobs, dtype, op, scale=1.0, stream=0):
+    """jobs: (src_ptrs, first, dst_ptr, numel) tuples, all of one element type and operation."""
+    arr, tables = reduce_jobs(jobs)
+    check(lib().mdh_reduce_many(arr, len(jobs), dtype, op, scale, stream))
+    del tables
 
 
 def gather(src_ptrs, dst_ptr, width, rows, src_pitch, dst_pitch, dst_shard_stride, stream=0):

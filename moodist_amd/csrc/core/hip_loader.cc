@@ -2,6 +2,7 @@
 
 #include <dlfcn.h>
 
+#include <atomic>
 #include <mutex>
 #include <stdexcept>
 #include <string>
@@ -60,6 +61,8 @@ HipRuntime load() {
   resolve(rt, rn, "hipMemcpyAsync", r.MemcpyAsync);
   resolve(rt, rn, "hipMemcpy2DAsync", r.Memcpy2DAsync);
   resolve(rt, rn, "hipStreamSynchronize", r.StreamSynchronize);
+  resolve(rt, rn, "hipStreamIsCapturing", r.StreamIsCapturing);
+  resolve(rt, rn, "hipGetLastError", r.GetLastError);
   resolve(rt, rn, "hipEventCreateWithFlags", r.EventCreateWithFlags);
   resolve(rt, rn, "hipEventDestroy", r.EventDestroy);
   resolve(rt, rn, "hipEventRecord", r.EventRecord);
@@ -90,11 +93,37 @@ HipRuntime load() {
   return r;
 }
 
+std::atomic<bool> g_loaded{false};
+
 } // namespace
 
 const HipRuntime& hip() {
-  static HipRuntime r = load();
+  static HipRuntime r = [] {
+    HipRuntime loaded = load();
+    g_loaded.store(true, std::memory_order_release);
+    return loaded;
+  }();
   return r;
+}
+
+bool hip_loaded() {
+  return g_loaded.load(std::memory_order_acquire);
+}
+
+void refuse_capture(void* stream, const char* what) {
+  const HipRuntime& h = hip();
+  int status = 0; // hipStreamCaptureStatusNone
+  const int rc = h.StreamIsCapturing(stream, &status);
+  // the legacy default stream reports a capture going on elsewhere as an error of its own
+  const bool capturing = rc == 0 ? status != 0 : rc == kHipErrorStreamCaptureImplicit;
+  if (rc != 0) {
+    h.GetLastError(); // anything else (no device, an unknown stream) is for the launch itself to report
+  }
+  if (capturing) {
+    throw std::runtime_error(std::string("moodist: ") + what +
+                             ": the stream is being captured into a graph; capture and replay of moodist collectives "
+                             "is not supported (call on a stream that is not capturing)");
+  }
 }
 
 void check_hip(int rc, const char* what) {

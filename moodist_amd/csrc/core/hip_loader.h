@@ -26,6 +26,8 @@ struct HipRuntime {
   int (*Memcpy2DAsync)(void* dst, size_t dpitch, const void* src, size_t spitch, size_t width, size_t height, int kind,
       void* stream);
   int (*StreamSynchronize)(void* stream);
+  int (*StreamIsCapturing)(void* stream, int* status);
+  int (*GetLastError)();
   int (*EventCreateWithFlags)(void** event, unsigned flags);
   int (*EventDestroy)(void* event);
   int (*EventRecord)(void* event, void* stream);
@@ -47,10 +49,18 @@ struct HipRuntime {
 
 constexpr int kHipMemcpyDeviceToDevice = 3;
 constexpr unsigned kHipEventDisableTiming = 2;
+constexpr int kHipErrorStreamCaptureImplicit = 906;
 
 // Loads on first call; throws std::runtime_error naming the missing library or
 // symbol.  There is no CPU fallback: without the kernel library nothing runs.
 const HipRuntime& hip();
+
+// Whether hip() has loaded the runtime and the kernel library already (it does on first GPU use).
+bool hip_loaded();
+
+// Throws when `stream` is being captured into a graph: nothing of a collective may be recorded,
+// because replaying a graph that holds these launches is not supported.  Loads the runtime.
+void refuse_capture(void* stream, const char* what);
 
 // Throws std::runtime_error("<what>: <hip error string>") when rc != 0.
 void check_hip(int rc, const char* what);

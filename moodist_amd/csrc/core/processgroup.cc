@@ -105,6 +105,15 @@ size_t bytes_of(const moodist_tensor& t) {
   return (size_t)t.numel * (size_t)t.itemsize;
 }
 
+// A rank's call on a capturing stream is refused when it is made, if the runtime is loaded by
+// then (it is from the first launch on); World::launch asks again for every rank's stream
+// before anything is enqueued, which also covers a process whose first collective is captured.
+void refuse_capture_early(void* stream, const char* what) {
+  if (hip_loaded()) {
+    refuse_capture(stream, what);
+  }
+}
+
 } // namespace
 
 size_t dtype_size(int dtype) {
@@ -189,6 +198,7 @@ void ProcessGroup::snapshot(moodist_tensor& input, void* stream, Keep& keep) {
   if (!options.snapshotInputs || internal_input || bytes == 0) {
     return;
   }
+  refuse_capture(stream, "snapshot_inputs");
   void* cleanup = nullptr;
   void* copy = world->allocator.alloc(bytes, &cleanup, stream, world->device);
   if (!copy) {
@@ -208,6 +218,7 @@ std::shared_ptr<Collective> ProcessGroup::all_gather(const moodist_tensor* outpu
 std::shared_ptr<Collective> ProcessGroup::all_gather_impl(const moodist_tensor* output, const moodist_tensor& input,
     void* stream, const moodist_tensor* copy_back, Keep keep) {
   Busy guard(*this);
+  refuse_capture_early(stream, "all_gather");
   check_device_tensor(input, world->device, "all_gather input");
   const size_t bytes = bytes_of(input);
   MD_CHECK(bytes > 0); // core/processgroup.cc:1078
@@ -236,6 +247,7 @@ std::shared_ptr<Collective> ProcessGroup::all_gather_impl(const moodist_tensor* 
 std::shared_ptr<Collective> ProcessGroup::all_gather_list(const moodist_tensor* outputs, size_t n_outputs,
     const moodist_tensor& input, void* stream, Keep keep) {
   Busy guard(*this);
+  refuse_capture_early(stream, "all_gather");
   check_device_tensor(input, world->device, "all_gather input");
   const size_t bytes = bytes_of(input);
   MD_CHECK(bytes > 0);
@@ -266,6 +278,7 @@ std::shared_ptr<Collective> ProcessGroup::all_gather_list(const moodist_tensor* 
 std::shared_ptr<Collective> ProcessGroup::all_gather_many(const moodist_tensor* outputs, const moodist_tensor* inputs,
     size_t n, void* stream, Keep keep) {
   Busy guard(*this);
+  refuse_capture_early(stream, "all_gather");
   if (n == 0 || n > 0xffffu) {
     throw std::runtime_error("moodist: a coalesced all_gather takes 1..65535 tensors, not " + std::to_string(n));
   }
@@ -296,6 +309,7 @@ std::shared_ptr<Collective> ProcessGroup::all_gather_many(const moodist_tensor* 
 std::shared_ptr<Collective> ProcessGroup::reduce_scatter(const moodist_tensor* output, const moodist_tensor& input,
     int reduce_op, void* stream, float premul, Keep keep) {
   Busy guard(*this);
+  refuse_capture_early(stream, "reduce_scatter");
   check_device_tensor(input, world->device, "reduce_scatter input");
   check_reduce_dtype(input.dtype);
   check_reduce_op(reduce_op);
@@ -356,6 +370,7 @@ std::shared_ptr<Collective> ProcessGroup::allreduce(const moodist_tensor& tensor
   check_device_tensor(*scratch, world->device, "allreduce scratch");
   MD_CHECK(scratch->dtype == tensor.dtype && scratch->numel >= padded);
   const size_t bytes = bytes_of(tensor);
+  refuse_capture(stream, "allreduce");
   check_hip(hip().MemcpyAsync(scratch->data, tensor.data, bytes, kHipMemcpyDeviceToDevice, stream), "hipMemcpyAsync");
   moodist_tensor whole = *scratch;
   whole.numel = padded;
@@ -416,6 +431,19 @@ std::shared_ptr<Collective> ProcessGroup::allreduce_static(const moodist_tensor&
     float premul, Keep keep) {
   check_device_tensor(tensor, world->device, "allreduce tensor");
   MD_CHECK(tensor.numel > 0);
+  // No allocation of any kind in this call: the option snapshot_inputs, which copies a posted
+  // input into memory from the wrapper's allocator, is not applied (the tensor is read when
+  // the collective launches).
+  struct NoSnapshot {
+    bool& flag;
+    const bool before;
+    explicit NoSnapshot(bool& f) : flag(f), before(f) {
+      flag = true;
+    }
+    ~NoSnapshot() {
+      flag = before;
+    }
+  } no_snapshot{internal_input};
   if (tensor.numel % size == 0) {
     return allreduce(tensor, nullptr, reduce_op, stream, premul, std::move(keep)); // in place, no temporary
   }
@@ -496,6 +524,7 @@ std::shared_ptr<Collective> ProcessGroup::custom_op(const std::shared_ptr<Compil
     const moodist_tensor* inputs, size_t n_inputs, const moodist_tensor* outputs, size_t n_outputs, void* stream,
     Keep keep) {
   Busy guard(*this);
+  refuse_capture_early(stream, "custom op");
   const RankPlan& plan = op->plans[(size_t)rank];
   // core/processgroup.cc:3180-3185, :3205-3216
   if (n_inputs != plan.inputs.size()) {
@@ -775,6 +804,17 @@ void World::launch(Collective& c, const std::shared_ptr<CompiledOp>& op) {
   check_hip(h.GetDevice(&current), "hipGetDevice");
   if (current != device) {
     check_hip(h.SetDevice(device), "hipSetDevice");
+  }
+  // before anything is enqueued -- an event record on a capturing stream would already be a
+  // node of its graph
+  for (int r = 0; r < size; ++r) {
+    bool seen = false;
+    for (int k = 0; k < r; ++k) {
+      seen = seen || c.post[(size_t)k].stream == c.post[(size_t)r].stream;
+    }
+    if (!seen) {
+      refuse_capture(c.post[(size_t)r].stream, "collective launch");
+    }
   }
   order_streams_before(c);
   std::vector<const void*> srcs((size_t)size);

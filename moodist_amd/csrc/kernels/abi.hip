@@ -30,6 +30,25 @@ Tuning& tuning() {
   return t;
 }
 
+int refuse_capture(hipStream_t stream, const char* who) {
+  if (tuning().allow_capture) {
+    return MDH_OK;
+  }
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  const hipError_t e = hipStreamIsCapturing(stream, &status);
+  // the legacy default stream reports a capture going on elsewhere as an error of its own
+  const bool capturing = e == hipSuccess ? status != hipStreamCaptureStatusNone : e == hipErrorStreamCaptureImplicit;
+  if (e != hipSuccess) {
+    (void)hipGetLastError(); // no device, or an unknown stream: the launch itself will say so
+  }
+  if (!capturing) {
+    return MDH_OK;
+  }
+  set_error("%s: the stream is being captured into a graph; capture and replay of these launches is not supported "
+            "(launch on a stream that is not capturing)", who);
+  return MDH_ECAPTURE;
+}
+
 } // namespace mdh
 
 extern "C" int mdh_abi_version(void) {
@@ -54,6 +73,8 @@ extern "C" const char* mdh_error_string(int code) {
     return "kernel launch failed";
   case MDH_ENODEVICE:
     return "no usable gfx950 device";
+  case MDH_ECAPTURE:
+    return "the stream is being captured into a graph, which these launches do not support";
   default:
     return "unknown error";
   }
@@ -98,6 +119,21 @@ int* knob(const char* name) {
   if (!std::strcmp(name, "copy_max_blocks")) {
     return &t.copy_max_blocks;
   }
+  if (!std::strcmp(name, "copy_xcd_run")) {
+    return &t.copy_xcd_run;
+  }
+  if (!std::strcmp(name, "copy_grid_order")) {
+    return &t.copy_grid_order;
+  }
+  if (!std::strcmp(name, "copy_tail_tiles")) {
+    return &t.copy_tail_tiles;
+  }
+  if (!std::strcmp(name, "copy_lds")) {
+    return &t.copy_lds;
+  }
+  if (!std::strcmp(name, "allow_capture")) {
+    return &t.allow_capture;
+  }
   return nullptr;
 }
 } // namespace
@@ -116,7 +152,7 @@ extern "C" int mdh_set_tuning(const char* name, int value) {
       return MDH_EINVAL;
     }
   } else if (value < 0 || (std::strstr(name, "wg_per_cu") && value > 9) || (!std::strcmp(name, "box_policy") && value > 2) ||
-             (!std::strcmp(name, "box_preload") && value > 1)) {
+             (!std::strcmp(name, "box_preload") && value > 1) || (!std::strcmp(name, "allow_capture") && value > 1)) {
     mdh::set_error("mdh_set_tuning: %s does not take %d", name, value);
     return MDH_EINVAL;
   }

@@ -16,6 +16,7 @@
 #include <algorithm>
 #include <cstring>
 #include <memory>
+#include <utility>
 #include <vector>
 
 namespace mdh {
@@ -508,24 +509,83 @@ __global__ __launch_bounds__(kBlock) void copy_flat_kernel(FlatArgs a) {
 // vectors, or whose destinations are off the 64-byte grid, cut to one common length of whole
 // vectors.  Workgroup 0 of every row copies its segment's edge bytes and the tiles are
 // workgroups 1, 2, ...: a workgroup knows which it is from blockIdx alone.
-template<int U, bool EDGES>
-__global__ __launch_bounds__(kBlock) void copy_flat8_kernel(uint32_t bytes, uint32_t, uint32_t l0, uint32_t l1, uint32_t l2,
+// VARIANT (measurement only; the tuning knobs copy_xcd_run, copy_grid_order, copy_tail_tiles and
+// copy_lds select it, the library by itself never does): 0 is the kernel as described above.
+//   1  the second leading argument carries a different dealing of the tiles: bits 0-4, n > 0:
+//      every XCD (workgroups go to the eight XCDs round-robin) takes runs of 2^(n-1) consecutive
+//      tiles instead of every eighth tile; bit 5: the grid is transposed, blockIdx.x the segment
+//      and blockIdx.y the tile, so that the segments advance together (and with eight segments
+//      every XCD copies one of them); bits 8-31: that many tiles at every segment's end are dealt
+//      as two halves each, so that the launch ends on short workgroups;
+//   2  the loads go straight to LDS (buffer_load ... lds) and the stores are fed from there by
+//      ds_read_b128: no vector register holds a byte in flight.
+constexpr uint32_t kVariantOrderMask = 31u, kVariantTransposed = 32u, kVariantTailShift = 8;
+
+constexpr int waitcnt_vm(int n) { // s_waitcnt vmcnt(n), other counters left alone (gfx9 encoding)
+  return (n & 0xf) | ((n >> 4) << 14) | (0x7 << 4) | (0xf << 8);
+}
+
+// Sub-tile I's load has landed when at most U-1-I loads are still out (they complete in order):
+// its 16 bytes per lane go from LDS to the destination while the later ones are still in flight.
+template<int U, int... I>
+__device__ __forceinline__ void drain_staged(std::integer_sequence<int, I...>, const char* staged, __amdgpu_buffer_rsrc_t rd,
+    uint32_t lane_byte) {
+  ((__builtin_amdgcn_s_waitcnt(waitcnt_vm(U - 1 - I)),
+       tile_store(rd, lane_byte + (uint32_t)I * (kBlock * 16), *(const u32x4*)(staged + I * (kBlock * 16) + lane_byte))),
+      ...);
+}
+
+template<int U, bool EDGES, int VARIANT = 0>
+__global__ __launch_bounds__(kBlock) void copy_flat8_kernel(uint32_t bytes, uint32_t opts, uint32_t l0, uint32_t l1, uint32_t l2,
     uint32_t l3, uint32_t l4, uint32_t l5, uint32_t l6, uint32_t l7, uint32_t h0, uint32_t h1, uint32_t h2, uint32_t h3,
     FlatArgs a) {
+  static_assert(VARIANT == 0 || !EDGES, "the measurement variants are for segments without edge bytes");
   constexpr uint32_t tile_bytes = kBlock * U * 16;
   const uint32_t lane_byte = threadIdx.x * 16;
-  const uint32_t seg = blockIdx.y;
+  uint32_t seg = blockIdx.y;
   if (EDGES && blockIdx.x == 0) {
     // FlatArgs follows the fourteen leading dwords in the argument segment
     const char* segment = (const char*)__builtin_amdgcn_kernarg_segment_ptr();
     copy_segment_edges((const FlatArgs*)(segment + sizeof(FlatLead)), seg, threadIdx.x);
     return;
   }
-  const uint32_t off = (blockIdx.x - (EDGES ? 1u : 0u)) * tile_bytes; // below the segment's length, which fits 32 bits
-  const uint32_t left = bytes - off;
-  const uint32_t n = left < tile_bytes ? left : tile_bytes;
+  uint32_t off = (blockIdx.x - (EDGES ? 1u : 0u)) * tile_bytes; // below the segment's length, which fits 32 bits
+  uint32_t reach = tile_bytes;
+  if (VARIANT == 1) {
+    uint32_t b = blockIdx.x;
+    if (opts & kVariantTransposed) {
+      seg = blockIdx.x, b = blockIdx.y;
+    }
+    const uint32_t order = opts & kVariantOrderMask;
+    if (order) {
+      const uint32_t lr = order - 1, xcd = b & 7u, idx = b >> 3;
+      b = ((((idx >> lr) << 3) | xcd) << lr) | (idx & ((1u << lr) - 1u));
+    }
+    const uint32_t tail = opts >> kVariantTailShift;
+    const uint32_t whole = (bytes + tile_bytes - 1) / tile_bytes - tail; // tiles dealt whole
+    off = b * tile_bytes;
+    if (b >= whole) {
+      off = whole * tile_bytes + (b - whole) * (tile_bytes / 2);
+      reach = tile_bytes / 2;
+    }
+  }
+  const uint32_t left = off < bytes ? bytes - off : 0;
+  const uint32_t n = left < reach ? left : reach;
   const char* src = (const char*)(uintptr_t)packed_source_address(seg, l0, l1, l2, l3, l4, l5, l6, l7, h0, h1, h2, h3);
   const __amdgpu_buffer_rsrc_t rs = tile_rsrc(src + off, n);
+  if (VARIANT == 2) {
+    extern __shared__ __attribute__((aligned(16))) char staged[];
+    const uint32_t wave_base = (threadIdx.x >> 6) * 1024u;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      // a wave's 64 lanes land in 1 KiB of LDS starting at the (wave-uniform) address given
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(staged + u * (kBlock * 16) + wave_base),
+          16, (int)(lane_byte + (uint32_t)u * (kBlock * 16)), 0, 0, MDH_LOAD_AUX);
+    }
+    const __amdgpu_buffer_rsrc_t rd = tile_rsrc(a.dst[seg] + off, n);
+    drain_staged<U>(std::make_integer_sequence<int, U>{}, staged, rd, lane_byte);
+    return;
+  }
   u32x4 v[U];
 #pragma unroll
   for (int u = 0; u < U; ++u) {
@@ -570,6 +630,9 @@ struct Step {
   bool plain_loads; // kBoxes16: plain instead of nt loads (tuning knob)
   bool preloaded = false; // equal boxes of full tiles / equal segments of one length: started from preloaded arguments
   bool edge_column = false; // kFlat, two-dimensional form: workgroup 0 of every row copies its segment's edge bytes
+  int variant = 0;          // copy_flat8_kernel's measurement variants (tuning knobs only)
+  uint32_t variant_opts = 0;
+  uint32_t variant_grid_x = 0, variant_grid_y = 0;
   size_t lds;
   FlatArgs flat;   // kFlat
   CopyArgs boxes;  // kBoxes16, kBoxes
@@ -668,16 +731,18 @@ inline bool uniform_segments(const FlatArgs& a) {
   return true;
 }
 
-inline bool make_flat_lead(const FlatArgs& a, FlatLead* lead) {
+inline bool make_flat_lead(const FlatArgs& a, FlatLead* lead, uint32_t opts = 0) {
   lead->bytes = (uint32_t)a.bytes[0];
-  lead->reserved = 0;
+  lead->reserved = opts;
   return pack_sources(a.src, a.nsegs, &lead->from);
 }
 
 // The grid a step is launched with: st.grid (x st.grid_y) tile workgroups, and in the
 // one-dimensional form of a flat step the edge workgroups in front of them.
 inline void launch_dims(const Step& st, uint32_t* x, uint32_t* y) {
-  if (st.grid_y > 0) {
+  if (st.variant != 0) {
+    *x = st.variant_grid_x, *y = st.variant_grid_y;
+  } else if (st.grid_y > 0) {
     *x = st.grid + (st.edge_column ? 1u : 0u);
     *y = st.grid_y;
   } else {
@@ -737,6 +802,44 @@ struct Launcher {
       cap = tuning().copy_wg_per_cu;
     }
     lds = cap >= 2 && cap <= 8 ? kLdsForCap[cap] : 0; // one per CU would need the LDS limit raised
+  }
+
+  // The measurement variants of copy_flat8_kernel, for launches that qualify (preloaded form, no
+  // edge bytes); a knob that does not fit the launch is ignored.
+  void choose_variant(Step& st, const FlatArgs& a) {
+    const Tuning& t = tuning();
+    if (!st.preloaded || st.edge_column || !(t.copy_xcd_run || t.copy_grid_order || t.copy_tail_tiles || t.copy_lds)) {
+      return;
+    }
+    const uint32_t tiles = a.tiles_per_seg;
+    if (t.copy_lds) {
+      st.variant = 2, st.variant_opts = 0;
+      st.variant_grid_x = st.grid, st.variant_grid_y = st.grid_y;
+      const size_t need = (size_t)kBlock * 16 * (size_t)st.unroll;
+      st.lds = st.lds > need ? st.lds : need;
+      return;
+    }
+    uint32_t opts = 0, gx = tiles;
+    const uint32_t tail = (uint32_t)t.copy_tail_tiles;
+    if (tail > 0 && tail < tiles && a.bytes[0] % ((uint64_t)kBlock * 16 * (uint64_t)st.unroll) == 0) {
+      opts |= tail << kVariantTailShift;
+      gx = tiles + tail;
+    }
+    const uint32_t run = (uint32_t)t.copy_xcd_run;
+    if (run >= 2 && (run & (run - 1)) == 0 && gx == tiles && tiles % (8 * run) == 0 && !t.copy_grid_order) {
+      uint32_t lr = 0;
+      while ((1u << lr) < run) {
+        ++lr;
+      }
+      opts |= lr + 1;
+    }
+    if (t.copy_grid_order) {
+      opts |= kVariantTransposed;
+      st.variant_grid_x = st.grid_y, st.variant_grid_y = gx;
+    } else {
+      st.variant_grid_x = gx, st.variant_grid_y = st.grid_y;
+    }
+    st.variant = 1, st.variant_opts = opts;
   }
 
   void flush_flat() {
@@ -841,6 +944,7 @@ struct Launcher {
         st.edge_column = edges;
         a.edge_wgs = edges ? 2 : 0;
         st.preloaded = t.box_preload != 1 && uniform_segments(a);
+        choose_variant(st, a);
       }
       submit(st, &a, nullptr);
     }
@@ -1210,6 +1314,30 @@ int launch_step(const Step& st, const FlatArgs* flat, const CopyArgs* boxes, hip
   switch (st.kind) {
   case Step::kFlat: {
     FlatLead L;
+    if (st.preloaded && st.variant != 0 && make_flat_lead(*flat, &L, st.variant_opts)) {
+#define MDH_LAUNCH_VARIANT(UU)                                                                                               \
+  if (st.variant == 1) {                                                                                                     \
+    hipLaunchKernelGGL((copy_flat8_kernel<UU, false, 1>), g, b, st.lds, stream, L.bytes, L.reserved, MDH_PACKED(L.from), *flat); \
+  } else {                                                                                                                   \
+    hipLaunchKernelGGL((copy_flat8_kernel<UU, false, 2>), g, b, st.lds, stream, L.bytes, L.reserved, MDH_PACKED(L.from), *flat); \
+  }
+      switch (st.unroll) {
+      case 1:
+        MDH_LAUNCH_VARIANT(1)
+        break;
+      case 2:
+        MDH_LAUNCH_VARIANT(2)
+        break;
+      case 4:
+        MDH_LAUNCH_VARIANT(4)
+        break;
+      default:
+        MDH_LAUNCH_VARIANT(8)
+        break;
+      }
+#undef MDH_LAUNCH_VARIANT
+      return check_launch("copy_flat8_kernel");
+    }
     if (st.preloaded && make_flat_lead(*flat, &L)) {
 #define MDH_LAUNCH_FLAT8(UU)                                                                                          \
   if (st.edge_column) {                                                                                               \
@@ -1589,6 +1717,11 @@ extern "C" int mdh_copy_plan_verify(const mdh_copy_plan* plan, const uint64_t* b
         return MDH_EINVAL;
       }
     }
+    if (st.variant != 0) {
+      set_error("mdh_copy_plan_verify: step %zu was prepared with a measurement knob set (copy_xcd_run, copy_grid_order, "
+                "copy_tail_tiles or copy_lds), which this check does not replay", s);
+      return MDH_EINVAL;
+    }
     if (st.kind == Step::kFlat) {
       const FlatArgs& a = st.flat;
       const uint32_t tile_bytes = (uint32_t)kBlock * (uint32_t)st.unroll * 16u;
@@ -1763,6 +1896,9 @@ extern "C" int mdh_copy_plan_launch(const mdh_copy_plan* plan, const void* const
     set_error("mdh_copy_plan_launch: the plan takes %d base addresses", plan ? plan->nbases : 0);
     return MDH_EINVAL;
   }
+  if (const int rc = refuse_capture((hipStream_t)stream, "mdh_copy_plan_launch")) {
+    return rc;
+  }
   uintptr_t low = 0;
   for (int i = 0; i < nbases; ++i) {
     low |= (uintptr_t)bases[i];
@@ -1839,7 +1975,7 @@ extern "C" int mdh_copy_plan_step_arguments(const mdh_copy_plan* plan, const voi
     patch_step(*plan, (size_t)step, at, bases, &flat, nullptr);
     from = &flat;
     *size = sizeof(FlatArgs);
-    if (st.preloaded && make_flat_lead(flat, &lead.flat)) {
+    if (st.preloaded && make_flat_lead(flat, &lead.flat, st.variant ? st.variant_opts : 0u)) {
       lead_bytes = sizeof(FlatLead);
       *size += lead_bytes;
     }
@@ -1882,6 +2018,11 @@ extern "C" int mdh_copy_boxes(const mdh_box* boxes, int nboxes, int itemsize, vo
   if (itemsize < 1 || itemsize > 16 || (itemsize & (itemsize - 1))) {
     set_error("mdh_copy_boxes: itemsize %d is not 1, 2, 4, 8 or 16", itemsize);
     return MDH_EINVAL;
+  }
+  if (nboxes > 0) {
+    if (const int rc = refuse_capture((hipStream_t)stream, "mdh_copy_boxes")) {
+      return rc;
+    }
   }
   Launcher L;
   L.stream = (hipStream_t)stream;
@@ -1942,6 +2083,9 @@ extern "C" int mdh_gather(const void* const* srcs, int nsrc, void* dst, size_t w
   if (nsrc > 1 && dst_shard_stride < extent) {
     set_error("mdh_gather: shards would overlap in the destination");
     return MDH_EINVAL;
+  }
+  if (const int rc = refuse_capture((hipStream_t)stream, "mdh_gather")) {
+    return rc;
   }
   Launcher L;
   L.stream = (hipStream_t)stream;

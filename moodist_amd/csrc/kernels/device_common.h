@@ -80,6 +80,11 @@ void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
 
 int check_launch(const char* what);
 
+// MDH_OK when launches may be enqueued on `stream`; MDH_ECAPTURE, with the message set, when the
+// stream is being captured into a graph (see MDH_ECAPTURE).  Every launch function asks before
+// it enqueues anything.
+int refuse_capture(hipStream_t stream, const char* who);
+
 // 0 = choose by size (the default); any other value is taken as given.
 struct Tuning {
   int reduce_unroll = 0; // KiB of each source per tile: 1, 2, 4, 8, 16
@@ -93,6 +98,12 @@ struct Tuning {
   int copy_wg_per_cu = 0; // as reduce_wg_per_cu, for the copy kernels
   int box_policy = 0;     // loads of the strided-box kernel: 1 plain, 0 or 2 nt
   int box_preload = 0;    // 1: never launch equal boxes of full tiles from preloaded arguments
+  // measurement variants of the dense copy of up to eight equal segments (see copy_flat8_kernel)
+  int copy_xcd_run = 0;    // 2, 4, 8, ...: every XCD takes runs of this many consecutive tiles
+  int copy_grid_order = 0; // 1: the grid is transposed, the segments advance together
+  int copy_tail_tiles = 0; // this many tiles at every segment's end are dealt as two halves each
+  int copy_lds = 0;        // 1: loads go straight to LDS, stores are fed from there
+  int allow_capture = 0;  // 1: launch functions accept a capturing stream (for a host-side check of what a capture records)
 };
 Tuning& tuning();
 

@@ -22,4 +22,9 @@ using f16 = f16_t;
 int MDH_CAT(reduce_launch_, MDH_TNAME, _, MDH_FNAME)(const ReduceArgs& a, hipStream_t stream) {
   return launch<MDH_TNAME, MDH_FNAME>(a, stream);
 }
+
+int MDH_CAT(reduce_many_launch_, MDH_TNAME, _, MDH_FNAME)(const ManyJob* jobs, int njobs, int mode, float scale,
+    hipStream_t stream) {
+  return launch_many<MDH_TNAME, MDH_FNAME>(jobs, njobs, mode, scale, stream);
+}
 } // namespace mdh

@@ -226,7 +226,8 @@ __device__ __forceinline__ void fold_chunk(float scale, const char* const (&src)
 // One element, folded in source order.  The loads of eight sources are issued together: one
 // after the other, every source would cost this lane a whole memory round trip.
 template<typename T, int F>
-__device__ __forceinline__ void reduce_one_elem(const ReduceArgs& a, int nsrc, int64_t i) {
+__device__ __forceinline__ void reduce_one_elem_from(const void* const* src, int nsrc, void* dst, int mode, float scale,
+    int64_t i) {
   using Tr = Traits<T>;
   using elem_t = typename Tr::elem_t;
   using acc_t = typename Tr::acc_t;
@@ -237,20 +238,25 @@ __device__ __forceinline__ void reduce_one_elem(const ReduceArgs& a, int nsrc, i
 #pragma unroll
     for (int k = 0; k < kBatch; ++k) {
       const int j = j0 + k < nsrc ? j0 + k : nsrc - 1; // past the end: the last source once more, unused
-      v[k] = ((const elem_t*)a.src[j])[i];
+      v[k] = ((const elem_t*)src[j])[i];
     }
 #pragma unroll
     for (int k = 0; k < kBatch; ++k) {
       if (j0 + k < nsrc) {
         acc_t x = Tr::widen(v[k]);
-        if (a.mode == kPremul) {
-          x = Tr::premul(x, a.scale);
+        if (mode == kPremul) {
+          x = Tr::premul(x, scale);
         }
         acc = j0 + k == 0 ? x : fold<F>(acc, x);
       }
     }
   }
-  ((elem_t*)a.dst)[i] = Tr::template finish<F>(acc, a.mode, a.scale);
+  ((elem_t*)dst)[i] = Tr::template finish<F>(acc, mode, scale);
+}
+
+template<typename T, int F>
+__device__ __forceinline__ void reduce_one_elem(const ReduceArgs& a, int nsrc, int64_t i) {
+  reduce_one_elem_from<T, F>(a.src, nsrc, a.dst, a.mode, a.scale, i);
 }
 
 // The head before the pointers (indices -head .. -1, fewer than 64 bytes) and the tail after the
@@ -282,9 +288,13 @@ __device__ __forceinline__ void fold_rest(float scale, int rest, const char* con
 
 // One tile: U KiB of every source (U sub-tiles of one wave-wide 16-byte load each), consumed CH
 // sources at a time in order, so the fold stays a left fold and CH*U loads are in flight.
-template<typename T, int F, int U, int CH, int MODE>
-__device__ __forceinline__ void reduce_tile(const ReduceArgs& a, const char* const (&early)[kEarlySources], int nsrc,
-    int mode_arg, float scale, uint64_t tile_byte, uint32_t tile_bytes) {
+// Where the source pointers come from is the caller's business: early(integral_constant<int, K>,
+// p) fills p with the pointers of sources K .. K+CH-1 for a K known at compile time (the first
+// two groups), later(first, p) does the same for any group.  Slots past the last source may hold
+// anything; they are never used.
+template<typename T, int F, int U, int CH, int MODE, typename Early, typename Later>
+__device__ __forceinline__ void reduce_tile_from(Early early_pointers, Later pointers, const char* dst, int nsrc, int mode_arg,
+    float scale, uint64_t tile_byte, uint32_t tile_bytes) {
   using Tr = Traits<T>;
   using elem_t = typename Tr::elem_t;
   using acc_t = typename Tr::acc_t;
@@ -293,25 +303,7 @@ __device__ __forceinline__ void reduce_tile(const ReduceArgs& a, const char* con
   acc_t acc[U][N];
   // The pointers of a group are read from the argument table one group AHEAD of their use: read
   // when needed, every group would start with a scalar round trip during which the wave has no
-  // load in flight.  (Slots past the last source are never used; 63 is the table's last index.)
-  auto pointers = [&](int first, const char* (&p)[CH]) {
-#pragma unroll
-    for (int k = 0; k < CH; ++k) {
-      const int j = first + k;
-      p[k] = (const char*)a.src[j < MDH_MAX_SOURCES ? j : MDH_MAX_SOURCES - 1];
-    }
-  };
-  // The first two groups' indices are compile-time constants: those below kEarlySources are
-  // the kernel's leading arguments, in registers when the wave starts, so the first vector
-  // loads wait for no scalar load at all.
-  auto early_pointers = [&](auto first, const char* (&p)[CH]) {
-#pragma unroll
-    for (int k = 0; k < CH; ++k) {
-      constexpr int kFirst = decltype(first)::value;
-      const int j = kFirst + k;
-      p[k] = j < kEarlySources ? early[j < kEarlySources ? j : 0] : (const char*)a.src[j < MDH_MAX_SOURCES ? j : MDH_MAX_SOURCES - 1];
-    }
-  };
+  // load in flight.
   const char* cur[CH];
   const char* nxt[CH];
   early_pointers(std::integral_constant<int, 0>{}, cur);
@@ -332,7 +324,7 @@ __device__ __forceinline__ void reduce_tile(const ReduceArgs& a, const char* con
   } else {
     fold_rest<T, F, U, CH, MODE, true>(scale, nsrc, cur, tile_byte, tile_bytes, lane_byte, acc);
   }
-  const __amdgpu_buffer_rsrc_t rd = tile_rsrc((const char*)a.dst + tile_byte, tile_bytes);
+  const __amdgpu_buffer_rsrc_t rd = tile_rsrc(dst + tile_byte, tile_bytes);
   u32x4 out[U];
   // AVG's extra multiply is decided once per tile (wave-uniform), not per element
   const int mode = MODE == kPremul ? (int)kPremul : mode_arg;
@@ -364,6 +356,33 @@ __device__ __forceinline__ void reduce_tile(const ReduceArgs& a, const char* con
   for (int u = 0; u < U; ++u) {
     tile_store(rd, lane_byte + (uint32_t)u * (kWave * 16), out[u]); // dropped by the hardware past the end
   }
+}
+
+// The tile of a single reduction: pointers from the launch's argument struct, the first
+// kEarlySources of them from the kernel's leading arguments.
+template<typename T, int F, int U, int CH, int MODE>
+__device__ __forceinline__ void reduce_tile(const ReduceArgs& a, const char* const (&early)[kEarlySources], int nsrc,
+    int mode_arg, float scale, uint64_t tile_byte, uint32_t tile_bytes) {
+  // (slots past the last source are never used; 63 is the table's last index)
+  auto pointers = [&](int first, const char* (&p)[CH]) {
+#pragma unroll
+    for (int k = 0; k < CH; ++k) {
+      const int j = first + k;
+      p[k] = (const char*)a.src[j < MDH_MAX_SOURCES ? j : MDH_MAX_SOURCES - 1];
+    }
+  };
+  // The first two groups' indices are compile-time constants: those below kEarlySources are
+  // the kernel's leading arguments, in registers when the wave starts, so the first vector
+  // loads wait for no scalar load at all.
+  auto early_pointers = [&](auto first, const char* (&p)[CH]) {
+#pragma unroll
+    for (int k = 0; k < CH; ++k) {
+      constexpr int kFirst = decltype(first)::value;
+      const int j = kFirst + k;
+      p[k] = j < kEarlySources ? early[j < kEarlySources ? j : 0] : (const char*)a.src[j < MDH_MAX_SOURCES ? j : MDH_MAX_SOURCES - 1];
+    }
+  };
+  reduce_tile_from<T, F, U, CH, MODE>(early_pointers, pointers, (const char*)a.dst, nsrc, mode_arg, scale, tile_byte, tile_bytes);
 }
 
 // A tile is kWave*U consecutive 16-byte vectors (U KiB); tiles are dealt to
@@ -582,10 +601,191 @@ int launch(const ReduceArgs& a, hipStream_t stream) {
   return launch_vec<T, F>(a, stream);
 }
 
+// ---- a list of reductions in one launch ----
+//
+// The coalesced collectives bring many small tensors at once (reduce_scatter_tensor_coalesced,
+// allreduce_coalesced: wrapper/processgroup_wrapper.cc:159-191 loop over them, one collective and
+// one kernel launch each).  Launches of a few KiB to a few MiB are bound by the 1.6 us an empty
+// launch takes, so here a list of reductions -- jobs, each with its own sources, destination and
+// length, all of one element type and operation -- shares launches: the jobs' tiles are numbered
+// through, a wave finds its tile's job in a table of cumulative tile counts (scalar selects), and
+// the fold is the same code as a single reduction's.
+constexpr int kManyJobs = 40;
+constexpr int kManyPointers = 320; // 40 jobs of 8 sources, 5 of 64
+constexpr int kManyTailSlots = 8;  // lanes per job for the elements after its last whole vector (at most 7)
+
+struct ManyArgs {
+  const void* ptr[kManyPointers]; // every job's sources in fold order, job after job
+  void* dst[kManyJobs];
+  uint32_t nvec[kManyJobs];     // whole 16-byte vectors
+  uint32_t tile_end[kManyJobs]; // cumulative tiles; unused entries are ~0
+  uint16_t first_ptr[kManyJobs];
+  uint8_t nsrc[kManyJobs];
+  uint8_t tail[kManyJobs]; // elements after the last whole vector
+  uint32_t njobs;
+  uint32_t total_tiles;
+  uint32_t tile_waves; // tile workgroups of the grid (the edge workgroups come first)
+  uint32_t edge_wgs;
+  float scale;
+  int mode;
+};
+static_assert(sizeof(ManyArgs) + 256 <= 4096, "kernel arguments are limited to 4 KiB");
+
+// The elements after each job's last whole vector, one per lane: job = lane index / 8.
+template<typename T, int F>
+__device__ __attribute__((noinline)) void reduce_many_edges(const ManyArgs* args, uint32_t wg, uint32_t lane_id) {
+  const ManyArgs& a = *args;
+  const uint32_t idx = wg * kWave + lane_id;
+  const uint32_t job = idx / kManyTailSlots, k = idx % kManyTailSlots;
+  if (job < a.njobs && k < a.tail[job]) {
+    const int64_t i = (int64_t)a.nvec[job] * per_vec<T>() + k;
+    reduce_one_elem_from<T, F>(a.ptr + a.first_ptr[job], a.nsrc[job], a.dst[job], a.mode, a.scale, i);
+  }
+}
+
+template<typename T, int F, int U, int CH, bool PREMUL>
+__global__ __launch_bounds__(kWave) void reduce_many_kernel(ManyArgs a) {
+  constexpr uint32_t tile_bytes = (uint32_t)kWave * U * 16;
+  if (blockIdx.x < a.edge_wgs) {
+    // (the argument segment's address has to be taken here, in the kernel)
+    reduce_many_edges<T, F>((const ManyArgs*)__builtin_amdgcn_kernarg_segment_ptr(), blockIdx.x, threadIdx.x);
+    return;
+  }
+  // the tile workgroups never outnumber the tiles: the first tile is taken untested
+  uint32_t tile = blockIdx.x - a.edge_wgs;
+  do {
+    uint32_t job = 0, start = 0;
+#pragma unroll
+    for (int k = 0; k < kManyJobs - 1; ++k) {
+      const uint32_t e = a.tile_end[k];
+      job = tile >= e ? (uint32_t)(k + 1) : job;
+      start = tile >= e ? e : start;
+    }
+    const uint64_t tile_byte = (uint64_t)(tile - start) * tile_bytes;
+    const uint64_t left = (uint64_t)a.nvec[job] * 16 - tile_byte;
+    const uint32_t n = (uint32_t)(left < tile_bytes ? left : tile_bytes);
+    const uint32_t base = a.first_ptr[job];
+    auto pointers = [&](int first, const char* (&p)[CH]) {
+#pragma unroll
+      for (int k = 0; k < CH; ++k) {
+        const uint32_t j = base + (uint32_t)(first + k);
+        p[k] = (const char*)a.ptr[j < (uint32_t)kManyPointers ? j : (uint32_t)kManyPointers - 1]; // unused past the job's last source
+      }
+    };
+    auto early_pointers = [&](auto first, const char* (&p)[CH]) { pointers(decltype(first)::value, p); };
+    reduce_tile_from<T, F, U, CH, PREMUL ? kPremul : kPlain>(early_pointers, pointers, (const char*)a.dst[job], (int)a.nsrc[job],
+        a.mode, a.scale, tile_byte, n);
+    tile += a.tile_waves;
+  } while (tile < a.total_tiles);
+}
+
+// One job of a list, as the host hands it over: sources already in fold order.
+struct ManyJob {
+  const void* const* src;
+  int nsrc;
+  void* dst;
+  uint64_t numel;
+};
+
+template<typename T, int F, bool PREMUL>
+int launch_many_one(const ManyArgs& a, int unroll, hipStream_t stream) {
+  const int chunk = unroll >= 16 ? 1 : 16 / unroll > 8 ? 8 : 16 / unroll;
+  dim3 g(a.edge_wgs + a.tile_waves), b(kWave);
+#define MDH_LAUNCH_MANY(UU, CC)                                                            \
+  if (unroll == UU && chunk == CC) {                                                       \
+    hipLaunchKernelGGL((reduce_many_kernel<T, F, UU, CC, PREMUL>), g, b, 0, stream, a);    \
+    return check_launch("reduce_many_kernel");                                             \
+  }
+  MDH_LAUNCH_MANY(16, 1)
+  MDH_LAUNCH_MANY(8, 2)
+  MDH_LAUNCH_MANY(4, 4)
+  MDH_LAUNCH_MANY(2, 8)
+  MDH_LAUNCH_MANY(1, 8)
+#undef MDH_LAUNCH_MANY
+  set_error("reduce_many: no kernel for %d sub-tiles", unroll);
+  return MDH_EINVAL;
+}
+
+// Packs the jobs into as few launches as the tables allow (kManyJobs jobs, kManyPointers source
+// pointers each) and enqueues them.  The tile is the longest of 16, 8, 4, 2, 1 KiB that leaves
+// the launch about a thousand tiles (a wave per SIMD), as for a single reduction.
+template<typename T, int F, bool PREMUL>
+int launch_many_typed(const ManyJob* jobs, int njobs, int mode, float scale, hipStream_t stream) {
+  using elem_t = typename Traits<T>::elem_t;
+  constexpr uint64_t kPerVec = 16 / sizeof(elem_t);
+  int at = 0;
+  while (at < njobs) {
+    // how many jobs this launch takes
+    int end = at, pointers = 0;
+    uint64_t vectors = 0;
+    while (end < njobs && end - at < kManyJobs && pointers + jobs[end].nsrc <= kManyPointers) {
+      pointers += jobs[end].nsrc;
+      vectors += jobs[end].numel / kPerVec;
+      ++end;
+    }
+    int u = 16;
+    while (u > 1 && vectors / ((uint64_t)kWave * u) < 1024) {
+      u >>= 1;
+    }
+    if (tuning().reduce_unroll) {
+      u = tuning().reduce_unroll;
+    }
+    ManyArgs a{};
+    const uint64_t tile_vecs = (uint64_t)kWave * u;
+    uint64_t tiles = 0;
+    uint32_t p = 0;
+    for (int k = 0; k < kManyJobs; ++k) {
+      a.tile_end[k] = 0xffffffffu;
+    }
+    for (int j = at; j < end; ++j) {
+      const ManyJob& job = jobs[j];
+      const int k = j - at;
+      const uint64_t nvec = job.numel / kPerVec;
+      a.first_ptr[k] = (uint16_t)p;
+      for (int q = 0; q < job.nsrc; ++q) {
+        a.ptr[p++] = job.src[q];
+      }
+      a.dst[k] = job.dst;
+      a.nvec[k] = (uint32_t)nvec;
+      a.nsrc[k] = (uint8_t)job.nsrc;
+      a.tail[k] = (uint8_t)(job.numel - nvec * kPerVec);
+      tiles += (nvec + tile_vecs - 1) / tile_vecs;
+      a.tile_end[k] = (uint32_t)tiles;
+    }
+    a.njobs = (uint32_t)(end - at);
+    a.total_tiles = (uint32_t)tiles;
+    // up to two tiles per SIMD a wave per tile, beyond that 1024 waves walk the tiles
+    a.tile_waves = (uint32_t)(tiles >= 2048 ? 1024 : tiles);
+    if (tuning().reduce_max_blocks > 0 && a.tile_waves > (uint32_t)tuning().reduce_max_blocks) {
+      a.tile_waves = (uint32_t)tuning().reduce_max_blocks;
+    }
+    a.edge_wgs = (a.njobs * kManyTailSlots + kWave - 1) / kWave;
+    a.scale = scale;
+    a.mode = mode;
+    const int rc = launch_many_one<T, F, PREMUL>(a, u, stream);
+    if (rc != MDH_OK) {
+      return rc;
+    }
+    at = end;
+  }
+  return MDH_OK;
+}
+
+template<typename T, int F>
+int launch_many(const ManyJob* jobs, int njobs, int mode, float scale, hipStream_t stream) {
+  if constexpr (F == kSum && (std::is_floating_point_v<T> || sizeof(typename Traits<T>::elem_t) == 2)) {
+    if (mode == kPremul) {
+      return launch_many_typed<T, F, true>(jobs, njobs, mode, scale, stream);
+    }
+  }
+  return launch_many_typed<T, F, false>(jobs, njobs, mode, scale, stream);
+}
+
 // One entry per (element type, fold), each instantiated in its own object
 // file (reduce_inst.hip compiled once per pair) so they build in parallel.
-#define MDH_REDUCE_ENTRY(tname, fname) \
-  int reduce_launch_##tname##_##fname(const ReduceArgs& a, hipStream_t stream)
+#define MDH_REDUCE_ENTRY(tname, fname)                                                  \
+  int reduce_launch_##tname##_##fname(const ReduceArgs& a, hipStream_t stream);         \
+  int reduce_many_launch_##tname##_##fname(const ManyJob* jobs, int njobs, int mode, float scale, hipStream_t stream)
 #define MDH_REDUCE_ENTRIES(tname) \
   MDH_REDUCE_ENTRY(tname, sum);   \
   MDH_REDUCE_ENTRY(tname, min);   \

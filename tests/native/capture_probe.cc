@@ -4,6 +4,8 @@
 // nodes are read back with hipGraphKernelNodeGetParams and their grid, block, LDS size and
 // kernel-argument bytes are compared with mdh_copy_plan_step_arguments.  The graph is destroyed
 // without being instantiated: NOTHING IS REPLAYED and no kernel of this program runs.
+// The library refuses a capturing stream (MDH_ECAPTURE): that is checked first, on every case,
+// and only then does the program set the knob "allow_capture", which exists for this comparison.
 //   capture_probe.bin <path to libmoodist_hip.so>
 // Built by __graft_entry__.build() with hipcc; run by tests/test_gpu_copy.py.
 #include <hip/hip_runtime.h>
@@ -51,7 +53,8 @@ int main(int argc, char** argv) {
   auto plan_args = (decltype(&mdh_copy_plan_step_arguments))dlsym(lib, "mdh_copy_plan_step_arguments");
   auto plan_destroy = (decltype(&mdh_copy_plan_destroy))dlsym(lib, "mdh_copy_plan_destroy");
   auto last_error = (decltype(&mdh_last_error))dlsym(lib, "mdh_last_error");
-  if (!plan_create || !plan_launch || !plan_launches || !plan_args || !plan_destroy || !last_error) {
+  auto set_tuning = (decltype(&mdh_set_tuning))dlsym(lib, "mdh_set_tuning");
+  if (!plan_create || !plan_launch || !plan_launches || !plan_args || !plan_destroy || !last_error || !set_tuning) {
     std::printf("missing symbol\n");
     return 2;
   }
@@ -124,7 +127,30 @@ int main(int argc, char** argv) {
     bases[P] = out;
     const int launches = plan_launches(plan);
 
+    // what every caller gets: the launch is refused, the capture goes on undisturbed and ends
+    // with an empty graph
     hipGraph_t graph = nullptr;
+    if (set_tuning("allow_capture", 0) != MDH_OK) {
+      std::printf("set_tuning: %s\n", last_error());
+      return 1;
+    }
+    CK(hipStreamBeginCapture(stream, hipStreamCaptureModeRelaxed));
+    const int refused = plan_launch(plan, bases.data(), P + 1, stream);
+    CK(hipStreamEndCapture(stream, &graph));
+    size_t refused_nodes = 0;
+    CK(hipGraphGetNodes(graph, nullptr, &refused_nodes));
+    CK(hipGraphDestroy(graph));
+    graph = nullptr;
+    if (refused != MDH_ECAPTURE || refused_nodes != 0 || !std::strstr(last_error(), "being captured")) {
+      std::printf("%s: a launch on a capturing stream returned %d and recorded %zu node(s): %s\n", c.name, refused,
+          refused_nodes, last_error());
+      return 1;
+    }
+    std::printf("%-42s refused on a capturing stream, nothing recorded\n", c.name);
+    if (set_tuning("allow_capture", 1) != MDH_OK) {
+      std::printf("set_tuning: %s\n", last_error());
+      return 1;
+    }
     CK(hipStreamBeginCapture(stream, hipStreamCaptureModeRelaxed));
     const int rc = plan_launch(plan, bases.data(), P + 1, stream);
     CK(hipStreamEndCapture(stream, &graph));

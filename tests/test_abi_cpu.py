@@ -65,6 +65,12 @@ def test_box_struct_layout_matches_header():
     # the box into 2^24 pieces
     (lambda: abi.copy_boxes([abi.make_box(16, 1 << 40, [4096, 4096, 2, 2, 2, 1], [2 ** 22, 2 ** 10, 64, 16, 4, 1],
                                           [2 ** 24, 2 ** 11, 128, 32, 8, 1])], 1), "more than 1048576 pieces"),
+    (lambda: abi.reduce_many([([16], 0, 32, 4), ([16, 48], 2, 64, 4)], abi.DTYPE_FLOAT32, abi.OP_SUM), r"first 2 outside 0..1 \(job 1\)"),
+    (lambda: abi.reduce_many([([16], 0, 32, 4), ([0], 0, 64, 4)], abi.DTYPE_FLOAT32, abi.OP_SUM), r"source 0 is null \(job 1\)"),
+    (lambda: abi.reduce_many([([16], 0, 32, 4)], 11, abi.OP_SUM), "Unsupported dtype"),
+    (lambda: abi.reduce_many([([16], 0, 32, 4)], abi.DTYPE_INT32, abi.OP_AVG), "Unsupported reduce operation"),
+    (lambda: abi.reduce_many([([16] * 65, 0, 32, 4)], abi.DTYPE_FLOAT32, abi.OP_SUM), "nsrc 65 outside"),
+    (lambda: abi.reduce_many([([64], 0, 68, 4)], abi.DTYPE_FLOAT32, abi.OP_SUM), "partially overlaps"),
     (lambda: abi.set_tuning("reduce_wg_per_cu", 10), "does not take 10"),
     (lambda: abi.set_tuning("no_such_knob", 1), "unknown knob"),
     (lambda: abi.set_tuning("reduce_unroll", 3), "does not take 3"),
@@ -77,6 +83,8 @@ def test_bad_arguments_are_refused_before_launch(call, match):
 
 def test_empty_work_is_a_no_op_without_a_device():
     abi.reduce([16], 0, 32, 0, abi.DTYPE_FLOAT32, abi.OP_SUM)  # numel == 0
+    abi.reduce_many([], abi.DTYPE_FLOAT32, abi.OP_SUM)
+    abi.reduce_many([([16], 0, 32, 0), ([16, 48], 1, 64, 0)], abi.DTYPE_BFLOAT16, abi.OP_MAX)
     abi.gather([16], 1024, 0, 1, 0, 0, 0)
     abi.gather([], 1024, 8, 1, 8, 8, 8)
     abi.copy_boxes([], 4)
@@ -122,3 +130,5 @@ def test_launch_without_a_device_is_an_error_not_a_crash():
         abi.reduce([4096, 8192], 0, 16384, 64, abi.DTYPE_FLOAT32, abi.OP_SUM)
     with pytest.raises(abi.MoodistError, match="launch failed"):
         abi.gather([4096], 16384, 64, 1, 64, 64, 64)
+    with pytest.raises(abi.MoodistError, match="launch failed"):
+        abi.reduce_many([([4096, 8192], 0, 16384, 64), ([4096], 0, 32768, 3)], abi.DTYPE_FLOAT32, abi.OP_SUM)

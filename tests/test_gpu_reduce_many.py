@@ -1,0 +1,116 @@
+"""Parity of a LIST of reductions in shared launches (mdh_reduce_many) against the CPU oracle, job
+by job, through the C ABI.  Same bar as for a single reduction: bit-exact with the oracle for
+every dtype and op (the oracle's 16-bit rule is fp32 accumulation, one rounding)."""
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from moodist_amd import _abi as abi
+from util import ALL_DTYPES, TORCH_TO_CODE, bits, random_sources, same_bits
+
+pytestmark = pytest.mark.gpu
+
+
+def scale_for(op, P):
+    return float(np.float32(1.0) / np.float32(P)) if op == oracle.OP_AVG else float(np.float32(0.37))
+
+
+def run_jobs(dev, dtype, op, specs, scale, offsets=None):
+    """specs: (P, n, first) per job.  Builds seeded sources, runs all jobs in one call and returns
+    [(out bits, oracle bits, spec)].  offsets: per job, element offset of every operand inside a
+    larger allocation (misalignment)."""
+    st = torch.cuda.current_stream().cuda_stream
+    jobs, keep, results = [], [], []
+    for k, (P, n, first) in enumerate(specs):
+        off = 0 if offsets is None else offsets[k]
+        srcs = random_sources(P, n, dtype, seed=1000 * k + 31 * P + n)
+        dev_full = [torch.zeros(n + off + 64, dtype=dtype, device=dev) for _ in range(P)]
+        for f, s in zip(dev_full, srcs):
+            f[off:off + n].copy_(s)
+        out_full = torch.full((n + off + 64,), 77, dtype=dtype, device=dev)
+        keep.append((dev_full, out_full))
+        isz = out_full.element_size()
+        jobs.append(([f.data_ptr() + off * isz for f in dev_full], first, out_full.data_ptr() + off * isz, n))
+        want = oracle.reduce([bits(s) for s in srcs], first, TORCH_TO_CODE[dtype], op, scale) if n else None
+        results.append((out_full, off, n, want, (P, n, first)))
+    abi.reduce_many(jobs, TORCH_TO_CODE[dtype], op, scale, st)
+    torch.cuda.synchronize()
+    for out_full, off, n, want, spec in results:
+        if n:
+            assert same_bits(bits(out_full[off:off + n]), want), (dtype, op, spec)
+        # nothing outside the job's elements was written
+        guard = torch.full((1,), 77, dtype=dtype)
+        assert torch.equal(out_full[:off].cpu(), guard.expand(off)), spec
+        assert torch.equal(out_full[off + n:].cpu(), guard.expand(64)), spec
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES, ids=str)
+def test_ragged_sizes_mixed_source_counts_all_ops(dev, dtype):
+    # sizes of the reference's stress test (tests/test_stress.py:241) plus tails, one element, an
+    # empty job; 1 to 64 sources in one list (more than one launch's pointer table holds)
+    specs = [(8, 1, 3), (3, 7, 0), (8, 64, 7), (1, 255, 0), (16, 1031, 5), (8, 4096 + 5, 2), (64, 70001, 63), (2, 0, 1),
+             (7, 65536, 6), (33, 12345, 17), (8, 300000 + 3, 1), (9, 2, 8), (64, 513, 0), (64, 31, 40), (64, 8, 1),
+             (17, 100000, 16)]
+    for op in (oracle.OP_SUM, oracle.OP_MIN, oracle.OP_MAX, oracle.OP_AVG, oracle.OP_PREMUL_SUM):
+        if op in (oracle.OP_AVG, oracle.OP_PREMUL_SUM) and not dtype.is_floating_point:
+            continue
+        run_jobs(dev, dtype, op, specs, scale_for(op, 8))
+
+
+def test_more_jobs_than_one_launch_holds(dev):
+    # 130 jobs of 8 sources: four launches of at most 40 jobs
+    rng = np.random.RandomState(5)
+    specs = [(8, int(rng.randint(1, 9000)), int(rng.randint(0, 8))) for _ in range(130)]
+    run_jobs(dev, torch.float32, oracle.OP_SUM, specs, 1.0)
+    run_jobs(dev, torch.bfloat16, oracle.OP_AVG, specs, scale_for(oracle.OP_AVG, 8))
+
+
+def test_operands_off_every_grid(dev):
+    # element offsets 0..15 of every operand inside its allocation: vectors start wherever the job starts
+    specs = [(8, 5000 + k, k % 8) for k in range(16)]
+    for dtype in (torch.float32, torch.bfloat16, torch.float64):
+        run_jobs(dev, dtype, oracle.OP_SUM, specs, 1.0, offsets=list(range(16)))
+
+
+def test_a_long_job_in_the_list_gets_its_own_launch(dev):
+    # 8 MiB per source and more leaves the shared launches; results are the same either way
+    n_big = (8 << 20) // 4 + 3
+    specs = [(4, 1000, 1), (4, n_big, 2), (4, 77, 0), (4, (1 << 20) + 1, 3)]
+    run_jobs(dev, torch.float32, oracle.OP_SUM, specs, 1.0)
+    run_jobs(dev, torch.float32, oracle.OP_MAX, specs, 1.0)
+
+
+@pytest.mark.parametrize("unroll", [1, 2, 4, 8, 16])
+@pytest.mark.parametrize("max_blocks", [0, 3])
+def test_every_tile_length_and_a_grid_that_walks(dev, unroll, max_blocks):
+    old = abi.get_tuning("reduce_unroll"), abi.get_tuning("reduce_max_blocks")
+    try:
+        abi.set_tuning("reduce_unroll", unroll)
+        abi.set_tuning("reduce_max_blocks", max_blocks)
+        specs = [(8, 40000 + 3, 1), (5, 12345, 4), (16, 65536, 0), (2, 17, 1), (8, 4096, 7)]
+        for dtype in (torch.float32, torch.bfloat16, torch.int64):
+            run_jobs(dev, dtype, oracle.OP_SUM, specs, 1.0)
+    finally:
+        abi.set_tuning("reduce_unroll", old[0])
+        abi.set_tuning("reduce_max_blocks", old[1])
+
+
+def test_in_place_jobs_and_equality_with_single_launches(dev):
+    # dst == srcs[first] (what an in-place allreduce passes), and the same bits as mdh_reduce job by job
+    st = torch.cuda.current_stream().cuda_stream
+    P = 8
+    sizes = [257, 4096, 100003, 1]
+    for dtype in (torch.float32, torch.float16):
+        sets = [[s.to(dev) for s in random_sources(P, n, dtype, seed=n)] for n in sizes]
+        singles = []
+        for k, srcs in enumerate(sets):
+            out = torch.zeros(sizes[k], dtype=dtype, device=dev)
+            abi.reduce([s.data_ptr() for s in srcs], k % P, out.data_ptr(), sizes[k], TORCH_TO_CODE[dtype], oracle.OP_SUM, 1.0, st)
+            singles.append(out)
+        jobs = [([s.data_ptr() for s in srcs], k % P, srcs[k % P].data_ptr(), sizes[k]) for k, srcs in enumerate(sets)]
+        abi.reduce_many(jobs, TORCH_TO_CODE[dtype], oracle.OP_SUM, 1.0, st)
+        torch.cuda.synchronize()
+        for k, srcs in enumerate(sets):
+            assert same_bits(bits(srcs[k % P]), bits(singles[k])), (dtype, k)
