@@ -18,6 +18,7 @@ not in the 256 MB Infinity Cache either.  Prints one JSON line.
     gather:<sources>:<bytes per shard>
     rows:<boxes>:<rows per box>:<run bytes>:<source pitch bytes>    strided rows into a dense destination
     transpose:<rows>:<cols>:<itemsize>                              2-D element transpose
+    coalesced:<tensors>:<elements>[:loop]                           allreduce_coalesced of eight local ranks
 """
 
 import argparse
@@ -270,6 +271,54 @@ def build_workload(name, torch, abi, dev, rotation_bytes):
                 # enqueued behind a long blocker kernel so that the GPU runs them back to back
                 "queue_prefilled": True}
         return desc, set_bytes, launch, check, box_kernel(abi)
+
+    if name.startswith("coalesced:"):
+        # coalesced:<tensors>:<elements>[:loop] -- allreduce_coalesced (MAX, fp32, in place) of a list of
+        # tensors of about that many elements each, called by all eight ranks of a local group: what
+        # a DDP or ZeRO bucket of many small tensors costs, host and GPU together.  With ":loop", one
+        # allreduce per tensor instead, as the reference serves the call
+        # (wrapper/processgroup_wrapper.cc:182-191).
+        import torch.distributed as dist
+
+        import moodist_amd
+
+        parts = name.split(":")
+        T, n = int(parts[1]), int(parts[2])
+        loop = len(parts) > 3 and parts[3] == "loop"
+        P = 8
+        world = moodist_amd.LocalWorld(P, dev)
+        sizes = [n + 8 * k for k in range(T)]  # multiples of the group size when n is
+        g = torch.Generator().manual_seed(4)
+        host = [[torch.rand(m, generator=g) for m in sizes] for _ in range(P)]
+        tensors = [[t.to(dev) for t in row] for row in host]
+        opts = dist.AllreduceCoalescedOptions()
+        opts.reduceOp = dist.ReduceOp.MAX  # idempotent: the launches can repeat on the same tensors
+        one = dist.AllreduceOptions()
+        one.reduceOp = dist.ReduceOp.MAX
+        set_bytes = sum(P * ((P + 1) * m // P + 2 * m * (P - 1) // P) * 4 for m in sizes)
+
+        def launch(i):
+            if loop:
+                for k in range(T):
+                    for r in range(P):
+                        world.groups[r].allreduce([tensors[r][k]], one)
+            else:
+                for r in range(P):
+                    world.groups[r].allreduce_coalesced(tensors[r], opts)
+
+        def check():
+            for k in range(T):
+                want = host[0][k]
+                for r in range(1, P):
+                    want = torch.maximum(want, host[r][k])
+                for r in range(P):
+                    if not torch.equal(tensors[r][k].cpu(), want):
+                        raise SystemExit("bench: result differs from the expected allreduce")
+
+        desc = {"workload": name, "op": "allreduce_coalesced MAX, eight local ranks" + (", one allreduce per tensor" if loop else ""),
+                "tensors": T, "numel": n, "dtype": "float32", "buffer_sets": 1,
+                "note": "a step is all eight ranks' calls; ms_per_step is host and GPU together"}
+        return desc, set_bytes, launch, check, "reduce_many_kernel + copy_flat_kernel"
 
     if name.startswith("rows:"):
         # rows:<boxes>:<rows per box>:<run bytes>:<source pitch bytes> -- every box is `rows` runs of

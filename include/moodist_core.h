@@ -47,6 +47,11 @@ extern "C" {
 /* api/moodist_version.h:12 (kMoodistApiVersion) */
 #define MOODIST_CORE_API_VERSION 2
 
+/* The number this library's build drew (build_host.sh), the same one its API table carries in
+ * `magic` (api/moodist_api.h:265-271): readable before the table is asked for.  No counterpart
+ * in the reference, where only the table holds it. */
+uint64_t moodist_build_magic(void);
+
 typedef struct moodist_tensor {
   void* data;         /* device pointer */
   int64_t numel;
@@ -109,6 +114,14 @@ int moodist_pg_all_gather_many(moodist_pg* pg, const moodist_tensor* outputs, co
  * reduce_op is a c10d RedOpType number; premul_value is used by PREMUL_SUM only. */
 int moodist_pg_reduce_scatter(moodist_pg* pg, const moodist_tensor* output, const moodist_tensor* input,
     int reduce_op, void* stream, float premul_value, moodist_work** work);
+/* c10d's reduce_scatter_tensor_coalesced, which the reference serves with one reduce_scatter per
+ * tensor (wrapper/processgroup_wrapper.cc:159-170), as ONE collective: outputs[t] receives this
+ * rank's chunk of every rank's inputs[t], reduced; a rank's reductions share kernel launches
+ * (mdh_reduce_many).  All tensors must have one element type; every rank must bring lists of the
+ * same length and sizes.  `outputs` may be NULL for a rank that only contributes.  The whole
+ * list is checked before anything is posted. */
+int moodist_pg_reduce_scatter_many(moodist_pg* pg, const moodist_tensor* outputs, const moodist_tensor* inputs, size_t n,
+    int reduce_op, void* stream, float premul_value, moodist_work** work);
 /* processGroupAllreduce (api/processgroup_api.h:48-49; core/processgroup.cc:1674-1722): a
  * reduce-scatter into the rank's own chunk followed by an all-gather, in place.  When numel
  * is not a multiple of the group size the reference allocates a padded temporary through
@@ -117,11 +130,12 @@ int moodist_pg_reduce_scatter(moodist_pg* pg, const moodist_tensor* output, cons
 int moodist_pg_allreduce(moodist_pg* pg, const moodist_tensor* tensor, const moodist_tensor* scratch, int reduce_op,
     void* stream, float premul_value, moodist_work** work);
 /* c10d's allreduce_coalesced (wrapper/processgroup_wrapper.cc:182-191), which the reference serves
- * with one allreduce per tensor, for tensors whose element counts the group size divides (the
- * others go through moodist_pg_allreduce one by one): a reduce_scatter per tensor into the
- * rank's own chunk, in place, then ONE all_gather of every tensor's chunks
- * (moodist_pg_all_gather_many).  `*work` is the last collective; the earlier ones have been
- * launched when it has. */
+ * with one allreduce per tensor, for tensors of one element type whose element counts the group
+ * size divides (the others go through moodist_pg_allreduce one by one): ONE reduce_scatter of
+ * the list into the rank's own chunks, in place (moodist_pg_reduce_scatter_many), then ONE
+ * all_gather of every tensor's chunks (moodist_pg_all_gather_many).  `*work` is the gather; the
+ * reduce_scatter has been launched when it has.  A list that is refused (mixed element types,
+ * an operation the type does not support) leaves nothing posted. */
 int moodist_pg_allreduce_many(moodist_pg* pg, const moodist_tensor* tensors, size_t n, int reduce_op, void* stream,
     float premul_value, moodist_work** work);
 /* No counterpart in the reference.  moodist_pg_allreduce for callers that cannot allocate

@@ -179,6 +179,14 @@ typedef struct mdh_box {
  * tensor to or from contiguous staging (core/cputhread.h:306-310).  A box with
  * both sides strided is the fused form Copy -> Read -> Copy, so no staging
  * buffer exists.  Destination boxes must not overlap each other or any source.
+ *
+ * A box may transpose: its source contiguous along one dimension, its destination along
+ * another (out[c][r] = in[r][c]).  The reference's planner never produces one (source and
+ * destination boxes of a redistribution share a dimension order,
+ * core/processgroup.cc:2848-2870); here such a box, when both dimensions are at least 16
+ * elements long, is copied in tiles of 64 x 64 (32 x 32 for 8- and 16-byte elements) that are
+ * read along the source's contiguous dimension, turned round in LDS and written along the
+ * destination's, so that both sides move whole cache lines.
  */
 int mdh_copy_boxes(const mdh_box* boxes, int nboxes, int itemsize, void* stream);
 
@@ -252,7 +260,9 @@ int mdh_static_workspace(void** address, size_t* bytes);
  * "copy_max_blocks", "copy_wg_per_cu" (2..8, 9 = never cap), "box_policy" (loads of the
  * strided-box kernel: 1 = plain, which pays when the sources are still in the Infinity Cache;
  * 0 or 2 = nt, the default), "box_preload" (1 = never start equal boxes of full tiles from
- * preloaded kernel arguments), four variants of the dense copy of up to eight equal segments that
+ * preloaded kernel arguments), "box_transpose" (1 = boxes that transpose take the plain strided
+ * kernel instead of LDS-staged tiles), "box_tile_cols" (a power of two: the columns, in 16-byte vectors, of
+ * a strided-box tile; its rows follow from the tile's 256 x box_unroll slots), four variants of the dense copy of up to eight equal segments that
  * exist for measurement and that the library never chooses by itself -- "copy_xcd_run" (2, 4, 8, ...:
  * each of the eight XCDs takes runs of that many consecutive tiles, where by default adjacent tiles
  * go to different XCDs), "copy_grid_order" (1: the segments advance together instead of one after

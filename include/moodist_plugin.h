@@ -44,8 +44,10 @@ struct ihipStream_t;
 
 namespace moodist {
 
-/* api/moodist_version.h:12; the build magic is a per-build random number there
- * (CMakeLists.txt:97-106), here a constant of this source tree. */
+/* api/moodist_version.h:12.  The build magic is a random number drawn once per build and
+ * compiled into both libraries, there by CMake (CMakeLists.txt:97-106), here by
+ * moodist_amd/csrc/build_host.sh; the constant below only serves a translation unit compiled on
+ * its own (a test driver), which then checks against a core built the same way. */
 constexpr uint32_t kMoodistApiVersion = 2;
 #ifndef MOODIST_BUILD_MAGIC
 #define MOODIST_BUILD_MAGIC 0x4d49333535584d44ULL /* "MI355XMD" */

@@ -13,6 +13,8 @@ from ._abi import MoodistError  # noqa: F401
 from .compile import compile_op  # noqa: F401
 from .options import MoodistOptions, MoodistOptionsContext  # noqa: F401
 from .process_group import (LocalWorld, MoodistProcessGroup, PreferKernelLessContext,  # noqa: F401
-                            find_process_group)
+                            create_moodist_backend, find_process_group, register_backend)
+
+register_backend()  # torch.distributed.init_process_group(backend="moodist", ...) from here on
 
 __version__ = "0.1.0"

@@ -145,6 +145,16 @@ int moodist_pg_all_gather_many(moodist_pg* pg, const moodist_tensor* outputs, co
   });
 }
 
+int moodist_pg_reduce_scatter_many(moodist_pg* pg, const moodist_tensor* outputs, const moodist_tensor* inputs, size_t n,
+    int reduce_op, void* stream, float premul_value, moodist_work** work) {
+  return guarded([&] {
+    if (!inputs) {
+      throw std::runtime_error("moodist: null tensor");
+    }
+    give(work, as_pg(pg)->reduce_scatter_many(outputs, inputs, n, reduce_op, stream, premul_value));
+  });
+}
+
 int moodist_pg_allreduce_many(moodist_pg* pg, const moodist_tensor* tensors, size_t n, int reduce_op, void* stream,
     float premul_value, moodist_work** work) {
   return guarded([&] {

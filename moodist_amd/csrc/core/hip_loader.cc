@@ -80,6 +80,7 @@ HipRuntime load() {
   resolve(kl, kn, "mdh_last_error", r.last_error);
   resolve(kl, kn, "mdh_error_string", r.error_string);
   resolve(kl, kn, "mdh_reduce", r.reduce);
+  resolve(kl, kn, "mdh_reduce_many", r.reduce_many);
   resolve(kl, kn, "mdh_gather", r.gather);
   resolve(kl, kn, "mdh_copy_boxes", r.copy_boxes);
   resolve(kl, kn, "mdh_copy_plan_create", r.copy_plan_create);

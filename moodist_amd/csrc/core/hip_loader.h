@@ -39,6 +39,7 @@ struct HipRuntime {
   decltype(&mdh_last_error) last_error;
   decltype(&mdh_error_string) error_string;
   decltype(&mdh_reduce) reduce;
+  decltype(&mdh_reduce_many) reduce_many;
   decltype(&mdh_gather) gather;
   decltype(&mdh_copy_boxes) copy_boxes;
   decltype(&mdh_copy_plan_create) copy_plan_create;

@@ -405,6 +405,10 @@ moodist::CoreApi* moodistGetApi(uint32_t expectedVersion, const moodist::Wrapper
   return &moodist::g_table;
 }
 
+uint64_t moodist_build_magic(void) {
+  return moodist::kMoodistBuildMagic;
+}
+
 moodist_pg* moodistGroupCHandle(moodist::api::ProcessGroup* group) {
   return group ? reinterpret_cast<moodist_pg*>(static_cast<moodist::GroupObject*>(group)->pg) : nullptr;
 }

@@ -85,6 +85,18 @@ void check_reduce_op(int op) {
   }
 }
 
+// AVG and PREMUL_SUM are defined for floating element types only (core/processgroup.cc:1315-1316,
+// :1340-1344: a multiply by 1/size or by the factor)
+void check_reduce_request(int dtype, int reduce_op) {
+  check_reduce_dtype(dtype);
+  check_reduce_op(reduce_op);
+  const bool floating = dtype == MDH_DTYPE_FLOAT32 || dtype == MDH_DTYPE_FLOAT64 || dtype == MDH_DTYPE_BFLOAT16 ||
+                        dtype == MDH_DTYPE_FLOAT16;
+  if ((reduce_op == MDH_OP_AVG || reduce_op == MDH_OP_PREMUL_SUM) && !floating) {
+    throw std::runtime_error("Unsupported reduce operation");
+  }
+}
+
 void check_device_tensor(const moodist_tensor& t, int device, const char* what) {
   if (!t.contiguous) {
     throw std::runtime_error(std::string("moodist: ") + what + " must be contiguous");
@@ -177,10 +189,24 @@ void ProcessGroup::set_option(const std::string& name, int64_t value) {
   } else if (name == "force_kernel_less") {
     options.forceKernelLess = value != 0;
   } else if (name == "num_chunks") {
+    if (value < -1 || value == 0 || value > 65535) {
+      throw std::runtime_error("moodist: num_chunks takes -1 (auto) or 1..65535, not " + std::to_string(value));
+    }
     options.numChunks = value;
   } else if (name == "chunk_size") {
+    if (value < -1 || value == 0) {
+      throw std::runtime_error("moodist: chunk_size takes -1 (auto) or a number of bytes, not " + std::to_string(value));
+    }
     options.chunkSize = value;
   } else if (name == "method") {
+    // -1 = auto, 0 = kernel, 1 = copy, 2 = direct (core/processgroup.cc:339)
+    if (value == 1) {
+      throw std::runtime_error("moodist: method 1 (copy) stages peers' chunks through the copy engine before reducing "
+                               "them; the ranks of a local group are read in place, by method 0 (kernel) or 2 (direct)");
+    }
+    if (value < -1 || value > 2) {
+      throw std::runtime_error("moodist: method takes -1 (auto), 0 (kernel) or 2 (direct), not " + std::to_string(value));
+    }
     options.method = value;
   } else if (name == "snapshot_inputs") {
     if (value != 0 && !world->allocator.alloc) {
@@ -311,22 +337,12 @@ std::shared_ptr<Collective> ProcessGroup::reduce_scatter(const moodist_tensor* o
   Busy guard(*this);
   refuse_capture_early(stream, "reduce_scatter");
   check_device_tensor(input, world->device, "reduce_scatter input");
-  check_reduce_dtype(input.dtype);
-  check_reduce_op(reduce_op);
-  const bool floating = input.dtype == MDH_DTYPE_FLOAT32 || input.dtype == MDH_DTYPE_FLOAT64 ||
-                        input.dtype == MDH_DTYPE_BFLOAT16 || input.dtype == MDH_DTYPE_FLOAT16;
-  if ((reduce_op == MDH_OP_AVG || reduce_op == MDH_OP_PREMUL_SUM) && !floating) {
-    throw std::runtime_error("Unsupported reduce operation");
-  }
+  check_reduce_request(input.dtype, reduce_op);
   const size_t in_bytes = bytes_of(input);
   MD_CHECK(in_bytes > 0 && in_bytes % (size_t)size == 0);
   const size_t bytes = in_bytes / (size_t)size;
   MD_CHECK(bytes % (size_t)input.itemsize == 0);
   Posting p;
-  p.input = input;
-  snapshot(p.input, stream, keep);
-  p.keep = std::move(keep);
-  p.stream = stream;
   if (output) {
     check_device_tensor(*output, world->device, "reduce_scatter output");
     MD_CHECK(output->dtype == input.dtype);   // core/processgroup.cc:1312
@@ -334,14 +350,92 @@ std::shared_ptr<Collective> ProcessGroup::reduce_scatter(const moodist_tensor* o
     p.output = *output;
     p.wants_output = true;
   }
+  p.input = input;
+  snapshot(p.input, stream, keep);
+  p.keep = std::move(keep);
+  p.stream = stream;
+  p.chunk_bytes = chunk_bytes_for(bytes);
   return last = world->post(Kind::reduce_scatter, next_seq++, rank, std::move(p), reduce_op, premul, bytes,
              input.dtype, 0, nullptr);
+}
+
+// num_chunks / chunk_size / method (core/processgroup.cc:334-340).  The reference cuts the chunk
+// a rank reduces for another node into pieces (its "direct" method: per destination and piece,
+// send = own (+) peers, core/reduce_scatter_direct.cc:165-177), with
+//   numChunks = clamp(bytes / 131072, 1, 4);  chunkSize = roundup(ceil(bytes / numChunks), 4096);
+//   numChunks = ceil(bytes / chunkSize)                                   (core/processgroup.cc:1494-1503)
+// and stores the three options without reading them.  Here they are honoured: chunk_size (bytes,
+// rounded up to 4096) or else num_chunks (through the arithmetic above) cut a reduce_scatter's
+// reduction into pieces, and method 2 ("direct") asks for the reference's own piece count when
+// neither is set.  Pieces shorter than 8 MiB share launches (mdh_reduce_many).
+size_t ProcessGroup::chunk_bytes_for(size_t bytes) const {
+  size_t chunk = 0;
+  if (options.chunkSize > 0) {
+    chunk = ((size_t)options.chunkSize + 4095u) / 4096u * 4096u;
+  } else {
+    size_t pieces = 0;
+    if (options.numChunks > 0) {
+      pieces = (size_t)options.numChunks;
+    } else if (options.method == 2) {
+      pieces = bytes / 131072 < 4 ? bytes / 131072 : 4;
+    }
+    if (pieces > 1) {
+      chunk = ((bytes + pieces - 1) / pieces + 4095u) / 4096u * 4096u;
+    }
+  }
+  return chunk >= bytes ? 0 : chunk;
+}
+
+// reduce_scatter_tensor_coalesced (wrapper/processgroup_wrapper.cc:159-170).  The reference loops
+// over the tensors, one collective and one kernel launch per rank each; here the list is one
+// collective and a rank's reductions share launches (mdh_reduce_many).  The whole list is
+// checked before anything is posted.
+std::shared_ptr<Collective> ProcessGroup::reduce_scatter_many(const moodist_tensor* outputs,
+    const moodist_tensor* inputs, size_t n, int reduce_op, void* stream, float premul, Keep keep) {
+  Busy guard(*this);
+  refuse_capture_early(stream, "reduce_scatter");
+  if (n == 0 || n > 0xffffu) {
+    throw std::runtime_error("moodist: a coalesced reduce_scatter takes 1..65535 tensors, not " + std::to_string(n));
+  }
+  size_t total = 0;
+  for (size_t t = 0; t < n; ++t) {
+    check_device_tensor(inputs[t], world->device, "reduce_scatter input");
+    check_reduce_request(inputs[t].dtype, reduce_op);
+    if (inputs[t].dtype != inputs[0].dtype) {
+      throw std::runtime_error("moodist: the tensors of a coalesced reduce_scatter must have one element type");
+    }
+    const size_t in_bytes = bytes_of(inputs[t]);
+    MD_CHECK(in_bytes > 0 && in_bytes % (size_t)size == 0);
+    const size_t bytes = in_bytes / (size_t)size;
+    MD_CHECK(bytes % (size_t)inputs[t].itemsize == 0);
+    if (outputs) {
+      check_device_tensor(outputs[t], world->device, "reduce_scatter output");
+      MD_CHECK(outputs[t].dtype == inputs[t].dtype); // core/processgroup.cc:1312
+      MD_CHECK(bytes_of(outputs[t]) == bytes);       // :1325
+    }
+    total += bytes;
+  }
+  Posting p;
+  for (size_t t = 0; t < n; ++t) {
+    moodist_tensor in = inputs[t];
+    snapshot(in, stream, keep);
+    p.inputs.push_back(in);
+    if (outputs) {
+      p.outputs.push_back(outputs[t]);
+    }
+  }
+  p.wants_output = outputs != nullptr;
+  p.keep = std::move(keep);
+  p.stream = stream;
+  return last = world->post(Kind::reduce_scatter_many, next_seq++, rank, std::move(p), reduce_op, premul, total,
+             inputs[0].dtype, (uint32_t)n, nullptr);
 }
 
 std::shared_ptr<Collective> ProcessGroup::allreduce(const moodist_tensor& tensor, const moodist_tensor* scratch,
     int reduce_op, void* stream, float premul, Keep keep) {
   check_device_tensor(tensor, world->device, "allreduce tensor");
   MD_CHECK(tensor.numel > 0); // core/processgroup.cc:1678
+  check_reduce_request(tensor.dtype, reduce_op); // before anything is enqueued or posted
   const int64_t n = tensor.numel;
   if (n % size == 0) {
     // in place: reduce into this rank's own chunk, then gather every rank's chunk (:1686-1693)
@@ -395,17 +489,23 @@ std::shared_ptr<Collective> ProcessGroup::allreduce(const moodist_tensor& tensor
 
 // allreduce_coalesced (wrapper/processgroup_wrapper.cc:182-191), for the tensors of the list that
 // need no padding: the reference runs one allreduce -- a reduce_scatter and an all_gather -- per
-// tensor; here the reductions are followed by one gather of every tensor's chunks.
+// tensor; here one reduce_scatter of the whole list (its reductions share launches) is followed
+// by one gather of every tensor's chunks.
 std::shared_ptr<Collective> ProcessGroup::allreduce_many(const moodist_tensor* tensors, size_t n, int reduce_op,
     void* stream, float premul, Keep keep) {
   if (n == 0 || n > 0xffffu) {
     throw std::runtime_error("moodist: a coalesced allreduce takes 1..65535 tensors, not " + std::to_string(n));
   }
   std::vector<moodist_tensor> chunks(n);
+  // the whole list is checked before anything is posted: a list that is refused leaves nothing
+  // pending and the rank's sequence where it was
   for (size_t t = 0; t < n; ++t) {
     check_device_tensor(tensors[t], world->device, "allreduce tensor");
     MD_CHECK(tensors[t].numel > 0 && tensors[t].numel % size == 0);
-    check_reduce_dtype(tensors[t].dtype); // before anything of the list is posted
+    check_reduce_request(tensors[t].dtype, reduce_op);
+    if (tensors[t].dtype != tensors[0].dtype) {
+      throw std::runtime_error("moodist: the tensors of a coalesced allreduce must have one element type");
+    }
   }
   for (size_t t = 0; t < n; ++t) {
     moodist_tensor& chunk = chunks[t];
@@ -414,8 +514,8 @@ std::shared_ptr<Collective> ProcessGroup::allreduce_many(const moodist_tensor* t
     chunk.data = (char*)tensors[t].data + (size_t)rank * (size_t)chunk.numel * (size_t)tensors[t].itemsize;
     chunk.ndim = 1;
     chunk.shape[0] = chunk.numel;
-    reduce_scatter(&chunk, tensors[t], reduce_op, stream, premul, keep);
   }
+  reduce_scatter_many(chunks.data(), tensors, n, reduce_op, stream, premul, keep); // both halves hold the tensors
   // the gather's inputs are what the reductions will have written by then: never snapshots
   internal_input = true;
   struct Reset {
@@ -784,7 +884,7 @@ void World::order_streams_after(Collective& c) {
 }
 
 void World::launch(Collective& c, const std::shared_ptr<CompiledOp>& op) {
-  if (c.kind == Kind::all_gather_many) {
+  if (c.kind == Kind::all_gather_many || c.kind == Kind::reduce_scatter_many) {
     // the ranks agreed on the number of tensors and their total size (post); now tensor by tensor
     const size_t n = c.post[0].inputs.size();
     for (int j = 0; j < size; ++j) {
@@ -822,6 +922,7 @@ void World::launch(Collective& c, const std::shared_ptr<CompiledOp>& op) {
       c.kind == Kind::reduce_scatter    ? "reduce_scatter"
       : c.kind == Kind::all_gather      ? "all_gather"
       : c.kind == Kind::all_gather_many ? "all_gather of a list"
+      : c.kind == Kind::reduce_scatter_many ? "reduce_scatter of a list"
                                         : "custom op",
       size, c.bytes, c.dtype);
 
@@ -841,7 +942,54 @@ void World::launch(Collective& c, const std::shared_ptr<CompiledOp>& op) {
       for (int j = 0; j < size; ++j) {
         srcs[(size_t)j] = (const char*)c.post[(size_t)j].input.data + c.bytes * (size_t)q;
       }
-      check_mdh(h.reduce(srcs.data(), size, q, pq.output.data, numel, c.dtype, c.reduce_op, scale, pq.stream));
+      if (pq.chunk_bytes == 0) {
+        check_mdh(h.reduce(srcs.data(), size, q, pq.output.data, numel, c.dtype, c.reduce_op, scale, pq.stream));
+        continue;
+      }
+      // in pieces (the options num_chunks / chunk_size / method of the rank that asks): piece k
+      // covers bytes [k * chunk, min(bytes, (k + 1) * chunk)) of every source and of the output
+      const size_t chunk = pq.chunk_bytes / itemsize * itemsize;
+      const size_t pieces = (c.bytes + chunk - 1) / chunk;
+      std::vector<const void*> tables(pieces * (size_t)size);
+      std::vector<mdh_reduce_job> jobs(pieces);
+      for (size_t k = 0; k < pieces; ++k) {
+        const size_t at = k * chunk;
+        for (int j = 0; j < size; ++j) {
+          tables[k * (size_t)size + (size_t)j] = (const char*)srcs[(size_t)j] + at;
+        }
+        jobs[k].srcs = tables.data() + k * (size_t)size;
+        jobs[k].nsrc = size;
+        jobs[k].first = q;
+        jobs[k].dst = (char*)pq.output.data + at;
+        jobs[k].numel = ((at + chunk < c.bytes ? chunk : c.bytes - at)) / itemsize;
+      }
+      check_mdh(h.reduce_many(jobs.data(), (int)pieces, c.dtype, c.reduce_op, scale, pq.stream));
+    }
+  } else if (c.kind == Kind::reduce_scatter_many) {
+    // out_q[t] = in_q[t][q] (+) in_{q+1}[t][q] (+) ... for every tensor t: one job per tensor, the
+    // jobs of a rank in shared launches
+    const size_t itemsize = dtype_size(c.dtype);
+    const size_t n = c.post[0].inputs.size();
+    const float scale = c.reduce_op == MDH_OP_AVG ? 1.0f / (float)size : c.premul;
+    std::vector<const void*> tables(n * (size_t)size);
+    std::vector<mdh_reduce_job> jobs(n);
+    for (int q = 0; q < size; ++q) {
+      const Posting& pq = c.post[(size_t)q];
+      if (!pq.wants_output) {
+        continue;
+      }
+      for (size_t t = 0; t < n; ++t) {
+        const size_t bytes = bytes_of(pq.inputs[t]) / (size_t)size;
+        for (int j = 0; j < size; ++j) {
+          tables[t * (size_t)size + (size_t)j] = (const char*)c.post[(size_t)j].inputs[t].data + bytes * (size_t)q;
+        }
+        jobs[t].srcs = tables.data() + t * (size_t)size;
+        jobs[t].nsrc = size;
+        jobs[t].first = q;
+        jobs[t].dst = pq.outputs[t].data;
+        jobs[t].numel = bytes / itemsize;
+      }
+      check_mdh(h.reduce_many(jobs.data(), (int)n, c.dtype, c.reduce_op, scale, pq.stream));
     }
   } else if (c.kind == Kind::all_gather) {
     // out_q[pitch*j .. +bytes] = in_j for every j (core/allgather.cc:381-390)

@@ -22,7 +22,7 @@ namespace moodist {
 
 class World;
 
-enum class Kind : int { all_gather = 0, reduce_scatter = 1, custom = 2, all_gather_many = 3 };
+enum class Kind : int { all_gather = 0, reduce_scatter = 1, custom = 2, all_gather_many = 3, reduce_scatter_many = 4 };
 
 // What one rank brought to a collective.
 struct Posting {
@@ -30,8 +30,10 @@ struct Posting {
   bool wants_output = false;
   moodist_tensor input{};
   moodist_tensor output{};
-  std::vector<moodist_tensor> inputs;  // custom op; all_gather of a list of tensors
-  std::vector<moodist_tensor> outputs; // custom op; all_gather into one tensor per rank, or of a list of tensors
+  std::vector<moodist_tensor> inputs;  // custom op; all_gather or reduce_scatter of a list of tensors
+  std::vector<moodist_tensor> outputs; // custom op; all_gather into one tensor per rank; all_gather or reduce_scatter of a list
+  // reduce_scatter: the rank's chunk is reduced in pieces of this many bytes (0 = in one piece)
+  size_t chunk_bytes = 0;
   bool kernel_less = false;   // this rank asked for the copy-engine form of all_gather
   bool has_copy_back = false; // allreduce through a padded temporary
   moodist_tensor copy_back{};
@@ -115,10 +117,14 @@ public:
       void* stream, Keep keep = {});
   std::shared_ptr<Collective> reduce_scatter(const moodist_tensor* output, const moodist_tensor& input, int reduce_op,
       void* stream, float premul, Keep keep = {});
+  // n reduce_scatters as one collective: outputs[t] receives this rank's chunk of every rank's
+  // inputs[t], reduced (outputs may be null for a rank that only contributes); one element type
+  std::shared_ptr<Collective> reduce_scatter_many(const moodist_tensor* outputs, const moodist_tensor* inputs, size_t n,
+      int reduce_op, void* stream, float premul, Keep keep = {});
   std::shared_ptr<Collective> allreduce(const moodist_tensor& tensor, const moodist_tensor* scratch, int reduce_op,
       void* stream, float premul, Keep keep = {});
-  // n in-place allreduces whose element counts the group size divides: one reduce_scatter each,
-  // then ONE gather of all the chunks
+  // n in-place allreduces of one element type whose element counts the group size divides: ONE
+  // reduce_scatter of the list into the rank's own chunks, then ONE gather of all the chunks
   std::shared_ptr<Collective> allreduce_many(const moodist_tensor* tensors, size_t n, int reduce_op, void* stream,
       float premul, Keep keep = {});
   // allreduce whose padded temporary is this rank's slice of the kernel library's fixed
@@ -145,6 +151,8 @@ private:
   // snapshot_inputs: replaces input.data by a copy made now on `stream`; the copy joins `keep`
   void snapshot(moodist_tensor& input, void* stream, Keep& keep);
   bool internal_input = false; // the second half of an allreduce: its input does not exist yet
+  // the pieces a reduce_scatter's chunk of `bytes` is reduced in, from the options (0 = one piece)
+  size_t chunk_bytes_for(size_t bytes) const;
   std::weak_ptr<Collective> static_user; // the last collective that reads this rank's workspace slice
 
   // "Concurrent use of process group detected" guard (core/processgroup.cc:172-183)

@@ -116,6 +116,12 @@ int* knob(const char* name) {
   if (!std::strcmp(name, "box_preload")) {
     return &t.box_preload;
   }
+  if (!std::strcmp(name, "box_transpose")) {
+    return &t.box_transpose;
+  }
+  if (!std::strcmp(name, "box_tile_cols")) {
+    return &t.box_tile_cols;
+  }
   if (!std::strcmp(name, "copy_max_blocks")) {
     return &t.copy_max_blocks;
   }
@@ -151,8 +157,13 @@ extern "C" int mdh_set_tuning(const char* name, int value) {
       mdh::set_error("mdh_set_tuning: %s does not take %d", name, value);
       return MDH_EINVAL;
     }
+  } else if (!std::strcmp(name, "box_tile_cols") || !std::strcmp(name, "copy_xcd_run")) {
+    if (value < 0 || (value & (value - 1)) != 0 || value > 2048) {
+      mdh::set_error("mdh_set_tuning: %s takes a power of two up to 2048, not %d", name, value);
+      return MDH_EINVAL;
+    }
   } else if (value < 0 || (std::strstr(name, "wg_per_cu") && value > 9) || (!std::strcmp(name, "box_policy") && value > 2) ||
-             (!std::strcmp(name, "box_preload") && value > 1) || (!std::strcmp(name, "allow_capture") && value > 1)) {
+             (!std::strcmp(name, "box_preload") && value > 1) || (!std::strcmp(name, "box_transpose") && value > 1) || (!std::strcmp(name, "allow_capture") && value > 1)) {
     mdh::set_error("mdh_set_tuning: %s does not take %d", name, value);
     return MDH_EINVAL;
   }

@@ -12,6 +12,7 @@
 // paid once per tile, never per vector.  Runs shorter than a wave's 1 KiB still
 // coalesce: consecutive lanes walk a run, then step to the next row.
 #include "device_common.h"
+#include "transpose_kernels.h"
 
 #include <algorithm>
 #include <cstring>
@@ -622,7 +623,7 @@ int vec_width(const HostBox& h) {
 // One kernel launch of a copy, with everything but the base addresses decided: what a
 // prepared plan replays.
 struct Step {
-  enum Kind { kFlat, kBoxes16, kBoxes } kind;
+  enum Kind { kFlat, kBoxes16, kBoxes, kTrans } kind;
   int vec;    // kBoxes: bytes per vector
   int unroll; // sub-tiles
   uint32_t grid;
@@ -636,9 +637,12 @@ struct Step {
   size_t lds;
   FlatArgs flat;   // kFlat
   CopyArgs boxes;  // kBoxes16, kBoxes
+  TransArgs trans; // kTrans: vec is the element size, plain_loads unused
+  bool wide = false; // kTrans: 16-byte global accesses
 };
 
-int launch_step(const Step& st, const FlatArgs* flat, const CopyArgs* boxes, hipStream_t stream);
+int launch_step(const Step& st, const FlatArgs* flat, const CopyArgs* boxes, hipStream_t stream,
+    const TransArgs* trans = nullptr);
 
 // Whether a launch of equal boxes qualifies for copy_rows16_kernel: at most eight boxes, one
 // strided extent, the same shape on the source side, rows a whole number of vectors, and no
@@ -740,7 +744,9 @@ inline bool make_flat_lead(const FlatArgs& a, FlatLead* lead, uint32_t opts = 0)
 // The grid a step is launched with: st.grid (x st.grid_y) tile workgroups, and in the
 // one-dimensional form of a flat step the edge workgroups in front of them.
 inline void launch_dims(const Step& st, uint32_t* x, uint32_t* y) {
-  if (st.variant != 0) {
+  if (st.kind == Step::kTrans) {
+    *x = st.grid, *y = 1;
+  } else if (st.variant != 0) {
     *x = st.variant_grid_x, *y = st.variant_grid_y;
   } else if (st.grid_y > 0) {
     *x = st.grid + (st.edge_column ? 1u : 0u);
@@ -763,6 +769,7 @@ struct Launcher {
     uint8_t head, tail;
   };
   std::vector<Segment> flat; // contiguous runs: whole vectors plus head and tail bytes
+  std::vector<TransBox> transposing[5][2]; // by log2(element size) and whether global accesses are 16 bytes wide
   int rc = MDH_OK;
   int unroll = 2; // sub-tiles of the box launch being assembled
 
@@ -952,17 +959,19 @@ struct Launcher {
   }
 
   // Enqueues the step now, or files it for a plan.
-  void submit(Step& st, const FlatArgs* f, const CopyArgs* c) {
+  void submit(Step& st, const FlatArgs* f, const CopyArgs* c, const TransArgs* x = nullptr) {
     if (record) {
       if (f) {
         st.flat = *f;
-      } else {
+      } else if (c) {
         st.boxes = *c;
+      } else {
+        st.trans = *x;
       }
       record->push_back(st);
       return;
     }
-    const int r = launch_step(st, f, c, stream);
+    const int r = launch_step(st, f, c, stream, x);
     if (r != MDH_OK) {
       rc = r;
     }
@@ -1009,18 +1018,31 @@ struct Launcher {
       bool equal = true;
       while (i < list.size() && a.nboxes < (uint32_t)kMaxBoxes) {
         BoxDesc d = list[i];
-        // Tile width: the power of two that covers the row, or the tile -- unless the column
-        // tiles of that width would be more than a sixteenth empty (a row of 513 vectors in tiles
-        // of 512 columns is two tiles, the second with one column in use: a gather of rows of
-        // 8200 bytes took 114 us, against 80 us for rows of 8192); then the widest that is not,
-        // down to 16 columns (256 bytes of a row per wave instruction) if the rows are many.
+        // Tile width: the power of two that covers the row, up to 64 columns -- 1 KiB, what one
+        // wave moves with one instruction, so that the four waves of a workgroup work on four rows
+        // rather than on 4 KiB of one: rows of 2 KiB at a pitch of 16 KiB (bf16 8192^2 over 8
+        // ranks) 7.45 -> 7.14 us, rows of 4 KiB at 32 KiB 11.77 -> 11.55 us, rows of 8 KiB into a
+        // padded pitch level (80.7 / 81.0 us); rows of a power-of-two pitch map to few DRAM
+        // channels at a time (the same rows at a pitch 256 bytes longer: 12.96 -> 12.18 us), and a
+        // workgroup spread over more rows evens that out.  Unless the column tiles of that width
+        // would be more than a sixteenth empty (a row of 513 vectors in tiles of 512 columns is
+        // two tiles, the second with one column in use: a gather of rows of 8200 bytes took
+        // 114 us, against 80 us for rows of 8192); then the widest that is not, down to 16
+        // columns (256 bytes of a row per wave instruction) if the rows are many.
+        constexpr uint32_t kWidestTile = 64;
         uint32_t tc = 1, log2tc = 0;
-        while (tc < d.cols && tc < slots) {
+        while (tc < d.cols && tc < slots && tc < kWidestTile) {
           tc <<= 1, ++log2tc;
         }
         while (tc > 16 && (slots >> (log2tc - 1)) <= d.rows &&
                (uint64_t)((d.cols + tc - 1) / tc) * tc * 16 > (uint64_t)d.cols * 17) {
           tc >>= 1, --log2tc;
+        }
+        if (const uint32_t forced = (uint32_t)tuning().box_tile_cols; forced != 0 && forced <= slots) {
+          tc = 1, log2tc = 0; // (measurement knob, a power of two: checked when it is set)
+          while (tc < forced) {
+            tc <<= 1, ++log2tc;
+          }
         }
         const uint32_t tr = slots >> log2tc;
         d.log2tc = log2tc;
@@ -1056,11 +1078,112 @@ struct Launcher {
     list.clear();
   }
 
+  void flush_transposing() {
+    for (int lg = 0; lg < 5; ++lg) {
+      for (int wide = 0; wide < 2; ++wide) {
+        std::vector<TransBox>& list = transposing[lg][wide];
+        size_t i = 0;
+        while (i < list.size()) {
+          TransArgs a{};
+          uint64_t tiles = 0;
+          for (int k = 0; k < kMaxTransBoxes; ++k) {
+            a.tile_end[k] = 0xffffffffu;
+          }
+          while (i < list.size() && a.nboxes < (uint32_t)kMaxTransBoxes) {
+            const TransBox& b = list[i];
+            const uint64_t n = (uint64_t)b.ta * b.tb * b.no[0] * b.no[1];
+            if (tiles + n > 0x7fffffffull) {
+              if (a.nboxes == 0) {
+                set_error("copy: one transposing box needs %llu tiles, more than a grid can index", (unsigned long long)n);
+                rc = MDH_EINVAL;
+                return;
+              }
+              break;
+            }
+            tiles += n;
+            a.tile_end[a.nboxes] = (uint32_t)tiles;
+            a.box[a.nboxes++] = b;
+            ++i;
+          }
+          a.total_tiles = (uint32_t)tiles;
+          Step st;
+          st.kind = Step::kTrans, st.vec = 1 << lg, st.unroll = 1, st.grid = a.total_tiles, st.grid_y = 0, st.lds = 0;
+          st.plain_loads = false, st.wide = wide != 0;
+          submit(st, nullptr, nullptr, &a);
+        }
+        list.clear();
+      }
+    }
+  }
+
   void flush() {
     flush_flat();
+    flush_transposing();
     for (int lg = 5; lg >= 0; --lg) {
       flush_class(lg);
     }
+  }
+
+  // A box whose contiguous run is one element and whose source is contiguous along one extent
+  // (A), its destination along another (B): copied tile by tile through LDS (transpose_kernel),
+  // so that both sides move consecutive bytes.  Both extents must be at least kMinTransExtent
+  // long (below that a tile would be mostly empty, and the plain kernel, which then still
+  // coalesces on one side, is no worse), and at most two other extents may remain.
+  static constexpr int64_t kMinTransExtent = 16;
+
+  bool try_transposing(const HostBox& h) {
+    if (tuning().box_transpose == 1 || h.nd < 2 || h.nd > 2 + kTransBatchDims || h.run > 16 || (h.run & (h.run - 1)) != 0) {
+      return false;
+    }
+    int A = -1, B = -1;
+    for (int d = 0; d < h.nd; ++d) {
+      if (A < 0 && h.sstride[d] == h.run && h.dstride[d] != h.run) {
+        A = d;
+      } else if (B < 0 && h.dstride[d] == h.run && h.sstride[d] != h.run) {
+        B = d;
+      }
+    }
+    if (A < 0 || B < 0 || h.shape[A] < kMinTransExtent || h.shape[B] < kMinTransExtent) {
+      return false;
+    }
+    const uint32_t E = (uint32_t)h.run;
+    TransBox b{};
+    b.src = h.src, b.dst = h.dst;
+    b.src_b = h.sstride[B], b.dst_a = h.dstride[A];
+    b.na = (uint32_t)h.shape[A], b.nb = (uint32_t)h.shape[B];
+    if ((int64_t)b.na != h.shape[A] || (int64_t)b.nb != h.shape[B]) {
+      return false;
+    }
+    b.no[0] = b.no[1] = 1;
+    int k = 0;
+    for (int d = h.nd - 1; d >= 0; --d) { // fastest first
+      if (d == A || d == B) {
+        continue;
+      }
+      if (h.shape[d] > 0x7fffffff) {
+        return false;
+      }
+      b.no[k] = (uint32_t)h.shape[d];
+      b.src_o[k] = h.sstride[d];
+      b.dst_o[k] = h.dstride[d];
+      ++k;
+    }
+    const uint32_t T = trans_tile(E);
+    b.ta = (b.na + T - 1) / T, b.tb = (b.nb + T - 1) / T;
+    const uint64_t align = (uint64_t)(uintptr_t)b.src | (uint64_t)(uintptr_t)b.dst | (uint64_t)b.src_b | (uint64_t)b.dst_a |
+                           (uint64_t)b.src_o[0] | (uint64_t)b.src_o[1] | (uint64_t)b.dst_o[0] | (uint64_t)b.dst_o[1] |
+                           (uint64_t)b.na * E | (uint64_t)b.nb * E;
+    const bool wide = (align & 15) == 0 && E < 16;
+    if (!count_piece()) {
+      return true;
+    }
+    int lg = 0;
+    while ((1u << lg) < E) {
+      ++lg;
+    }
+    // (an element of 16 bytes is a vector already: the element-wise form moves 16 bytes per lane)
+    transposing[lg][wide ? 1 : 0].push_back(b);
+    return true;
   }
 
   // A box the kernels cannot index (more than kMaxOuter strided extents, or more than 2^31
@@ -1164,6 +1287,9 @@ struct Launcher {
         return;
       }
       emit(h);
+      return;
+    }
+    if (try_transposing(h)) {
       return;
     }
     uint64_t rows = 1;
@@ -1272,7 +1398,37 @@ void launch_boxes_vec(const Step& st, const CopyArgs& a, hipStream_t stream) {
   }
 }
 
-int launch_step(const Step& st, const FlatArgs* flat, const CopyArgs* boxes, hipStream_t stream) {
+template<int E>
+void launch_transposing(const Step& st, const TransArgs& a, hipStream_t stream) {
+  dim3 g(st.grid), b(kBlock);
+  if (st.wide) {
+    hipLaunchKernelGGL((transpose_kernel<E, true>), g, b, 0, stream, a);
+  } else {
+    hipLaunchKernelGGL((transpose_kernel<E, false>), g, b, 0, stream, a);
+  }
+}
+
+int launch_step(const Step& st, const FlatArgs* flat, const CopyArgs* boxes, hipStream_t stream, const TransArgs* trans) {
+  if (st.kind == Step::kTrans) {
+    switch (st.vec) {
+    case 1:
+      launch_transposing<1>(st, *trans, stream);
+      break;
+    case 2:
+      launch_transposing<2>(st, *trans, stream);
+      break;
+    case 4:
+      launch_transposing<4>(st, *trans, stream);
+      break;
+    case 8:
+      launch_transposing<8>(st, *trans, stream);
+      break;
+    default:
+      launch_transposing<16>(st, *trans, stream);
+      break;
+    }
+    return check_launch("transpose_kernel");
+  }
   const bool equal = st.grid_y > 0;
   uint32_t gx, gy;
   launch_dims(st, &gx, &gy);
@@ -1592,13 +1748,16 @@ extern "C" int mdh_copy_plan_create(const mdh_box* boxes, const int32_t* src_slo
   };
   for (size_t s = 0; s < p->steps.size(); ++s) {
     Step& st = p->steps[s];
-    const uint32_t n = st.kind == Step::kFlat ? st.flat.nsegs : st.boxes.nboxes;
+    const uint32_t n = st.kind == Step::kFlat ? st.flat.nsegs : st.kind == Step::kTrans ? st.trans.nboxes : st.boxes.nboxes;
     for (uint32_t k = 0; k < n; ++k) {
       Patch pa;
       pa.step = (uint32_t)s, pa.entry = k;
       if (st.kind == Step::kFlat) {
         split(st.flat.src[k], &pa.src_slot, &pa.src_off);
         split(st.flat.dst[k], &pa.dst_slot, &pa.dst_off);
+      } else if (st.kind == Step::kTrans) {
+        split(st.trans.box[k].src, &pa.src_slot, &pa.src_off);
+        split(st.trans.box[k].dst, &pa.dst_slot, &pa.dst_off);
       } else {
         split(st.boxes.box[k].src, &pa.src_slot, &pa.src_off);
         split(st.boxes.box[k].dst, &pa.dst_slot, &pa.dst_off);
@@ -1701,6 +1860,47 @@ extern "C" int mdh_copy_plan_verify(const mdh_copy_plan* plan, const uint64_t* b
   };
   for (size_t s = 0; s < plan->steps.size(); ++s) {
     const Step& st = plan->steps[s];
+    if (st.kind == Step::kTrans) {
+      // one tile per workgroup, every element of every tile through the kernel's own index function
+      const TransArgs& a = st.trans;
+      const uint32_t E = (uint32_t)st.vec, T = trans_tile(E);
+      if (st.grid != a.total_tiles || a.nboxes == 0 || a.nboxes > (uint32_t)kMaxTransBoxes) {
+        set_error("mdh_copy_plan_verify: step %zu has a grid of %u workgroups for %u tiles", s, st.grid, a.total_tiles);
+        return MDH_EINVAL;
+      }
+      for (uint32_t tile = 0; tile < a.total_tiles; ++tile) {
+        const TransLoc t = trans_locate(a, tile, E);
+        if (t.box >= a.nboxes) {
+          set_error("mdh_copy_plan_verify: step %zu tile %u lands in box %u of %u", s, tile, t.box, a.nboxes);
+          return MDH_EINVAL;
+        }
+        const TransBox& B = a.box[t.box];
+        if (t.ia >= B.na || t.ib >= B.nb) {
+          set_error("mdh_copy_plan_verify: step %zu tile %u starts outside its box", s, tile);
+          return MDH_EINVAL;
+        }
+        int ss, ds;
+        uint64_t sbase, dbase;
+        split(B.src, &ss, &sbase);
+        split(B.dst, &ds, &dbase);
+        const uint32_t na = B.na - t.ia < T ? B.na - t.ia : T, nb = B.nb - t.ib < T ? B.nb - t.ib : T;
+        if (st.wide && ((na * E) % 16 != 0 || (nb * E) % 16 != 0 || ((sbase + (uint64_t)t.src_off) & 15) != 0 ||
+                           ((dbase + (uint64_t)t.dst_off) & 15) != 0 || (B.src_b & 15) != 0 || (B.dst_a & 15) != 0)) {
+          set_error("mdh_copy_plan_verify: step %zu box %u: 16-byte accesses do not fit this box", s, t.box);
+          return MDH_EINVAL;
+        }
+        for (uint32_t ib = 0; ib < nb; ++ib) {
+          for (uint32_t ia = 0; ia < na; ++ia) {
+            const int64_t so = t.src_off + (int64_t)ib * B.src_b + (int64_t)ia * E;
+            const int64_t dof = t.dst_off + (int64_t)ia * B.dst_a + (int64_t)ib * E;
+            if (!move(ss, sbase + (uint64_t)so, ds, dbase + (uint64_t)dof, E, s)) {
+              return MDH_EINVAL;
+            }
+          }
+        }
+      }
+      continue;
+    }
     // every workgroup takes its first tile untested: the grid must not exceed the tile count
     const uint32_t step_tiles = st.kind == Step::kFlat ? st.flat.total_tiles : st.boxes.total_tiles;
     if (st.grid == 0 || st.grid > step_tiles) {
@@ -1874,7 +2074,7 @@ extern "C" int mdh_copy_plan_launches(const mdh_copy_plan* plan) {
 // Writes the caller's addresses into a copy of launch `s`'s argument block; `at` is the first
 // patch of that launch, the return value the first patch of the next.
 static size_t patch_step(const mdh_copy_plan& plan, size_t s, size_t at, const void* const* bases, mdh::FlatArgs* flat,
-    mdh::CopyArgs* boxes) {
+    mdh::CopyArgs* boxes, mdh::TransArgs* trans = nullptr) {
   for (; at < plan.patches.size() && plan.patches[at].step == s; ++at) {
     const mdh::Patch& pa = plan.patches[at];
     const char* src = (const char*)bases[pa.src_slot] + pa.src_off;
@@ -1882,9 +2082,12 @@ static size_t patch_step(const mdh_copy_plan& plan, size_t s, size_t at, const v
     if (flat) {
       flat->src[pa.entry] = src;
       flat->dst[pa.entry] = dst;
-    } else {
+    } else if (boxes) {
       boxes->box[pa.entry].src = src;
       boxes->box[pa.entry].dst = dst;
+    } else {
+      trans->box[pa.entry].src = src;
+      trans->box[pa.entry].dst = dst;
     }
   }
   return at;
@@ -1928,6 +2131,10 @@ extern "C" int mdh_copy_plan_launch(const mdh_copy_plan* plan, const void* const
       FlatArgs a = st.flat;
       at = patch_step(*plan, s, at, bases, &a, nullptr);
       rc = launch_step(st, &a, nullptr, (hipStream_t)stream);
+    } else if (st.kind == Step::kTrans) {
+      TransArgs a = st.trans;
+      at = patch_step(*plan, s, at, bases, nullptr, nullptr, &a);
+      rc = launch_step(st, nullptr, nullptr, (hipStream_t)stream, &a);
     } else {
       CopyArgs a = st.boxes;
       at = patch_step(*plan, s, at, bases, nullptr, &a);
@@ -1963,6 +2170,7 @@ extern "C" int mdh_copy_plan_step_arguments(const mdh_copy_plan* plan, const voi
   }
   FlatArgs flat;
   CopyArgs boxes;
+  TransArgs trans;
   union {
     RowsLead rows;
     FlatLead flat;
@@ -1970,7 +2178,12 @@ extern "C" int mdh_copy_plan_step_arguments(const mdh_copy_plan* plan, const voi
   static_assert(sizeof(RowsLead) == sizeof(FlatLead), "one size of leading arguments");
   size_t lead_bytes = 0;
   const void* from;
-  if (st.kind == Step::kFlat) {
+  if (st.kind == Step::kTrans) {
+    trans = st.trans;
+    patch_step(*plan, (size_t)step, at, bases, nullptr, nullptr, &trans);
+    from = &trans;
+    *size = sizeof(TransArgs);
+  } else if (st.kind == Step::kFlat) {
     flat = st.flat;
     patch_step(*plan, (size_t)step, at, bases, &flat, nullptr);
     from = &flat;

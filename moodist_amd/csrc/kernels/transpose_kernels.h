@@ -1,0 +1,201 @@
+// LDS-staged tiles for boxes that TRANSPOSE: the dimension along which the source is contiguous
+// (A) is not the one along which the destination is (B).  Copied vector by vector along either
+// side, such a box coalesces on that side only and moves one element per lane and memory
+// transaction on the other (a 4096 x 4096 fp32 transpose: 107 us, 16 % of the HBM rate).  Here a
+// workgroup takes a tile of T x T elements, reads it along A -- consecutive lanes, consecutive
+// source bytes --, turns it round in LDS and writes it along B -- consecutive lanes, consecutive
+// destination bytes: both sides move whole 64-byte units.
+//
+// The reference has no such copy: its planner gives source and destination boxes of a
+// redistribution one dimension order (core/processgroup.cc:2848-2870), so a compiled custom op
+// never transposes, and its Copy is an {offset, shape} box of a contiguous tensor
+// (core/cputhread.h:306-310).  mdh_copy_boxes takes any strides, transposing ones included.
+#pragma once
+#include "device_common.h"
+
+namespace mdh {
+
+#ifndef MDH_HD
+#define MDH_HD __host__ __device__ __forceinline__
+#endif
+
+constexpr int kMaxTransBoxes = 16;
+constexpr int kTransBatchDims = 2;
+
+struct TransBox {
+  const char* src;
+  char* dst;
+  int64_t src_b; // source bytes between neighbours along B (along A: the element size)
+  int64_t dst_a; // destination bytes between neighbours along A (along B: the element size)
+  int64_t src_o[kTransBatchDims]; // the other extents, fastest first
+  int64_t dst_o[kTransBatchDims];
+  uint32_t na, nb; // elements along A and B
+  uint32_t no[kTransBatchDims];
+  uint32_t ta, tb; // tiles along A and B
+};
+
+struct TransArgs {
+  TransBox box[kMaxTransBoxes];
+  uint32_t tile_end[kMaxTransBoxes]; // cumulative tiles; unused entries are ~0
+  uint32_t nboxes;
+  uint32_t total_tiles;
+};
+static_assert(sizeof(TransArgs) + 256 <= 4096, "kernel arguments are limited to 4 KiB");
+
+// Elements along a tile's edge: 64 for elements of up to 4 bytes, 32 for 8 and 16 (tiles of
+// 4-16 KiB).
+MDH_HD constexpr uint32_t trans_tile(uint32_t elem) {
+  return elem <= 4 ? 64u : 32u;
+}
+
+struct TransLoc {
+  uint32_t box;
+  uint32_t ia, ib; // the tile's first element along A and B
+  int64_t src_off, dst_off; // of that element, from the box's src and dst
+};
+
+// Which box a tile belongs to and where it starts: the cumulative ends ascend, the last one at
+// or below the tile names the box (scalar selects on the device); inside a box the tiles run
+// along A first, then B, then the other extents.  Shared by the kernel and by the host-side
+// check of a prepared plan.
+MDH_HD TransLoc trans_locate(const TransArgs& a, uint32_t tile, uint32_t elem) {
+  uint32_t b = 0, start = 0;
+#pragma unroll
+  for (int k = 0; k < kMaxTransBoxes - 1; ++k) {
+    const uint32_t e = a.tile_end[k];
+    b = tile >= e ? (uint32_t)(k + 1) : b;
+    start = tile >= e ? e : start;
+  }
+  const TransBox& B = a.box[b];
+  uint32_t local = tile - start;
+  const uint32_t T = trans_tile(elem);
+  const uint32_t ta_i = local % B.ta;
+  local /= B.ta;
+  const uint32_t tb_i = local % B.tb;
+  local /= B.tb;
+  const uint32_t o0 = local % B.no[0], o1 = local / B.no[0];
+  TransLoc t;
+  t.box = b;
+  t.ia = ta_i * T;
+  t.ib = tb_i * T;
+  t.src_off = (int64_t)o0 * B.src_o[0] + (int64_t)o1 * B.src_o[1] + (int64_t)t.ib * B.src_b + (int64_t)t.ia * (int64_t)elem;
+  t.dst_off = (int64_t)o0 * B.dst_o[0] + (int64_t)o1 * B.dst_o[1] + (int64_t)t.ia * B.dst_a + (int64_t)t.ib * (int64_t)elem;
+  return t;
+}
+
+template<int E>
+struct ElemType;
+template<>
+struct ElemType<1> {
+  using type = uint8_t;
+};
+template<>
+struct ElemType<2> {
+  using type = uint16_t;
+};
+template<>
+struct ElemType<4> {
+  using type = uint32_t;
+};
+template<>
+struct ElemType<8> {
+  using type = u32x2;
+};
+template<>
+struct ElemType<16> {
+  using type = u32x4;
+};
+
+// One tile per workgroup.  LDS holds the tile TRANSPOSED, rows along A, each row T elements
+// along B plus 16 bytes of padding (rows stay 16-byte aligned and start in different banks).
+//
+// WIDE: every row of the box starts on the 16-byte grid on both sides and holds a whole number
+// of 16-byte vectors -- the host checks addresses, strides and extents: global memory moves as
+// 16-byte vectors (V = 16 / E elements); going in, a vector's elements are scattered over V
+// rows of LDS, going out, a row of LDS is read 16 bytes at a time.  Otherwise every access is
+// one element: still consecutive lanes on consecutive addresses on both sides, E bytes each.
+template<int E, bool WIDE>
+__global__ __launch_bounds__(kBlock) void transpose_kernel(TransArgs a) {
+  using elem_t = typename ElemType<E>::type;
+  constexpr uint32_t T = trans_tile(E);
+  constexpr uint32_t kPitch = T * E + 16;
+  __shared__ __attribute__((aligned(16))) char tile[T * kPitch];
+  const TransLoc t = trans_locate(a, blockIdx.x, E);
+  const TransBox& B = a.box[t.box];
+  const char* src = B.src + t.src_off;
+  char* dst = B.dst + t.dst_off;
+  // what of the tile lies inside the box
+  const uint32_t na = B.na - t.ia < T ? B.na - t.ia : T;
+  const uint32_t nb = B.nb - t.ib < T ? B.nb - t.ib : T;
+  const int64_t src_b = B.src_b, dst_a = B.dst_a;
+  if (WIDE) {
+    constexpr uint32_t V = 16 / E;       // elements per vector
+    constexpr uint32_t kRowVecs = T / V; // vectors along a tile's edge
+    constexpr uint32_t kPerLane = T * kRowVecs / kBlock;
+    u32x4 v[kPerLane];
+#pragma unroll
+    for (uint32_t i = 0; i < kPerLane; ++i) {
+      const uint32_t idx = i * kBlock + threadIdx.x;
+      const uint32_t row_b = idx / kRowVecs, col = idx % kRowVecs;
+      v[i] = u32x4{0, 0, 0, 0};
+      if (row_b < nb && col * V < na) {
+        v[i] = stream_load((const u32x4*)(src + (int64_t)row_b * src_b + (int64_t)col * 16));
+      }
+    }
+#pragma unroll
+    for (uint32_t i = 0; i < kPerLane; ++i) {
+      const uint32_t idx = i * kBlock + threadIdx.x;
+      const uint32_t row_b = idx / kRowVecs, col = idx % kRowVecs;
+      elem_t e[V];
+      __builtin_memcpy(e, &v[i], 16);
+#pragma unroll
+      for (uint32_t k = 0; k < V; ++k) {
+        *(elem_t*)(tile + (col * V + k) * kPitch + row_b * E) = e[k];
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (uint32_t i = 0; i < kPerLane; ++i) {
+      const uint32_t idx = i * kBlock + threadIdx.x;
+      const uint32_t row_a = idx / kRowVecs, col = idx % kRowVecs;
+      if (row_a < na && col * V < nb) {
+        const u32x4 out = *(const u32x4*)(tile + row_a * kPitch + col * 16);
+        stream_store((u32x4*)(dst + (int64_t)row_a * dst_a + (int64_t)col * 16), out);
+      }
+    }
+  } else {
+    constexpr uint32_t kPerLane = T * T / kBlock;
+    // (loads in batches of eight: sixteen or more in flight per lane buy nothing here)
+    constexpr uint32_t kBatch = kPerLane < 8 ? kPerLane : 8;
+    for (uint32_t i0 = 0; i0 < kPerLane; i0 += kBatch) {
+      elem_t e[kBatch];
+#pragma unroll
+      for (uint32_t i = 0; i < kBatch; ++i) {
+        const uint32_t idx = (i0 + i) * kBlock + threadIdx.x;
+        const uint32_t row_b = idx / T, col_a = idx % T;
+        e[i] = elem_t{};
+        if (row_b < nb && col_a < na) {
+          e[i] = stream_load((const elem_t*)(src + (int64_t)row_b * src_b + (int64_t)col_a * E));
+        }
+      }
+#pragma unroll
+      for (uint32_t i = 0; i < kBatch; ++i) {
+        const uint32_t idx = (i0 + i) * kBlock + threadIdx.x;
+        const uint32_t row_b = idx / T, col_a = idx % T;
+        *(elem_t*)(tile + col_a * kPitch + row_b * E) = e[i];
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (uint32_t i = 0; i < kPerLane; ++i) {
+      const uint32_t idx = i * kBlock + threadIdx.x;
+      const uint32_t row_a = idx / T, col_b = idx % T;
+      if (row_a < na && col_b < nb) {
+        const elem_t out = *(const elem_t*)(tile + row_a * kPitch + col_b * E);
+        stream_store((elem_t*)(dst + (int64_t)row_a * dst_a + (int64_t)col_b * E), out);
+      }
+    }
+  }
+}
+
+} // namespace mdh

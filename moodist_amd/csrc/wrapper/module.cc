@@ -64,6 +64,7 @@ struct CoreExtras {
   MOODIST_EXTRA(moodist_pg_all_gather_list)
   MOODIST_EXTRA(moodist_pg_all_gather_many)
   MOODIST_EXTRA(moodist_pg_allreduce_many)
+  MOODIST_EXTRA(moodist_pg_reduce_scatter_many)
   MOODIST_EXTRA(moodist_pg_stage_input)
   MOODIST_EXTRA(moodist_pg_last_work)
   MOODIST_EXTRA(moodist_pg_keep_alive)
@@ -236,6 +237,7 @@ void load_core() {
   MOODIST_EXTRA(moodist_pg_all_gather_list)
   MOODIST_EXTRA(moodist_pg_all_gather_many)
   MOODIST_EXTRA(moodist_pg_allreduce_many)
+  MOODIST_EXTRA(moodist_pg_reduce_scatter_many)
   MOODIST_EXTRA(moodist_pg_stage_input)
   MOODIST_EXTRA(moodist_pg_last_work)
   MOODIST_EXTRA(moodist_pg_keep_alive)
@@ -439,17 +441,41 @@ public:
     return result;
   }
 
-  // wrapper/processgroup_wrapper.cc:159-170
+  // wrapper/processgroup_wrapper.cc:159-170 loops over the tensors; here a list of two or more of
+  // one element type is one collective whose reductions share launches
+  // (moodist_pg_reduce_scatter_many)
   c10::intrusive_ptr<c10d::Work> reduce_scatter_tensor_coalesced(std::vector<at::Tensor>& outputs,
       std::vector<at::Tensor>& inputs, const c10d::ReduceScatterOptions& opts = c10d::ReduceScatterOptions()) override {
     TORCH_CHECK(outputs.size() == inputs.size());
     auto result = c10::make_intrusive<WorkImpl>();
-    for (size_t k = 0; k < inputs.size(); ++k) {
-      Wrapped o(outputs[k]), i(inputs[k]);
-      core->processGroupReduceScatter(handle_.get(), o.ptr, i.ptr, reduce_op_code(opts.reduceOp),
-          stream_of(inputs[k]), premul_value(opts.reduceOp, inputs[k].scalar_type()));
-      add_last(*result);
+    bool one_type = inputs.size() >= 2;
+    for (size_t k = 1; k < inputs.size(); ++k) {
+      one_type = one_type && inputs[k].scalar_type() == inputs[0].scalar_type();
     }
+    if (!one_type) {
+      for (size_t k = 0; k < inputs.size(); ++k) {
+        Wrapped o(outputs[k]), i(inputs[k]);
+        core->processGroupReduceScatter(handle_.get(), o.ptr, i.ptr, reduce_op_code(opts.reduceOp),
+            stream_of(inputs[k]), premul_value(opts.reduceOp, inputs[k].scalar_type()));
+        add_last(*result);
+      }
+      result->tensors = outputs;
+      return result;
+    }
+    std::vector<moodist_tensor> outs, ins;
+    for (size_t k = 0; k < inputs.size(); ++k) {
+      outs.push_back(describe(outputs[k]));
+      ins.push_back(describe(inputs[k]));
+    }
+    moodist_work* w = nullptr;
+    check(extra.moodist_pg_reduce_scatter_many(c_, outs.data(), ins.data(), ins.size(),
+        static_cast<int>(reduce_op_code(opts.reduceOp)), stream_of(inputs[0]),
+        premul_value(opts.reduceOp, inputs[0].scalar_type()), &w));
+    result->parts.push_back(w);
+    auto held = new std::vector<at::Tensor>(outputs);
+    held->insert(held->end(), inputs.begin(), inputs.end());
+    // the core owns `held` from the call on and releases it exactly once, also when it fails
+    check(extra.moodist_pg_keep_alive(c_, held, release_tensors));
     result->tensors = outputs;
     return result;
   }
@@ -469,13 +495,21 @@ public:
   c10::intrusive_ptr<c10d::Work> allreduce_coalesced(std::vector<at::Tensor>& tensors,
       const c10d::AllreduceCoalescedOptions& opts = c10d::AllreduceCoalescedOptions()) override {
     auto result = c10::make_intrusive<WorkImpl>();
-    // The tensors that need no padded temporary -- same element type, element count a multiple
-    // of the group size -- are reduced one by one and gathered together
-    // (moodist_pg_allreduce_many); the others take one allreduce each, as in the reference.
-    // Every rank holds the same list, so every rank splits it the same way.
+    // The tensors that need no padded temporary -- element count a multiple of the group size,
+    // element type that of the first such tensor -- are reduced and gathered as two collectives
+    // for the whole set (moodist_pg_allreduce_many); the others take one allreduce each, as in
+    // the reference, in list order.  What decides membership is the same on every rank (sizes
+    // and element types, which the ranks' lists must share), never a property of one rank's
+    // tensor: a tensor that is not contiguous is refused before anything is posted, on every
+    // path, as the core refuses it (core/processgroup.cc:1062-1063).
+    for (at::Tensor& t : tensors) {
+      if (!t.is_contiguous()) {
+        throw std::runtime_error("moodist: allreduce tensor must be contiguous");
+      }
+    }
     std::vector<at::Tensor> together;
     for (at::Tensor& t : tensors) {
-      if (t.is_cuda() && t.is_contiguous() && t.numel() > 0 && t.numel() % getSize() == 0 &&
+      if (t.numel() > 0 && t.numel() % getSize() == 0 &&
           (together.empty() || t.scalar_type() == together[0].scalar_type())) {
         together.push_back(t);
       }

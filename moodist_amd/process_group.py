@@ -95,6 +95,23 @@ def _group_type():
     return _type
 
 
+def create_moodist_backend(store, rank, size, timeout):
+    """What ``torch.distributed`` calls to make a group of the "moodist" backend
+    (py/moodist/backend.py:71-78): the group is built the reference's way and entered into the
+    name registry.  The ranks of one local world are the groups built on one store object."""
+    return _group_type()(store, rank, size)
+
+
+def register_backend():
+    """Registers "moodist" with torch.distributed (py/moodist/backend.py:112-116), for GPU tensors
+    only: this build has no CPU path.  Importing the package does this once."""
+    import torch.distributed as dist
+
+    if not dist.is_available() or "MOODIST" in getattr(dist.Backend, "_plugins", {}):
+        return
+    dist.Backend.register_backend("moodist", create_moodist_backend, devices=("cuda",))
+
+
 def __getattr__(name):
     # the type lives in the C++ module, which is only loaded when first needed
     if name == "MoodistProcessGroup":

@@ -50,6 +50,8 @@ def core():
                                              ctypes.c_void_p, ctypes.c_void_p]
     L.moodist_pg_allreduce_many.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int,
                                             ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p]
+    L.moodist_pg_reduce_scatter_many.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
+                                                 ctypes.c_int, ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p]
     L.moodist_pg_allreduce.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
                                        ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p]
     L.moodist_work_wait.argtypes = [ctypes.c_void_p]
@@ -107,6 +109,77 @@ def test_options_by_name(core):
     assert v.value == 4096
     assert core.moodist_pg_set_option(pg, b"bogus", 1) != 0
     assert core.moodist_last_error() == b"Unknown option: bogus"  # core/processgroup.cc:2469
+    # num_chunks / chunk_size / method are honoured (they cut a reduce_scatter's reduction into
+    # pieces), so values that mean nothing are refused instead of stored
+    for name, bad in ((b"num_chunks", 0), (b"num_chunks", -2), (b"chunk_size", 0), (b"method", 3), (b"method", -2)):
+        assert core.moodist_pg_set_option(pg, name, bad) != 0, (name, bad)
+    assert core.moodist_pg_set_option(pg, b"method", 1) != 0  # copy: no counterpart among local ranks
+    assert b"method 1 (copy)" in core.moodist_last_error()
+    for name, good in ((b"num_chunks", 4), (b"num_chunks", -1), (b"method", 0), (b"method", 2), (b"method", -1),
+                       (b"chunk_size", -1)):
+        assert core.moodist_pg_set_option(pg, name, good) == 0, (name, good)
+        core.moodist_pg_get_option(pg, name, ctypes.byref(v))
+        assert v.value == good
+    core.moodist_world_destroy(w)
+
+
+def test_a_refused_list_leaves_nothing_posted(core):
+    # a coalesced allreduce or reduce_scatter whose list is refused (mixed element types, an
+    # operation one of the types does not support) has posted none of its tensors: the rank's next
+    # collective still is its collective number 0, which the other rank's number 0 then meets
+    T = type(fake(4))
+    for attempt in ("allreduce_many", "reduce_scatter_many"):
+        w = make_world(core, 2)
+        a, b = core.moodist_world_group(w, 0), core.moodist_world_group(w, 1)
+        work = ctypes.c_void_p()
+        mixed = (T * 3)(fake(16), fake(8), fake(24, dtype=3))  # fp32, fp32, int32
+        if attempt == "allreduce_many":
+            assert core.moodist_pg_allreduce_many(a, mixed, 3, 1, None, 0.0, ctypes.byref(work)) != 0  # AVG
+            assert core.moodist_pg_allreduce_many(a, mixed, 3, 0, None, 0.0, ctypes.byref(work)) != 0  # SUM
+            assert b"one element type" in core.moodist_last_error()
+        else:
+            outs = (T * 3)(fake(8), fake(4), fake(12, dtype=3))
+            assert core.moodist_pg_reduce_scatter_many(a, outs, mixed, 3, 1, None, 0.0, ctypes.byref(work)) != 0
+            assert core.moodist_pg_reduce_scatter_many(a, outs, mixed, 3, 0, None, 0.0, ctypes.byref(work)) != 0
+            assert b"one element type" in core.moodist_last_error()
+            outs[1] = fake(5)
+            same = (T * 3)(fake(16), fake(8), fake(24))
+            assert core.moodist_pg_reduce_scatter_many(a, outs, same, 3, 0, None, 0.0, ctypes.byref(work)) != 0
+        # rank 0's collective number 0 is this all_gather ...
+        assert core.moodist_pg_all_gather(a, ctypes.byref(fake(8)), ctypes.byref(fake(4)), None, ctypes.byref(work)) == 0
+        core.moodist_work_destroy(work)
+        # ... so a reduce_scatter as rank 1's number 0 is a mismatch, and the same all_gather is not
+        assert core.moodist_pg_reduce_scatter(b, ctypes.byref(fake(4)), ctypes.byref(fake(8)), 0, None, 0.0,
+                                              ctypes.byref(work)) != 0
+        assert b"different operation" in core.moodist_last_error()
+        core.moodist_world_destroy(w)
+
+
+def test_a_list_of_reduce_scatters_is_checked_like_one(core):
+    T = type(fake(4))
+    w = make_world(core, 4)
+    pg = core.moodist_world_group(w, 0)
+    work = ctypes.c_void_p()
+    ins = (T * 2)(fake(16), fake(24))
+    outs = (T * 2)(fake(4), fake(6))
+    assert core.moodist_pg_reduce_scatter_many(pg, outs, ins, 0, 0, None, 0.0, ctypes.byref(work)) != 0
+    assert b"1..65535 tensors" in core.moodist_last_error()
+    assert core.moodist_pg_reduce_scatter_many(pg, outs, None, 2, 0, None, 0.0, ctypes.byref(work)) != 0
+    assert core.moodist_pg_reduce_scatter_many(pg, outs, ins, 2, 2, None, 0.0, ctypes.byref(work)) != 0  # PRODUCT
+    assert core.moodist_last_error() == b"Unsupported reduce operation"
+    ins[1] = fake(25)  # not a multiple of the group size
+    assert core.moodist_pg_reduce_scatter_many(pg, outs, ins, 2, 0, None, 0.0, ctypes.byref(work)) != 0
+    ins[1] = fake(24, contiguous=0)
+    assert core.moodist_pg_reduce_scatter_many(pg, outs, ins, 2, 0, None, 0.0, ctypes.byref(work)) != 0
+    assert b"must be contiguous" in core.moodist_last_error()
+    ins[1] = fake(24)
+    assert core.moodist_pg_reduce_scatter_many(pg, outs, ins, 2, 0, None, 0.0, ctypes.byref(work)) == 0  # posted
+    core.moodist_work_destroy(work)
+    # another rank with a list of other sizes: the same total, caught before the launch
+    other = core.moodist_world_group(w, 1)
+    assert core.moodist_pg_reduce_scatter_many(other, None, (T * 2)(fake(20), fake(20)), 2, 0, None, 0.0,
+                                               ctypes.byref(work)) == 0
+    core.moodist_work_destroy(work)
     core.moodist_world_destroy(w)
 
 
@@ -496,6 +569,38 @@ def test_reference_constructor_joins_ranks_through_the_store():
     with pg.prefer_kernel_less(False):
         assert pg.get_prefer_kernel_less() is False
     assert pg.get_prefer_kernel_less() is True
+
+
+def test_backend_is_registered_with_torch_distributed():
+    # py/moodist/backend.py:71-78, :112-116: "moodist" is a torch.distributed backend whose creator
+    # builds the group the reference's way and enters it into the name registry
+    import subprocess
+    import sys
+    from datetime import timedelta
+
+    import torch.distributed as dist
+
+    assert dist.Backend("moodist") == "moodist" and dist.Backend.MOODIST == "moodist"
+    assert "MOODIST" in dist.Backend._plugins
+    assert dist.Backend.backend_capability["moodist"] == ["cuda"] or tuple(dist.Backend.backend_capability["moodist"]) == ("cuda",)
+    creator = dist.Backend._plugins["MOODIST"].creator_fn
+    assert creator is moodist_amd.create_moodist_backend
+    store = dist.HashStore()
+    groups = [creator(store, r, 2, timedelta(seconds=30)) for r in range(2)]
+    for r, g in enumerate(groups):
+        assert isinstance(g, dist.ProcessGroup) and g.rank() == r and g.size() == 2
+        assert moodist_amd.find_process_group(g.moodist_name()) is g
+    moodist_amd.register_backend()  # a second call changes nothing
+    # init_process_group finds it by name (its own process: the default group is process-wide state)
+    code = ("import torch.distributed as dist, moodist_amd\n"
+            "dist.init_process_group('moodist', store=dist.HashStore(), rank=0, world_size=1)\n"
+            "pg = dist.group.WORLD\n"
+            "assert dist.get_backend() == 'moodist' and pg.size() == 1\n"
+            "assert moodist_amd.find_process_group(pg.moodist_name()) is pg\n"
+            "dist.destroy_process_group()\nprint('ok')\n")
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300,
+                       cwd=ROOT)
+    assert r.returncode == 0 and "ok" in r.stdout, r.stderr[-2000:]
 
 
 def test_compile_op_accepts_dtensor_like_specs():

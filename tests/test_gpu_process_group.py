@@ -602,3 +602,99 @@ def test_kernel_less_gather_from_padded_staging_equals_the_kernel_path(world, de
             assert torch.equal(outs[r], want2)
     for pg in world:
         pg.options().force_kernel_less = False
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.int64], ids=str)
+def test_reduce_scatter_coalesced_is_one_collective_and_matches_the_oracle(world, dev, dtype):
+    # reference wrapper/processgroup_wrapper.cc:159-170 runs one reduce_scatter per tensor; here a
+    # list of one element type is one collective whose reductions share launches.  Rank q's
+    # output k is the fold of every rank's chunk q of tensor k, starting at rank q.
+    g = torch.Generator().manual_seed(17)
+    chunk_sizes = [1, 7, 64, 255, 1031, 4096 + 5, 70001, 3, 100000, 12, 513, 8191] * 4  # 48 tensors
+    ops = [("SUM", oracle.OP_SUM, dist.ReduceOp.SUM), ("MAX", oracle.OP_MAX, dist.ReduceOp.MAX)]
+    if dtype.is_floating_point:
+        ops.append(("AVG", oracle.OP_AVG, dist.ReduceOp.AVG))
+    for name, code, op in ops:
+        if dtype.is_floating_point:
+            host = [[(torch.randn(n * P, generator=g) * 3).to(dtype) for n in chunk_sizes] for _ in range(P)]
+        else:
+            host = [[torch.randint(-2 ** 40, 2 ** 40, (n * P,), generator=g) for n in chunk_sizes] for _ in range(P)]
+        ins = [[t.to(dev) for t in row] for row in host]
+        outs = [[torch.zeros(n, dtype=dtype, device=dev) for n in chunk_sizes] for _ in range(P)]
+        opts = dist.ReduceScatterOptions()
+        opts.reduceOp = op
+        each_rank(world, lambda r, pg: pg.reduce_scatter_tensor_coalesced(outs[r], ins[r], opts))
+        for k, n in enumerate(chunk_sizes):
+            for q in range(P):
+                want = oracle.reduce([bits(host[j][k][q * n:(q + 1) * n]) for j in range(P)], q, TORCH_TO_CODE[dtype], code,
+                                     1.0 / P if code == oracle.OP_AVG else 1.0)
+                assert same_bits(bits(outs[q][k]), want), (name, k, n, q)
+        for r in range(P):  # inputs untouched
+            assert torch.equal(ins[r][5].cpu(), host[r][5])
+
+
+def test_reduce_scatter_coalesced_of_mixed_element_types_goes_tensor_by_tensor(world, dev):
+    dtypes = [torch.float32, torch.int32, torch.float32]
+    n = 1000
+    ins = [[torch.full((n * P,), r + 1, device=dev).to(dt) for dt in dtypes] for r in range(P)]
+    outs = [[torch.zeros(n, dtype=dt, device=dev) for dt in dtypes] for _ in range(P)]
+    each_rank(world, lambda r, pg: pg.reduce_scatter_tensor_coalesced(outs[r], ins[r]))
+    for r in range(P):
+        for k, dt in enumerate(dtypes):
+            assert torch.equal(outs[r][k], torch.full((n,), 36, device=dev).to(dt))
+
+
+@pytest.mark.parametrize("option,value", [("num_chunks", 3), ("num_chunks", 64), ("chunk_size", 8192), ("chunk_size", 100000),
+                                          ("method", 2)])
+def test_chunk_options_cut_a_reduce_scatter_into_pieces_with_the_same_bits(world, dev, option, value):
+    # The options the reference stores for its direct method (core/processgroup.cc:334-340) are
+    # honoured here: the rank's chunk is reduced in pieces -- chunk_size bytes, or num_chunks
+    # pieces by the reference's arithmetic (:1494-1503), or with method 2 the reference's own
+    # count -- and the result is the unchunked fold, bit for bit.
+    for pg in world:
+        setattr(pg.options(), option, value)
+    try:
+        for dtype, n in ((torch.float32, 200003), (torch.bfloat16, 333337), (torch.float32, 1000), (torch.float64, 70001)):
+            host = [torch.stack(random_sources(P, n, dtype, seed=31 * r + n)).reshape(-1) for r in range(P)]
+            ins = [t.to(dev) for t in host]
+            outs = [torch.zeros(n, dtype=dtype, device=dev) for _ in range(P)]
+            each_rank(world, lambda r, pg: pg._reduce_scatter_base(outs[r], ins[r]))
+            for q in range(P):
+                want = oracle.reduce([bits(host[j][q * n:(q + 1) * n]) for j in range(P)], q, TORCH_TO_CODE[dtype],
+                                     oracle.OP_SUM)
+                assert same_bits(bits(outs[q]), want), (option, value, dtype, n, q)
+    finally:
+        for pg in world:
+            setattr(pg.options(), option, None)
+    with pytest.raises(RuntimeError, match=r"method 1 \(copy\)"):
+        world.groups[0].options().method = 1
+
+
+def test_init_process_group_with_the_moodist_backend(dev):
+    # reference py/moodist/backend.py:112-116: torch.distributed finds the backend by name.  In a
+    # process of its own: the default group is process-wide state.
+    import os
+    import subprocess
+    import sys
+
+    code = """
+import torch, torch.distributed as dist
+import moodist_amd
+dist.init_process_group("moodist", store=dist.HashStore(), rank=0, world_size=1)
+assert dist.get_backend() == "moodist"
+x = torch.arange(1000, dtype=torch.float32, device="cuda") + 1
+dist.all_reduce(x)
+out = torch.zeros(1000, device="cuda")
+dist.all_gather_into_tensor(out, x)
+shard = torch.zeros(1000, device="cuda")
+dist.reduce_scatter_tensor(shard, x)
+torch.cuda.synchronize()
+want = torch.arange(1000, dtype=torch.float32, device="cuda") + 1
+assert torch.equal(x, want) and torch.equal(out, want) and torch.equal(shard, want)
+assert moodist_amd.find_process_group(dist.group.WORLD.moodist_name()) is dist.group.WORLD
+dist.destroy_process_group()
+print("ok")
+"""
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300, cwd=root)
+    assert r.returncode == 0 and "ok" in r.stdout, (r.stdout[-1000:], r.stderr[-3000:])

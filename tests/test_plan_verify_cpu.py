@@ -50,7 +50,7 @@ def test_equal_boxes_of_full_tiles_start_from_leading_scalar_arguments():
     words = struct.unpack("<14I", args[:56])
     assert words[0] == 8192 * 4                       # source row pitch in bytes
     log2tc, nct = words[1] & 31, words[1] >> 5
-    assert (1 << log2tc) == 4096 // 16 and nct == 1   # a row of 4 KiB is one tile's width
+    assert (1 << log2tc) == 64 and nct == 4            # a row of 4 KiB is four tiles of 64 vectors (1 KiB) wide
     assert gx % nct == 0 and 1024 % (gx // nct) == 0  # whole rows of tiles, each of the same number of rows
     for s in range(8):
         pair = words[10 + s // 2]
@@ -143,6 +143,33 @@ def test_ragged_rows_transposes_and_many_dimensions(itemsize):
     ]
     sizes = [s[0] + 64 for s in specs] + [80000 * itemsize]
     plan_for(specs, itemsize).verify(sizes)
+
+
+@pytest.mark.parametrize("itemsize", [1, 2, 4, 8, 16])
+def test_transposing_boxes_take_tiles_through_lds(itemsize):
+    # out[c][r] = in[r][c]: source contiguous along one dimension, destination along the other.  With
+    # both dimensions at least 16 long the box is copied in tiles turned round in LDS; the check
+    # replays every tile through the kernel's own index function.
+    import struct
+
+    for R, C, soff, doff, spad, dpad in ((64, 64, 0, 0, 0, 0), (100, 36, 0, 0, 0, 0), (17, 333, 3, 5, 1, 2),
+                                         (130, 70, 4, 8, 4, 12), (16, 16, 0, 1, 0, 0)):
+        specs = [((R * (C + spad) + soff + 4) * itemsize, soff, doff, [C, R], [1, C + spad], [R + dpad, 1])]
+        p = plan_for(specs, itemsize)
+        assert p.launches == 1
+        p.verify([specs[0][0], (C * (R + dpad) + doff + 4) * itemsize])
+        args, lead, gx, gy, block, lds = p.step_arguments([0x7F00_0000_0000, 0x7E00_0000_0000], 0)
+        tile = 64 if itemsize <= 4 else 32
+        assert lead == 0 and gy == 1 and block == 256 and gx == -(-R // tile) * -(-C // tile)
+        src0, dst0 = struct.unpack("<QQ", args[:16])
+        assert src0 == 0x7F00_0000_0000 + soff * itemsize and dst0 == 0x7E00_0000_0000 + doff * itemsize
+    # two batch dimensions around the transposed pair, and the pair in the middle of the box
+    specs = [(3 * 4 * 50 * 40 * itemsize + 64, 0, 0, [3, 4, 40, 50], [4 * 50 * 40, 50 * 40, 1, 40], [4 * 40 * 50, 40 * 50, 50, 1]),
+             (20 * 30 * 6 * itemsize + 64, 2, 3 * 4 * 50 * 40 + 7, [30, 6, 20], [1, 20 * 30, 30], [6 * 20, 20, 1])]
+    plan_for(specs, itemsize).verify([specs[0][0], specs[1][0], (3 * 4 * 50 * 40 + 7 + 30 * 6 * 20 + 4) * itemsize])
+    # below 16 elements on one side the plain strided kernel keeps the box (one launch of it)
+    small = [(8 * 500 * itemsize + 64, 0, 0, [500, 8], [1, 500], [8, 1])]
+    plan_for(small, itemsize).verify([small[0][0], 500 * 8 * itemsize + 64])
 
 
 def test_random_boxes():

@@ -15,7 +15,14 @@ LIB = os.path.join(ROOT, "moodist_amd", "libmoodist.so")
 HEADER = os.path.join(ROOT, "include", "moodist_plugin.h")
 REFERENCE_HEADER = "/root/reference/api/moodist_api.h"
 API_VERSION = 2
-BUILD_MAGIC = 0x4D49333535584D44
+SOURCE_TREE_MAGIC = 0x4D49333535584D44  # what a translation unit compiled on its own carries
+
+
+def build_magic():
+    """The number the built libmoodist.so drew (moodist_amd/csrc/build_host.sh)."""
+    L = ctypes.CDLL(LIB)
+    L.moodist_build_magic.restype = ctypes.c_uint64
+    return L.moodist_build_magic()
 
 
 def struct_members(text, name):
@@ -85,7 +92,8 @@ def test_version_mismatch_gives_null_and_the_table_carries_the_build_magic(lib, 
         assert lib.moodistGetApi(wrong, table) is None
     api = lib.moodistGetApi(API_VERSION, table)
     assert api
-    assert ctypes.c_uint64.from_address(api).value == BUILD_MAGIC
+    assert ctypes.c_uint64.from_address(api).value == build_magic()
+    assert build_magic() != SOURCE_TREE_MAGIC and build_magic() != 0  # drawn by the build, not the header's constant
     # one table per core: asking again gives the same one
     assert lib.moodistGetApi(API_VERSION, table) == api
 
@@ -157,5 +165,38 @@ def test_the_python_module_loaded_its_core_through_the_entry():
     from moodist_amd import _C
 
     info = _C.core_api_info()
-    assert info["entry"] == "moodistGetApi" and info["version"] == API_VERSION and info["magic"] == BUILD_MAGIC
+    assert info["entry"] == "moodistGetApi" and info["version"] == API_VERSION and info["magic"] == build_magic()
     assert info["slots"] == 69 and os.path.samefile(info["path"], LIB)
+
+
+def test_a_core_of_another_build_is_refused_by_its_magic(tmp_path):
+    # The reference draws a build magic per configure so that a stale libmoodist.so beside a new
+    # _C is caught (CMakeLists.txt:97-106; wrapper/moodist_loader.cc:363-386).  Here: a Python
+    # module built with another magic, placed beside the built core, must refuse to load it.
+    import shutil
+    import subprocess
+    import sys
+    import sysconfig
+
+    suffix = sysconfig.get_config_var("EXT_SUFFIX")
+    other = tmp_path / ("_C" + suffix)
+    env = dict(os.environ, MOODIST_BUILD_MAGIC="0x0123456789abcdefULL")
+    subprocess.run([sys.executable, os.path.join(ROOT, "moodist_amd", "csrc", "wrapper", "build_wrapper.py"), str(other)],
+                   check=True, capture_output=True, text=True, env=env)
+    shutil.copy(LIB, tmp_path / "libmoodist.so")
+    code = ("import importlib.util, sys\n"
+            "spec = importlib.util.spec_from_file_location('_C', %r)\n"
+            "m = importlib.util.module_from_spec(spec)\n"
+            "spec.loader.exec_module(m)\n" % str(other))
+    r = subprocess.run([sys.executable, "-c", "import torch\n" + code], capture_output=True, text=True, timeout=300)
+    assert r.returncode != 0
+    assert "build magic mismatch" in r.stderr, r.stderr[-2000:]
+    # and the module of THIS build loads the same copy of the core
+    mine = tmp_path / "same" / ("_C" + suffix)
+    os.makedirs(mine.parent)
+    shutil.copy(os.path.join(ROOT, "moodist_amd", "_C" + suffix), mine)
+    shutil.copy(LIB, mine.parent / "libmoodist.so")
+    r = subprocess.run([sys.executable, "-c", "import torch\n" + code.replace(str(other), str(mine)) +
+                        "print(m.core_api_info()['magic'])\n"], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert int(r.stdout.strip()) == build_magic()

@@ -52,9 +52,15 @@ def test_plugin_entry_and_reference_lifetimes_under_sanitizers(tmp_path):
 def test_plugin_entry_of_the_built_library_through_dlsym(tmp_path):
     # the same walk against the shipped libmoodist.so: dlopen + dlsym("moodistGetApi"), the
     # driver's own destroy() going back through the table
+    import ctypes
+
     lib = os.path.join(ROOT, "moodist_amd", "libmoodist.so")
     exe = str(tmp_path / "driver")
-    subprocess.run(["g++", "-std=c++20", "-O1", "-g", "-DMOODIST_DRIVER_DLOPEN", "-I" + os.path.join(ROOT, "include"),
+    # the driver checks the table's magic against its own: compiled with the built library's
+    L = ctypes.CDLL(lib)
+    L.moodist_build_magic.restype = ctypes.c_uint64
+    subprocess.run(["g++", "-std=c++20", "-O1", "-g", "-DMOODIST_DRIVER_DLOPEN",
+                    "-DMOODIST_BUILD_MAGIC=0x%xULL" % L.moodist_build_magic(), "-I" + os.path.join(ROOT, "include"),
                     os.path.join(HERE, "sanitize", "plugin_driver.cc"), "-ldl", "-o", exe],
                    check=True, capture_output=True, text=True)
     r = subprocess.run([exe, lib], cwd=str(tmp_path), capture_output=True, text=True, timeout=300)

@@ -191,6 +191,49 @@ def test_device_memory_in_use_does_not_change_over_a_call(core):
         world.close()
 
 
+def test_back_to_back_calls_with_every_rank_on_its_own_stream(core):
+    # Four ranks, each on a stream of its own, two padded allreduces in a row with different
+    # data and nothing waited for in between: rank r's second copy into its workspace slice must
+    # wait for the other ranks' first reductions, which read that slice on THEIR streams.  With
+    # one shared stream that order is the stream's; here it is the events the world places.
+    size, numel = 4, 999_999  # pads to 1,000,000: 4 MB of a rank's 16 MiB slice
+    world = World(core, size)
+    try:
+        streams = [torch.cuda.Stream() for _ in range(size)]
+        rounds = [inputs(size, numel, torch.float32, seed) for seed in (21, 22)]
+        # the answer: moodist_pg_allreduce with a caller's temporary, one round at a time
+        want = []
+        padded = (numel + size - 1) // size * size
+        for host in rounds:
+            a = [t.cuda() for t in host]
+            temporaries = [torch.empty(padded, dtype=torch.float32, device="cuda") for _ in range(size)]
+            torch.cuda.synchronize()
+            works = []
+            for r in range(size):
+                rc, w = world.with_temporary(r, a[r], temporaries[r], SUM)
+                assert rc == 0, core.moodist_last_error()
+                works.append(w)
+            world.finish(works)
+            want.append([t.cpu() for t in a])
+        tensors = [[t.cuda() for t in host] for host in rounds]
+        torch.cuda.synchronize()
+        works = []
+        for k in range(2):
+            print("round", k, flush=True)
+            for r in range(size):
+                work = ctypes.c_void_p()
+                rc = core.moodist_pg_allreduce_static(world.groups[r], ctypes.byref(describe(tensors[k][r])), SUM,
+                                                      ctypes.c_void_p(streams[r].cuda_stream), 0.0, ctypes.byref(work))
+                assert rc == 0, core.moodist_last_error()
+                works.append(work)
+        world.finish(works)
+        for k in range(2):
+            for r in range(size):
+                assert torch.equal(bits(tensors[k][r].cpu()), bits(want[k][r])), (k, r)
+    finally:
+        world.close()
+
+
 def test_limits(core):
     world = World(core, 8)
     try:
