@@ -883,6 +883,38 @@ void World::order_streams_after(Collective& c) {
   }
 }
 
+namespace {
+
+// A rank's chunk of this size and less makes a launch that is over in a few microseconds, most
+// of them the launch itself; such collectives share launches among the ranks of a stream.
+constexpr size_t kSharedLaunchBytes = (size_t)1 << 20;
+
+// The ranks that asked for an output and whose reduction is not cut into pieces, grouped by the
+// stream they passed, in rank order.
+std::vector<std::vector<int>> ranks_by_stream(const Collective& c) {
+  std::vector<std::vector<int>> groups;
+  for (size_t q = 0; q < c.post.size(); ++q) {
+    const Posting& pq = c.post[q];
+    if (!pq.wants_output || pq.chunk_bytes != 0) {
+      continue;
+    }
+    bool placed = false;
+    for (std::vector<int>& g : groups) {
+      if (c.post[(size_t)g[0]].stream == pq.stream) {
+        g.push_back((int)q);
+        placed = true;
+        break;
+      }
+    }
+    if (!placed) {
+      groups.push_back({(int)q});
+    }
+  }
+  return groups;
+}
+
+} // namespace
+
 void World::launch(Collective& c, const std::shared_ptr<CompiledOp>& op) {
   if (c.kind == Kind::all_gather_many || c.kind == Kind::reduce_scatter_many) {
     // the ranks agreed on the number of tensors and their total size (post); now tensor by tensor
@@ -934,9 +966,34 @@ void World::launch(Collective& c, const std::shared_ptr<CompiledOp>& op) {
     // AVG is SUM then a multiply by 1.0f/size (core/processgroup.cc:1664-1667); PREMUL_SUM
     // multiplies every input by the factor first (:1374-1378)
     const float scale = c.reduce_op == MDH_OP_AVG ? 1.0f / (float)size : c.premul;
+    // Short reductions are bound by the launch, not by memory: the ranks that share a stream
+    // (in one process they usually all do) share ONE launch, a job per rank (mdh_reduce_many).
+    std::vector<bool> done((size_t)size, false);
+    if (c.bytes <= kSharedLaunchBytes) {
+      for (const std::vector<int>& ranks : ranks_by_stream(c)) {
+        if (ranks.size() < 2) {
+          continue;
+        }
+        std::vector<const void*> tables(ranks.size() * (size_t)size);
+        std::vector<mdh_reduce_job> jobs(ranks.size());
+        for (size_t k = 0; k < ranks.size(); ++k) {
+          const int q = ranks[k];
+          for (int j = 0; j < size; ++j) {
+            tables[k * (size_t)size + (size_t)j] = (const char*)c.post[(size_t)j].input.data + c.bytes * (size_t)q;
+          }
+          jobs[k].srcs = tables.data() + k * (size_t)size;
+          jobs[k].nsrc = size;
+          jobs[k].first = q;
+          jobs[k].dst = c.post[(size_t)q].output.data;
+          jobs[k].numel = numel;
+          done[(size_t)q] = true;
+        }
+        check_mdh(h.reduce_many(jobs.data(), (int)jobs.size(), c.dtype, c.reduce_op, scale, c.post[(size_t)ranks[0]].stream));
+      }
+    }
     for (int q = 0; q < size; ++q) {
       const Posting& pq = c.post[(size_t)q];
-      if (!pq.wants_output) {
+      if (!pq.wants_output || done[(size_t)q]) {
         continue;
       }
       for (int j = 0; j < size; ++j) {
@@ -993,9 +1050,52 @@ void World::launch(Collective& c, const std::shared_ptr<CompiledOp>& op) {
     }
   } else if (c.kind == Kind::all_gather) {
     // out_q[pitch*j .. +bytes] = in_j for every j (core/allgather.cc:381-390)
+    // Short gathers, like short reductions: the ranks that share a stream share one launch, a
+    // contiguous copy per destination rank and source rank.
+    std::vector<bool> done((size_t)size, false);
+    if (c.bytes <= kSharedLaunchBytes) {
+      for (const std::vector<int>& ranks : ranks_by_stream(c)) {
+        bool plain = ranks.size() >= 2;
+        for (int q : ranks) {
+          plain = plain && c.post[(size_t)q].outputs.empty() && !c.post[(size_t)q].kernel_less;
+        }
+        if (!plain) {
+          continue;
+        }
+        std::vector<mdh_box> boxes;
+        boxes.reserve(ranks.size() * (size_t)size);
+        for (int q : ranks) {
+          for (int j = 0; j < size; ++j) {
+            mdh_box b{};
+            b.src = c.post[(size_t)j].input.data;
+            b.dst = (char*)c.post[(size_t)q].output.data + c.bytes * (size_t)j;
+            if (b.src == b.dst) {
+              continue; // already in place
+            }
+            b.ndim = 1;
+            b.shape[0] = (int64_t)c.bytes;
+            b.src_strides[0] = b.dst_strides[0] = 1;
+            boxes.push_back(b);
+          }
+          done[(size_t)q] = true;
+        }
+        void* stream = c.post[(size_t)ranks[0]].stream;
+        if (!boxes.empty()) {
+          check_mdh(h.copy_boxes(boxes.data(), (int)boxes.size(), 1, stream));
+        }
+        for (int q : ranks) {
+          const Posting& pq = c.post[(size_t)q];
+          if (pq.has_copy_back) { // allreduce through a padded temporary (core/processgroup.cc:1716-1720)
+            check_hip(h.MemcpyAsync(pq.copy_back.data, pq.output.data,
+                          (size_t)pq.copy_back.numel * (size_t)pq.copy_back.itemsize, kHipMemcpyDeviceToDevice, stream),
+                "hipMemcpyAsync");
+          }
+        }
+      }
+    }
     for (int q = 0; q < size; ++q) {
       const Posting& pq = c.post[(size_t)q];
-      if (!pq.wants_output) {
+      if (!pq.wants_output || done[(size_t)q]) {
         continue;
       }
       for (int j = 0; j < size; ++j) {

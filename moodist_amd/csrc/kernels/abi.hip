@@ -163,7 +163,7 @@ extern "C" int mdh_set_tuning(const char* name, int value) {
       return MDH_EINVAL;
     }
   } else if (value < 0 || (std::strstr(name, "wg_per_cu") && value > 9) || (!std::strcmp(name, "box_policy") && value > 2) ||
-             (!std::strcmp(name, "box_preload") && value > 1) || (!std::strcmp(name, "box_transpose") && value > 1) || (!std::strcmp(name, "allow_capture") && value > 1)) {
+             (!std::strcmp(name, "box_preload") && value > 1) || (!std::strcmp(name, "box_transpose") && value > 2) || (!std::strcmp(name, "allow_capture") && value > 1)) {
     mdh::set_error("mdh_set_tuning: %s does not take %d", name, value);
     return MDH_EINVAL;
   }

@@ -570,7 +570,11 @@ __global__ __launch_bounds__(kBlock) void copy_flat8_kernel(uint32_t bytes, uint
       reach = tile_bytes / 2;
     }
   }
-  const uint32_t left = off < bytes ? bytes - off : 0;
+  // (Wave-uniform, and it must stay in scalar registers: it is the size of the tile's buffer
+  // descriptors.  Written as a saturating subtraction it is compiled to a vector instruction,
+  // and every load and store then runs inside a loop that makes its descriptor uniform again --
+  // 2 us of an 80 us launch.  Only a variant's half tiles can start past the segment's end.)
+  const uint32_t left = VARIANT == 1 ? bytes - (uint32_t)__builtin_amdgcn_readfirstlane((int)(off < bytes ? off : bytes)) : bytes - off;
   const uint32_t n = left < reach ? left : reach;
   const char* src = (const char*)(uintptr_t)packed_source_address(seg, l0, l1, l2, l3, l4, l5, l6, l7, h0, h1, h2, h3);
   const __amdgpu_buffer_rsrc_t rs = tile_rsrc(src + off, n);
@@ -1106,6 +1110,7 @@ struct Launcher {
             ++i;
           }
           a.total_tiles = (uint32_t)tiles;
+          a.diagonal = tuning().box_transpose == 2 ? 0u : 1u;
           Step st;
           st.kind = Step::kTrans, st.vec = 1 << lg, st.unroll = 1, st.grid = a.total_tiles, st.grid_y = 0, st.lds = 0;
           st.plain_loads = false, st.wide = wide != 0;

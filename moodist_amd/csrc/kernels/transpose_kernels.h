@@ -39,6 +39,7 @@ struct TransArgs {
   uint32_t tile_end[kMaxTransBoxes]; // cumulative tiles; unused entries are ~0
   uint32_t nboxes;
   uint32_t total_tiles;
+  uint32_t diagonal; // 0: a box's tiles run along A first, then B; 1: along its diagonals (see trans_locate)
 };
 static_assert(sizeof(TransArgs) + 256 <= 4096, "kernel arguments are limited to 4 KiB");
 
@@ -55,8 +56,8 @@ struct TransLoc {
 };
 
 // Which box a tile belongs to and where it starts: the cumulative ends ascend, the last one at
-// or below the tile names the box (scalar selects on the device); inside a box the tiles run
-// along A first, then B, then the other extents.  Shared by the kernel and by the host-side
+// or below the tile names the box (scalar selects on the device); inside a box the tiles of one
+// A x B plane come first, then the other extents.  Shared by the kernel and by the host-side
 // check of a prepared plan.
 MDH_HD TransLoc trans_locate(const TransArgs& a, uint32_t tile, uint32_t elem) {
   uint32_t b = 0, start = 0;
@@ -69,10 +70,23 @@ MDH_HD TransLoc trans_locate(const TransArgs& a, uint32_t tile, uint32_t elem) {
   const TransBox& B = a.box[b];
   uint32_t local = tile - start;
   const uint32_t T = trans_tile(elem);
-  const uint32_t ta_i = local % B.ta;
-  local /= B.ta;
-  const uint32_t tb_i = local % B.tb;
-  local /= B.tb;
+  // Consecutive workgroups run at the same time.  Along A first, the tiles of a moment share
+  // their destination columns: they write a strip 256 bytes wide down every row of the
+  // destination, and with a power-of-two pitch that strip lives in a few DRAM channels (along
+  // B first it is the reads).  Along the diagonals -- B advances with every tile and A with it --
+  // both sides spread over rows and columns alike.
+  uint32_t ta_i, tb_i;
+  if (a.diagonal) {
+    tb_i = local % B.tb;
+    local /= B.tb;
+    ta_i = (local % B.ta + tb_i) % B.ta;
+    local /= B.ta;
+  } else {
+    ta_i = local % B.ta;
+    local /= B.ta;
+    tb_i = local % B.tb;
+    local /= B.tb;
+  }
   const uint32_t o0 = local % B.no[0], o1 = local / B.no[0];
   TransLoc t;
   t.box = b;

@@ -8,12 +8,14 @@
 // -fsanitize=address,undefined; and with -DMOODIST_DRIVER_DLOPEN against the built
 // libmoodist.so (path in argv[1]), resolving moodistGetApi with dlsym as a wrapper does.
 #include "moodist_plugin.h"
+#include "moodist_core.h"
 
 #ifdef MOODIST_DRIVER_DLOPEN
 #include <dlfcn.h>
 #endif
 
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <stdexcept>
 #include <string>
@@ -49,6 +51,7 @@ using namespace moodist;
 
 static int live_tensors = 0;
 static int empties_made = 0;
+static int device_allocations = 0; // calls of the wrapper's caching allocator (snapshot_inputs)
 
 static Tensor* make(int64_t numel, DType dtype = DType::Float32, int itemsize = 4, int device = 0) {
   Tensor* t = new Tensor;
@@ -317,6 +320,65 @@ int main(int argc, char** argv) {
     api::ProcessGroupHandle again = core->createProcessGroup(&store_a, 0, 8);
     EXPECT(core->processGroupSize(again.get()) == 8);
   }
+  // The allreduce that allocates nothing, with the one option that allocates switched on: a
+  // table that HAS a device allocator (and counts its calls), a world made after it was handed
+  // over, snapshot_inputs = 1.  moodist_pg_allreduce_static must not ask the allocator for
+  // anything -- neither when the group size divides the element count (its reduce_scatter half
+  // would snapshot the tensor) nor on the padded path (which ends early here: the fixed
+  // workspace needs a device) -- while a plain reduce_scatter on the same group does ask.
+  {
+    WrapperApi with_allocator = wrapper_table();
+    with_allocator.cudaCachingAllocatorAlloc = [](size_t bytes, void** cleanup) -> void* {
+      ++device_allocations;
+      void* p = std::malloc(bytes ? bytes : 1);
+      *cleanup = p;
+      return p;
+    };
+    with_allocator.cudaCachingAllocatorFree = [](void* cleanup) { std::free(cleanup); };
+    EXPECT(moodistGetApi(kMoodistApiVersion, &with_allocator) == core);
+    int store_c = 0;
+    std::vector<api::ProcessGroupHandle> h;
+    for (int r = 0; r < 4; ++r) {
+      h.push_back(core->createProcessGroup(&store_c, r, 4));
+    }
+    core->processGroupSetOption(h[0].get(), "snapshot_inputs", 1);
+    EXPECT(core->processGroupGetOption(h[0].get(), "snapshot_inputs") == 1);
+    auto allreduce_static = reinterpret_cast<decltype(&moodist_pg_allreduce_static)>(
+#ifdef MOODIST_DRIVER_DLOPEN
+        dlsym(lib, "moodist_pg_allreduce_static")
+#else
+        reinterpret_cast<void*>(&moodist_pg_allreduce_static)
+#endif
+    );
+    EXPECT(allreduce_static != nullptr);
+    moodist_tensor even{};
+    even.data = (void*)0x200000, even.numel = 4096, even.itemsize = 4, even.dtype = 6, even.device = 0;
+    even.contiguous = 1, even.ndim = 1, even.shape[0] = 4096;
+    moodist_work* work = nullptr;
+    const int before = device_allocations;
+    EXPECT(allreduce_static(moodistGroupCHandle(h[0].get()), &even, 0, nullptr, 0.0f, &work) == 0); // posted, pending
+    EXPECT(device_allocations == before);
+    moodist_tensor odd = even;
+    odd.numel = 4097, odd.shape[0] = 4097;
+    moodist_work* none = nullptr;
+    EXPECT(allreduce_static(moodistGroupCHandle(h[1].get()), &odd, 0, nullptr, 0.0f, &none) != 0); // no device here
+    EXPECT(device_allocations == before);
+    // the same option on a plain reduce_scatter goes for the snapshot, which cannot be made here
+    // (no kernel library or no device, depending on the build): the call fails, and whatever it
+    // took from the allocator it has given back
+    TensorPtr in(make(16)), out(make(4));
+    EXPECT(!thrown([&] { core->processGroupReduceScatter(h[0].get(), out, in, ReduceOp::SUM, nullptr, 0.0f); }).empty());
+    EXPECT(device_allocations == before || device_allocations == before + 1);
+    EXPECT(in.get()->refcount.load() == 1 && out.get()->refcount.load() == 1);
+    w.tensorDecRef(in.release());
+    w.tensorDecRef(out.release());
+#ifdef MOODIST_DRIVER_DLOPEN
+    reinterpret_cast<decltype(&moodist_work_destroy)>(dlsym(lib, "moodist_work_destroy"))(work);
+#else
+    moodist_work_destroy(work);
+#endif
+  }
+  EXPECT(live_tensors == 0);
   std::puts("plugin driver done");
   return 0;
 }
