@@ -35,17 +35,20 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 CLOCK_WARMUP_S = 0.3   # untimed launches before the first timed window
 TIMED_WINDOWS = 11     # windows of `steps` launches; the median window is reported
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch), each
-# scaled by what the same counter reads for the flat copy of exactly 256 MiB (FETCH_SIZE x 1.99982,
+# scaled by what the same counter reads for the flat copy of exactly 256 MiB (FETCH_SIZE x 1.99992,
 # WRITE_SIZE x 1.00000): profiles/hbm_traffic_pmc_reduce_and_copy_kernels.md.  E.g. the headline:
-# 65,552.29 x 1.99982 + 16,384.00 KiB = 147,476.6 KiB.  Workloads without an entry were not measured.
+# 65,560.15 x 1.99992 + 16,384.00 KiB = 147,498.9 KiB.  Workloads without an entry were not measured.
 MEASURED_TRAFFIC_BYTES = {
-    "reduce_fp32_p8": 151016081,
-    "reduce_bf16_p16": 1140854653,
-    "reduce_fp32_p64_sum": 272663625,
+    "reduce_fp32_p8": 151038850,
+    "reduce_bf16_p16": 1140907970,
+    "reduce_fp32_p64_sum": 272676956,
+    "reduce_fp32_p64_avg": 272677784,
+    "reduce_fp32_p64_max": 272690521,
     "allgather_bf16_p8": 536870912,
-    "allgather_bf16_p8_strided": 536884313,
-    "redistribute_fp32_8192": 67144034,
-    "redistribute_bf16_3d": 16799525,
+    "allgather_bf16_p8_strided": 536897643,
+    "redistribute_fp32_8192": 67145701,
+    "redistribute_bf16_8192": 33591324,
+    "redistribute_bf16_3d": 16799942,
 }
 
 DTYPE_NAMES = {"float32": "f32", "bfloat16": "bf16", "float16": "f16", "float64": "f64", "int32": "i32", "int64": "i64",
