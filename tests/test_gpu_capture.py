@@ -21,7 +21,13 @@ class Capture:
     has loaded.  Leaving the block ends the capture, counts the graph's nodes and destroys it."""
 
     def __init__(self, stream):
-        self.hip = ctypes.CDLL("libamdhip64.so")
+        # the copy of the runtime this process has mapped already (torch's), not a second one
+        path = "libamdhip64.so"
+        for line in open("/proc/self/maps"):
+            if "libamdhip64.so" in line:
+                path = line.split()[-1]
+                break
+        self.hip = ctypes.CDLL(path)
         self.hip.hipStreamBeginCapture.argtypes = [ctypes.c_void_p, ctypes.c_int]
         self.hip.hipStreamEndCapture.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p)]
         self.hip.hipGraphGetNodes.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.POINTER(ctypes.c_size_t)]

@@ -106,3 +106,54 @@ def test_many_transposing_boxes_in_one_call(dev):
     torch.cuda.synchronize()
     for k, (got, want) in enumerate(checks):
         assert torch.equal(got.cpu(), want), k
+
+
+def test_random_permuted_boxes_against_the_oracle(dev):
+    """Random boxes whose source is a permuted view of a padded parent (so that its contiguous
+    dimension is any of the box's dimensions), extents 1..90, one to four dimensions, every element
+    size, several boxes per call: the oracle's element-by-element copy decides, and bytes outside
+    the boxes must stay as they were."""
+    import oracle
+
+    rng = np.random.RandomState(23)
+    for trial in range(60):
+        itemsize = int(rng.choice([1, 2, 4, 8, 16]))
+        nboxes = int(rng.randint(1, 4))
+        specs, dst_elems = [], 0
+        for _ in range(nboxes):
+            nd = int(rng.randint(2, 5))
+            shape = [int(rng.choice([1, 2, 3, 17, 33, 64, 90])) for _ in range(nd)]
+            big = rng.choice(nd, 2, replace=False)  # at least two long extents: a transposing pair is possible
+            for d in big:
+                shape[d] = int(rng.choice([16, 31, 64, 70, 90]))
+            pshape = [s + int(rng.randint(0, 3)) for s in shape]
+            perm = list(rng.permutation(nd))
+            sstr = [0] * nd
+            acc = 1
+            for d in reversed(range(nd)):
+                sstr[perm[d]] = acc
+                acc *= pshape[perm[d]]
+            soff = int(rng.randint(0, 3))
+            dshape = [s + int(rng.randint(0, 2)) for s in shape]
+            dstr = [0] * nd
+            acc2 = 1
+            for d in reversed(range(nd)):
+                dstr[d] = acc2
+                acc2 *= dshape[d]
+            specs.append((shape, sstr, soff, acc + soff, dstr, dst_elems + int(rng.randint(0, 3)), acc2))
+            dst_elems = specs[-1][5] + acc2
+        dst_elems += 3
+        dst_host = rng.randint(0, 256, dst_elems * itemsize).astype(np.uint8)
+        want = dst_host.copy()
+        dst_dev = torch.from_numpy(dst_host.copy()).to(dev)
+        boxes, keep = [], []
+        for shape, sstr, soff, src_numel, dstr, doff, _ in specs:
+            src_host = rng.randint(0, 256, src_numel * itemsize).astype(np.uint8)
+            src_dev = torch.from_numpy(src_host).to(dev)
+            keep.append(src_dev)
+            oracle.copy_box(src_host, soff, want, doff, shape, sstr, dstr, itemsize)
+            boxes.append(abi.make_box(src_dev.data_ptr() + soff * itemsize, dst_dev.data_ptr() + doff * itemsize, shape,
+                                      sstr, dstr))
+        abi.copy_boxes(boxes, itemsize, st())
+        torch.cuda.synchronize()
+        assert np.array_equal(dst_dev.cpu().numpy(), want), (trial, itemsize, specs)

@@ -172,6 +172,38 @@ def test_transposing_boxes_take_tiles_through_lds(itemsize):
     plan_for(small, itemsize).verify([small[0][0], 500 * 8 * itemsize + 64])
 
 
+def test_random_permuted_boxes():
+    # sources that are permuted views of padded parents, extents up to 90: transposing pairs with
+    # batch dimensions around them, partial tiles, every element size, several boxes per plan
+    rng = np.random.RandomState(23)
+    for trial in range(20):
+        itemsize = int(rng.choice([1, 2, 4, 8, 16]))
+        nboxes = int(rng.randint(1, 4))
+        boxes, sizes, dst_elems = [], [], 0
+        for _ in range(nboxes):
+            nd = int(rng.randint(2, 5))
+            shape = [int(rng.choice([1, 2, 3, 17, 33, 64, 90])) for _ in range(nd)]
+            for d in rng.choice(nd, 2, replace=False):
+                shape[d] = int(rng.choice([16, 31, 64, 70, 90]))
+            pshape = [s + int(rng.randint(0, 3)) for s in shape]
+            perm = list(rng.permutation(nd))
+            sstr, acc = [0] * nd, 1
+            for d in reversed(range(nd)):
+                sstr[perm[d]] = acc
+                acc *= pshape[perm[d]]
+            soff = int(rng.randint(0, 3))
+            dstr, acc2 = [0] * nd, 1
+            for d in reversed(range(nd)):
+                dstr[d] = acc2
+                acc2 *= shape[d] + int(rng.randint(0, 2))
+            doff = dst_elems + int(rng.randint(0, 3))
+            boxes.append(abi.make_box(soff * itemsize, doff * itemsize, shape, sstr, dstr))
+            sizes.append((acc + soff + 4) * itemsize)
+            dst_elems = doff + acc2
+        plan = abi.CopyPlan(boxes, list(range(nboxes)), [nboxes] * nboxes, itemsize, nboxes + 1)
+        plan.verify(sizes + [(dst_elems + 4) * itemsize])
+
+
 def test_random_boxes():
     rng = np.random.RandomState(11)
     for trial in range(60):
