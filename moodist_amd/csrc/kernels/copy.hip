@@ -1111,6 +1111,8 @@ struct Launcher {
           }
           a.total_tiles = (uint32_t)tiles;
           a.diagonal = tuning().box_transpose == 2 ? 0u : 1u;
+          const TransShape shape = trans_shape(1u << lg, wide ? tuning().box_transpose_tile : 0);
+          a.tile_a = shape.a, a.tile_b = shape.b;
           Step st;
           st.kind = Step::kTrans, st.vec = 1 << lg, st.unroll = 1, st.grid = a.total_tiles, st.grid_y = 0, st.lds = 0;
           st.plain_loads = false, st.wide = wide != 0;
@@ -1173,12 +1175,12 @@ struct Launcher {
       b.dst_o[k] = h.dstride[d];
       ++k;
     }
-    const uint32_t T = trans_tile(E);
-    b.ta = (b.na + T - 1) / T, b.tb = (b.nb + T - 1) / T;
     const uint64_t align = (uint64_t)(uintptr_t)b.src | (uint64_t)(uintptr_t)b.dst | (uint64_t)b.src_b | (uint64_t)b.dst_a |
                            (uint64_t)b.src_o[0] | (uint64_t)b.src_o[1] | (uint64_t)b.dst_o[0] | (uint64_t)b.dst_o[1] |
                            (uint64_t)b.na * E | (uint64_t)b.nb * E;
     const bool wide = (align & 15) == 0 && E < 16;
+    const TransShape shape = trans_shape(E, wide ? tuning().box_transpose_tile : 0);
+    b.ta = (b.na + shape.a - 1) / shape.a, b.tb = (b.nb + shape.b - 1) / shape.b;
     if (!count_piece()) {
       return true;
     }
@@ -1406,10 +1408,22 @@ void launch_boxes_vec(const Step& st, const CopyArgs& a, hipStream_t stream) {
 template<int E>
 void launch_transposing(const Step& st, const TransArgs& a, hipStream_t stream) {
   dim3 g(st.grid), b(kBlock);
-  if (st.wide) {
-    hipLaunchKernelGGL((transpose_kernel<E, true>), g, b, 0, stream, a);
-  } else {
-    hipLaunchKernelGGL((transpose_kernel<E, false>), g, b, 0, stream, a);
+  constexpr uint32_t T = trans_shape(E, 0).a;
+  if (!st.wide) {
+    hipLaunchKernelGGL((transpose_kernel<E, false, T, T>), g, b, 0, stream, a);
+    return;
+  }
+  if constexpr (E < 16) {
+    // (the shapes other than T x T are measurement variants: the knob box_transpose_tile)
+    if (a.tile_a == T && a.tile_b == 2 * T) {
+      hipLaunchKernelGGL((transpose_kernel<E, true, T, 2 * T>), g, b, 0, stream, a);
+    } else if (a.tile_a == 2 * T && a.tile_b == T) {
+      hipLaunchKernelGGL((transpose_kernel<E, true, 2 * T, T>), g, b, 0, stream, a);
+    } else if (a.tile_a == 2 * T && a.tile_b == 2 * T) {
+      hipLaunchKernelGGL((transpose_kernel<E, true, 2 * T, 2 * T>), g, b, 0, stream, a);
+    } else {
+      hipLaunchKernelGGL((transpose_kernel<E, true, T, T>), g, b, 0, stream, a);
+    }
   }
 }
 
@@ -1868,8 +1882,9 @@ extern "C" int mdh_copy_plan_verify(const mdh_copy_plan* plan, const uint64_t* b
     if (st.kind == Step::kTrans) {
       // one tile per workgroup, every element of every tile through the kernel's own index function
       const TransArgs& a = st.trans;
-      const uint32_t E = (uint32_t)st.vec, T = trans_tile(E);
-      if (st.grid != a.total_tiles || a.nboxes == 0 || a.nboxes > (uint32_t)kMaxTransBoxes) {
+      const uint32_t E = (uint32_t)st.vec;
+      if (st.grid != a.total_tiles || a.nboxes == 0 || a.nboxes > (uint32_t)kMaxTransBoxes || a.tile_a == 0 ||
+          a.tile_b == 0) {
         set_error("mdh_copy_plan_verify: step %zu has a grid of %u workgroups for %u tiles", s, st.grid, a.total_tiles);
         return MDH_EINVAL;
       }
@@ -1888,7 +1903,7 @@ extern "C" int mdh_copy_plan_verify(const mdh_copy_plan* plan, const uint64_t* b
         uint64_t sbase, dbase;
         split(B.src, &ss, &sbase);
         split(B.dst, &ds, &dbase);
-        const uint32_t na = B.na - t.ia < T ? B.na - t.ia : T, nb = B.nb - t.ib < T ? B.nb - t.ib : T;
+        const uint32_t na = B.na - t.ia < a.tile_a ? B.na - t.ia : a.tile_a, nb = B.nb - t.ib < a.tile_b ? B.nb - t.ib : a.tile_b;
         if (st.wide && ((na * E) % 16 != 0 || (nb * E) % 16 != 0 || ((sbase + (uint64_t)t.src_off) & 15) != 0 ||
                            ((dbase + (uint64_t)t.dst_off) & 15) != 0 || (B.src_b & 15) != 0 || (B.dst_a & 15) != 0)) {
           set_error("mdh_copy_plan_verify: step %zu box %u: 16-byte accesses do not fit this box", s, t.box);

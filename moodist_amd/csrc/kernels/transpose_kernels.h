@@ -2,7 +2,7 @@
 // (A) is not the one along which the destination is (B).  Copied vector by vector along either
 // side, such a box coalesces on that side only and moves one element per lane and memory
 // transaction on the other (a 4096 x 4096 fp32 transpose: 107 us, 16 % of the HBM rate).  Here a
-// workgroup takes a tile of T x T elements, reads it along A -- consecutive lanes, consecutive
+// workgroup takes a tile of TA x TB elements, reads it along A -- consecutive lanes, consecutive
 // source bytes --, turns it round in LDS and writes it along B -- consecutive lanes, consecutive
 // destination bytes: both sides move whole 64-byte units.
 //
@@ -40,13 +40,19 @@ struct TransArgs {
   uint32_t nboxes;
   uint32_t total_tiles;
   uint32_t diagonal; // 0: a box's tiles run along A first, then B; 1: along its diagonals (see trans_locate)
+  uint32_t tile_a, tile_b; // elements along a tile's edges (the kernel's template arguments)
 };
 static_assert(sizeof(TransArgs) + 256 <= 4096, "kernel arguments are limited to 4 KiB");
 
-// Elements along a tile's edge: 64 for elements of up to 4 bytes, 32 for 8 and 16 (tiles of
-// 4-16 KiB).
-MDH_HD constexpr uint32_t trans_tile(uint32_t elem) {
-  return elem <= 4 ? 64u : 32u;
+// Elements along a tile's edges, A x B.  Square tiles of 4-16 KiB by default: 64 x 64 for elements
+// of up to 4 bytes, 32 x 32 for 8 and 16.  The shapes the kernel is compiled for are listed in
+// trans_shape(); `which` (the tuning knob box_transpose_tile) picks another one for measurement.
+struct TransShape {
+  uint32_t a, b;
+};
+MDH_HD constexpr TransShape trans_shape(uint32_t elem, int which) {
+  const uint32_t t = elem <= 4 ? 64u : 32u;
+  return which == 1 ? TransShape{t, 2 * t} : which == 2 ? TransShape{2 * t, t} : which == 3 ? TransShape{2 * t, 2 * t} : TransShape{t, t};
 }
 
 struct TransLoc {
@@ -69,7 +75,6 @@ MDH_HD TransLoc trans_locate(const TransArgs& a, uint32_t tile, uint32_t elem) {
   }
   const TransBox& B = a.box[b];
   uint32_t local = tile - start;
-  const uint32_t T = trans_tile(elem);
   // Consecutive workgroups run at the same time.  Along A first, the tiles of a moment share
   // their destination columns: they write a strip 256 bytes wide down every row of the
   // destination, and with a power-of-two pitch that strip lives in a few DRAM channels (along
@@ -90,8 +95,8 @@ MDH_HD TransLoc trans_locate(const TransArgs& a, uint32_t tile, uint32_t elem) {
   const uint32_t o0 = local % B.no[0], o1 = local / B.no[0];
   TransLoc t;
   t.box = b;
-  t.ia = ta_i * T;
-  t.ib = tb_i * T;
+  t.ia = ta_i * a.tile_a;
+  t.ib = tb_i * a.tile_b;
   t.src_off = (int64_t)o0 * B.src_o[0] + (int64_t)o1 * B.src_o[1] + (int64_t)t.ib * B.src_b + (int64_t)t.ia * (int64_t)elem;
   t.dst_off = (int64_t)o0 * B.dst_o[0] + (int64_t)o1 * B.dst_o[1] + (int64_t)t.ia * B.dst_a + (int64_t)t.ib * (int64_t)elem;
   return t;
@@ -120,37 +125,39 @@ struct ElemType<16> {
   using type = u32x4;
 };
 
-// One tile per workgroup.  LDS holds the tile TRANSPOSED, rows along A, each row T elements
-// along B plus 16 bytes of padding (rows stay 16-byte aligned and start in different banks).
+// One tile of TA x TB elements per workgroup.  LDS holds the tile TRANSPOSED, TA rows along A, each
+// row TB elements along B plus 16 bytes of padding (rows stay 16-byte aligned and start in
+// different banks).
 //
 // WIDE: every row of the box starts on the 16-byte grid on both sides and holds a whole number
 // of 16-byte vectors -- the host checks addresses, strides and extents: global memory moves as
 // 16-byte vectors (V = 16 / E elements); going in, a vector's elements are scattered over V
 // rows of LDS, going out, a row of LDS is read 16 bytes at a time.  Otherwise every access is
 // one element: still consecutive lanes on consecutive addresses on both sides, E bytes each.
-template<int E, bool WIDE>
+template<int E, bool WIDE, int TA, int TB>
 __global__ __launch_bounds__(kBlock) void transpose_kernel(TransArgs a) {
   using elem_t = typename ElemType<E>::type;
-  constexpr uint32_t T = trans_tile(E);
-  constexpr uint32_t kPitch = T * E + 16;
-  __shared__ __attribute__((aligned(16))) char tile[T * kPitch];
+  constexpr uint32_t kPitch = TB * E + 16;
+  __shared__ __attribute__((aligned(16))) char tile[TA * kPitch];
   const TransLoc t = trans_locate(a, blockIdx.x, E);
   const TransBox& B = a.box[t.box];
   const char* src = B.src + t.src_off;
   char* dst = B.dst + t.dst_off;
   // what of the tile lies inside the box
-  const uint32_t na = B.na - t.ia < T ? B.na - t.ia : T;
-  const uint32_t nb = B.nb - t.ib < T ? B.nb - t.ib : T;
+  const uint32_t na = B.na - t.ia < (uint32_t)TA ? B.na - t.ia : (uint32_t)TA;
+  const uint32_t nb = B.nb - t.ib < (uint32_t)TB ? B.nb - t.ib : (uint32_t)TB;
   const int64_t src_b = B.src_b, dst_a = B.dst_a;
   if (WIDE) {
-    constexpr uint32_t V = 16 / E;       // elements per vector
-    constexpr uint32_t kRowVecs = T / V; // vectors along a tile's edge
-    constexpr uint32_t kPerLane = T * kRowVecs / kBlock;
+    constexpr uint32_t V = 16 / E;      // elements per vector
+    constexpr uint32_t kVecsA = TA / V; // vectors along A: a source row of the tile
+    constexpr uint32_t kVecsB = TB / V; // vectors along B: a destination row of the tile
+    constexpr uint32_t kPerLane = TB * kVecsA / kBlock;
+    static_assert(TB * kVecsA % kBlock == 0 && TA * kVecsB == TB * kVecsA, "whole vectors per lane");
     u32x4 v[kPerLane];
 #pragma unroll
     for (uint32_t i = 0; i < kPerLane; ++i) {
       const uint32_t idx = i * kBlock + threadIdx.x;
-      const uint32_t row_b = idx / kRowVecs, col = idx % kRowVecs;
+      const uint32_t row_b = idx / kVecsA, col = idx % kVecsA;
       v[i] = u32x4{0, 0, 0, 0};
       if (row_b < nb && col * V < na) {
         v[i] = stream_load((const u32x4*)(src + (int64_t)row_b * src_b + (int64_t)col * 16));
@@ -159,7 +166,7 @@ __global__ __launch_bounds__(kBlock) void transpose_kernel(TransArgs a) {
 #pragma unroll
     for (uint32_t i = 0; i < kPerLane; ++i) {
       const uint32_t idx = i * kBlock + threadIdx.x;
-      const uint32_t row_b = idx / kRowVecs, col = idx % kRowVecs;
+      const uint32_t row_b = idx / kVecsA, col = idx % kVecsA;
       elem_t e[V];
       __builtin_memcpy(e, &v[i], 16);
 #pragma unroll
@@ -171,14 +178,14 @@ __global__ __launch_bounds__(kBlock) void transpose_kernel(TransArgs a) {
 #pragma unroll
     for (uint32_t i = 0; i < kPerLane; ++i) {
       const uint32_t idx = i * kBlock + threadIdx.x;
-      const uint32_t row_a = idx / kRowVecs, col = idx % kRowVecs;
+      const uint32_t row_a = idx / kVecsB, col = idx % kVecsB;
       if (row_a < na && col * V < nb) {
         const u32x4 out = *(const u32x4*)(tile + row_a * kPitch + col * 16);
         stream_store((u32x4*)(dst + (int64_t)row_a * dst_a + (int64_t)col * 16), out);
       }
     }
   } else {
-    constexpr uint32_t kPerLane = T * T / kBlock;
+    constexpr uint32_t kPerLane = TA * TB / kBlock;
     // (loads in batches of eight: sixteen or more in flight per lane buy nothing here)
     constexpr uint32_t kBatch = kPerLane < 8 ? kPerLane : 8;
     for (uint32_t i0 = 0; i0 < kPerLane; i0 += kBatch) {
@@ -186,7 +193,7 @@ __global__ __launch_bounds__(kBlock) void transpose_kernel(TransArgs a) {
 #pragma unroll
       for (uint32_t i = 0; i < kBatch; ++i) {
         const uint32_t idx = (i0 + i) * kBlock + threadIdx.x;
-        const uint32_t row_b = idx / T, col_a = idx % T;
+        const uint32_t row_b = idx / TA, col_a = idx % TA;
         e[i] = elem_t{};
         if (row_b < nb && col_a < na) {
           e[i] = stream_load((const elem_t*)(src + (int64_t)row_b * src_b + (int64_t)col_a * E));
@@ -195,7 +202,7 @@ __global__ __launch_bounds__(kBlock) void transpose_kernel(TransArgs a) {
 #pragma unroll
       for (uint32_t i = 0; i < kBatch; ++i) {
         const uint32_t idx = (i0 + i) * kBlock + threadIdx.x;
-        const uint32_t row_b = idx / T, col_a = idx % T;
+        const uint32_t row_b = idx / TA, col_a = idx % TA;
         *(elem_t*)(tile + col_a * kPitch + row_b * E) = e[i];
       }
     }
@@ -203,7 +210,7 @@ __global__ __launch_bounds__(kBlock) void transpose_kernel(TransArgs a) {
 #pragma unroll
     for (uint32_t i = 0; i < kPerLane; ++i) {
       const uint32_t idx = i * kBlock + threadIdx.x;
-      const uint32_t row_a = idx / T, col_b = idx % T;
+      const uint32_t row_a = idx / TB, col_b = idx % TB;
       if (row_a < na && col_b < nb) {
         const elem_t out = *(const elem_t*)(tile + row_a * kPitch + col_b * E);
         stream_store((elem_t*)(dst + (int64_t)row_a * dst_a + (int64_t)col_b * E), out);
