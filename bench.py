@@ -19,6 +19,7 @@ not in the 256 MB Infinity Cache either.  Prints one JSON line.
     rows:<boxes>:<rows per box>:<run bytes>:<source pitch bytes>    strided rows into a dense destination
     transpose:<rows>:<cols>:<itemsize>                              2-D element transpose
     coalesced:<tensors>:<elements>[:loop]                           allreduce_coalesced of eight local ranks
+    reduce_many:<jobs>:<sources>:<elements>[:single]                a list of reductions in shared launches
 """
 
 import argparse
@@ -92,7 +93,7 @@ def build_workload(name, torch, abi, dev, rotation_bytes):
         # at most 512 sets: launches that touch less than 8 MiB rotate over less than 4 GiB
         return min(512, max(2, -(-rotation_bytes // touched_bytes)))
 
-    if name.startswith("reduce"):
+    if name.startswith("reduce") and not name.startswith("reduce_many:"):
         # reduce_fp32_p8 (headline), reduce_bf16_p16, reduce_fp32_p64_{sum,avg,max}
         spec = {
             "reduce_fp32_p8": (8, 4194304, torch.float32, abi.DTYPE_FLOAT32, abi.OP_SUM, "randn", 1.0),
@@ -274,6 +275,52 @@ def build_workload(name, torch, abi, dev, rotation_bytes):
                 # enqueued behind a long blocker kernel so that the GPU runs them back to back
                 "queue_prefilled": True}
         return desc, set_bytes, launch, check, box_kernel(abi)
+
+    if name.startswith("reduce_many:"):
+        # reduce_many:<jobs>:<sources>:<elements>[:single] -- a list of fp32 SUM reductions of that many
+        # elements each in one call of mdh_reduce_many (shared launches); with ":single", the same
+        # jobs as one mdh_reduce call each.  A step is the whole list.
+        parts = name.split(":")
+        J, P, N = int(parts[1]), int(parts[2]), int(parts[3])
+        single = len(parts) > 4 and parts[4] == "single"
+        set_bytes = J * (P + 1) * N * 4
+        nsets = nsets_for(set_bytes)
+        g = torch.Generator().manual_seed(6)
+        base = [[torch.rand(N, generator=g) * 2 - 1 for _ in range(P)] for _ in range(J)]
+        on_device = [[t.to(dev) for t in job] for job in base]
+        sets = [on_device] + [[[t.clone() for t in job] for job in on_device] for _ in range(nsets - 1)]
+        outs = [[torch.empty(N, device=dev) for _ in range(J)] for _ in range(nsets)]
+        tables = [abi.reduce_jobs([([t.data_ptr() for t in sets[k][j]], j % P, outs[k][j].data_ptr(), N) for j in range(J)])
+                  for k in range(nsets)]
+        singles = [[(abi.ptr_table([t.data_ptr() for t in sets[k][j]]), P, j % P, outs[k][j].data_ptr(), N,
+                     abi.DTYPE_FLOAT32, abi.OP_SUM, 1.0, stream) for j in range(J)] for k in range(nsets)]
+
+        def launch(i):
+            k = i % nsets
+            if single:
+                for call in singles[k]:
+                    rc = L.mdh_reduce(*call)
+                    if rc:
+                        abi.check(rc)
+            else:
+                rc = L.mdh_reduce_many(tables[k][0], J, abi.DTYPE_FLOAT32, abi.OP_SUM, 1.0, stream)
+                if rc:
+                    abi.check(rc)
+
+        def check():
+            import numpy as np
+
+            import oracle
+
+            for j in range(J):
+                want = oracle.reduce([t.numpy() for t in base[j]], j % P, oracle.DT_F32, oracle.OP_SUM)
+                for k in range(nsets):
+                    if not np.array_equal(outs[k][j].cpu().numpy().view(np.uint32), want.view(np.uint32)):
+                        raise SystemExit("bench: result differs from the oracle")
+
+        desc = {"workload": name, "op": "a list of reductions, " + ("one launch per job" if single else "shared launches"),
+                "jobs": J, "sources": P, "numel": N, "dtype": "float32", "buffer_sets": nsets}
+        return desc, set_bytes, launch, check, "reduce_vec_kernel" if single else "reduce_many_kernel"
 
     if name.startswith("coalesced:"):
         # coalesced:<tensors>:<elements>[:loop] -- allreduce_coalesced (MAX, fp32, in place) of a list of
