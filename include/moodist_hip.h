@@ -122,8 +122,8 @@ int mdh_reduce(const void* const* srcs, int nsrc, int first, void* dst, size_t n
  * reduce_scatter_tensor_coalesced, :182-191 for allreduce_coalesced; the fold of each is
  * core/reduce_scatter.cc:104-142).  Launches of a few KiB to a few MiB are bound by the launch
  * itself, so the jobs share launches: up to 40 jobs and 320 source pointers per launch, their
- * tiles numbered through.  A job of 8 MiB per source and more gets a launch of its own, shaped
- * as mdh_reduce shapes it.  Jobs with numel == 0 are skipped.
+ * tiles numbered through, about 96 MiB of every source at most.  A job of 16 MiB per source and
+ * more gets a launch of its own, shaped as mdh_reduce shapes it.  Jobs with numel == 0 are skipped.
  *
  * The jobs must be independent: no job's destination may overlap another job's sources or
  * destination (within a job, dst may equal srcs[first], as for mdh_reduce).  Every job is

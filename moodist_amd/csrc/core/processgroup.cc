@@ -367,7 +367,7 @@ std::shared_ptr<Collective> ProcessGroup::reduce_scatter(const moodist_tensor* o
 // and stores the three options without reading them.  Here they are honoured: chunk_size (bytes,
 // rounded up to 4096) or else num_chunks (through the arithmetic above) cut a reduce_scatter's
 // reduction into pieces, and method 2 ("direct") asks for the reference's own piece count when
-// neither is set.  Pieces shorter than 8 MiB share launches (mdh_reduce_many).
+// neither is set.  Pieces shorter than 16 MiB share launches (mdh_reduce_many).
 size_t ProcessGroup::chunk_bytes_for(size_t bytes) const {
   size_t chunk = 0;
   if (options.chunkSize > 0) {

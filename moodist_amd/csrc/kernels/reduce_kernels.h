@@ -715,10 +715,14 @@ int launch_many_typed(const ManyJob* jobs, int njobs, int mode, float scale, hip
   constexpr uint64_t kPerVec = 16 / sizeof(elem_t);
   int at = 0;
   while (at < njobs) {
-    // how many jobs this launch takes
+    // How many jobs this launch takes: what the tables hold, and no more than about kSplitTiles
+    // tiles of 16 KiB -- over more tiles per wave the waves drift apart like those of one long
+    // reduction (40 jobs of 8 x 4 MiB in one launch: 73.8 % of the HBM rate, 8 such jobs: 77.7 %).
     int end = at, pointers = 0;
     uint64_t vectors = 0;
-    while (end < njobs && end - at < kManyJobs && pointers + jobs[end].nsrc <= kManyPointers) {
+    constexpr uint64_t kLaunchVectors = (kSplitTiles + kSplitTiles / 2) * (uint64_t)kWave * 16;
+    while (end < njobs && end - at < kManyJobs && pointers + jobs[end].nsrc <= kManyPointers &&
+           (end == at || vectors + jobs[end].numel / kPerVec <= kLaunchVectors)) {
       pointers += jobs[end].nsrc;
       vectors += jobs[end].numel / kPerVec;
       ++end;
@@ -754,8 +758,10 @@ int launch_many_typed(const ManyJob* jobs, int njobs, int mode, float scale, hip
     }
     a.njobs = (uint32_t)(end - at);
     a.total_tiles = (uint32_t)tiles;
-    // up to two tiles per SIMD a wave per tile, beyond that 1024 waves walk the tiles
-    a.tile_waves = (uint32_t)(tiles >= 2048 ? 1024 : tiles);
+    // up to two tiles per SIMD a wave per tile, beyond that the waves walk the tiles, as many of
+    // them as a single reduction of that many tiles gets (choose_shape)
+    constexpr bool half = sizeof(elem_t) == 2;
+    a.tile_waves = (uint32_t)(half ? (tiles >= 4096 ? 512 : tiles >= 2048 ? 1024 : tiles) : (tiles >= 2048 ? 512 : tiles));
     if (tuning().reduce_max_blocks > 0 && a.tile_waves > (uint32_t)tuning().reduce_max_blocks) {
       a.tile_waves = (uint32_t)tuning().reduce_max_blocks;
     }

@@ -75,9 +75,10 @@ def test_operands_off_every_grid(dev):
 
 
 def test_a_long_job_in_the_list_gets_its_own_launch(dev):
-    # 8 MiB per source and more leaves the shared launches; results are the same either way
-    n_big = (8 << 20) // 4 + 3
-    specs = [(4, 1000, 1), (4, n_big, 2), (4, 77, 0), (4, (1 << 20) + 1, 3)]
+    # 16 MiB per source and more leaves the shared launches; results are the same either way.  The
+    # 12 and 15 MiB jobs stay in them and, with the 4 MiB one, fill more than one launch's share of tiles.
+    n_big = (16 << 20) // 4 + 3
+    specs = [(4, 1000, 1), (4, n_big, 2), (4, 77, 0), (4, (1 << 20) + 1, 3), (8, (3 << 20) + 5, 7), (8, (15 << 20) // 4, 0)]
     run_jobs(dev, torch.float32, oracle.OP_SUM, specs, 1.0)
     run_jobs(dev, torch.float32, oracle.OP_MAX, specs, 1.0)
 
