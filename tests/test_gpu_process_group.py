@@ -350,6 +350,40 @@ def test_ranks_on_different_streams(world, dev):
         assert torch.equal(outs[r], torch.full((n,), 36.0, device=dev))
 
 
+@pytest.mark.parametrize("n", [1000, 100_000, 600_000])
+def test_ranks_on_two_streams_share_launches_stream_by_stream(world, dev, n):
+    # ranks 0-3 post on one stream, ranks 4-7 on another: short collectives (the first two sizes)
+    # go out as one launch per stream with a job per rank, long ones as one launch per rank; either
+    # way every rank's data is produced on its own stream and must be seen by all launches
+    streams = [torch.cuda.Stream(device=dev), torch.cuda.Stream(device=dev)]
+    host = [torch.stack(random_sources(P, n, torch.float32, seed=7 * r + n)).reshape(-1) for r in range(P)]
+    ins, outs, full, sums = [None] * P, [None] * P, [None] * P, [None] * P
+    torch.cuda.synchronize()
+    works = []
+    for r, pg in enumerate(world):
+        with torch.cuda.stream(streams[r // 4]):
+            ins[r] = host[r].to(dev, non_blocking=False) * 1.0  # produced on the rank's stream
+            outs[r] = torch.zeros(n, device=dev)
+            works.append(pg._reduce_scatter_base(outs[r], ins[r]))
+    for r, pg in enumerate(world):
+        with torch.cuda.stream(streams[r // 4]):
+            full[r] = torch.zeros(P * n, device=dev)
+            works.append(pg._allgather_base(full[r], outs[r]))
+    for r, pg in enumerate(world):
+        with torch.cuda.stream(streams[r // 4]):
+            sums[r] = ins[r].clone()
+            works.append(pg.allreduce([sums[r]]))
+    for w in works:
+        w.wait()
+    torch.cuda.synchronize()
+    chunks = [oracle.reduce([bits(host[j][q * n:(q + 1) * n]) for j in range(P)], q, oracle.DT_F32, oracle.OP_SUM)
+              for q in range(P)]
+    for q in range(P):
+        assert same_bits(bits(outs[q]), chunks[q]), q
+        assert same_bits(bits(full[q]), np.concatenate(chunks)), q
+        assert same_bits(bits(sums[q]), np.concatenate(chunks)), q
+
+
 # ---- reference tests/test_stress.py ----
 
 def test_stress_rapid_collectives(world, dev):
