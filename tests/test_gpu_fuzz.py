@@ -248,3 +248,98 @@ def test_process_group_random_sequences_match_the_oracle(dev):
                                                      TORCH_TO_CODE[dtype], ops[name][1], 1.0) for q in range(P)])[:n]
                 for r in range(P):
                     assert same_bits(bits(ts[r]), want), what + (name, r)
+
+
+def test_process_group_random_coalesced_sequences_match_the_oracle(dev):
+    # random worlds running random sequences of the coalesced collectives (lists of 1..12 tensors of
+    # random sizes, one or two element types), with random chunk options on the groups and the ranks
+    # spread over one, two or as many streams as ranks: results against the oracle's composition,
+    # tensor by tensor
+    rng = random.Random(11)
+    dts = [torch.float32, torch.float64, torch.int32, torch.int64, torch.bfloat16, torch.float16]
+    ops = {"SUM": (dist.ReduceOp.SUM, oracle.OP_SUM), "MIN": (dist.ReduceOp.MIN, oracle.OP_MIN),
+           "MAX": (dist.ReduceOp.MAX, oracle.OP_MAX), "AVG": (dist.ReduceOp.AVG, oracle.OP_AVG)}
+    for case in range(40):
+        P = rng.choice([1, 2, 3, 4, 8, 16])
+        world = moodist_amd.LocalWorld(P, dev)
+        nstreams = rng.choice([1, 1, 2, P])
+        streams = [torch.cuda.Stream(device=dev) for _ in range(nstreams)]
+        option = rng.choice([None, None, ("num_chunks", rng.choice([2, 3, 7])), ("chunk_size", rng.choice([4096, 65536])),
+                             ("method", 2)])
+        if option:
+            for pg in world:
+                setattr(pg.options(), option[0], option[1])
+        for step in range(rng.randint(1, 4)):
+            kind = rng.choice(["rsc", "agc", "arc"])
+            T = rng.randint(1, 12)
+            dtypes = [rng.choice(dts)] * T
+            if rng.random() < 0.25 and T > 1:
+                dtypes[rng.randrange(T)] = rng.choice(dts)  # a second element type somewhere in the list
+            sizes = [rng.choice([1, 2, 5, 64, 1000, 4097, rng.randint(1, 30000)]) for _ in range(T)]
+            g = torch.Generator().manual_seed(case * 1000 + step)
+
+            def rnd(m, dtype):
+                if dtype.is_floating_point:
+                    return (torch.randn(m, generator=g) * 3).to(dtype)
+                return torch.randint(-1000, 1000, (m,), generator=g).to(dtype)
+
+            name = rng.choice(list(ops))
+            if name == "AVG" and not all(dt.is_floating_point for dt in dtypes):
+                name = "SUM"
+            scale = float(np.float32(1.0) / np.float32(P))
+            what = (case, step, kind, P, nstreams, option, T, name)
+            torch.cuda.synchronize()
+            works = []
+            if kind == "rsc":
+                ins = [[rnd(n * P, dt) for n, dt in zip(sizes, dtypes)] for _ in range(P)]
+                d_in = [[t.to(dev) for t in row] for row in ins]
+                outs = [[torch.zeros(n, dtype=dt, device=dev) for n, dt in zip(sizes, dtypes)] for _ in range(P)]
+                opts = dist.ReduceScatterOptions()
+                opts.reduceOp = ops[name][0]
+                torch.cuda.synchronize()
+                for r, pg in enumerate(world):
+                    with torch.cuda.stream(streams[r % nstreams]):
+                        works.append(pg.reduce_scatter_tensor_coalesced(outs[r], d_in[r], opts))
+                for w in works:
+                    w.wait()
+                torch.cuda.synchronize()
+                for k, (n, dt) in enumerate(zip(sizes, dtypes)):
+                    for r in range(P):
+                        want = oracle.reduce([bits(ins[j][k][r * n:(r + 1) * n]) for j in range(P)], r, TORCH_TO_CODE[dt],
+                                             ops[name][1], scale)
+                        assert same_bits(bits(outs[r][k]), want), what + (k, r)
+            elif kind == "agc":
+                ins = [[rnd(n, dt) for n, dt in zip(sizes, dtypes)] for _ in range(P)]
+                d_in = [[t.to(dev) for t in row] for row in ins]
+                outs = [[torch.zeros(n * P, dtype=dt, device=dev) for n, dt in zip(sizes, dtypes)] for _ in range(P)]
+                torch.cuda.synchronize()
+                for r, pg in enumerate(world):
+                    with torch.cuda.stream(streams[r % nstreams]):
+                        works.append(pg.allgather_into_tensor_coalesced(outs[r], d_in[r]))
+                for w in works:
+                    w.wait()
+                torch.cuda.synchronize()
+                for k in range(T):
+                    want = bits(torch.cat([ins[j][k] for j in range(P)]))
+                    for r in range(P):
+                        assert same_bits(bits(outs[r][k]), want), what + (k, r)
+            else:
+                ins = [[rnd(n, dt) for n, dt in zip(sizes, dtypes)] for _ in range(P)]
+                ts = [[t.to(dev) for t in row] for row in ins]
+                opts = dist.AllreduceCoalescedOptions()
+                opts.reduceOp = ops[name][0]
+                torch.cuda.synchronize()
+                for r, pg in enumerate(world):
+                    with torch.cuda.stream(streams[r % nstreams]):
+                        works.append(pg.allreduce_coalesced(ts[r], opts))
+                for w in works:
+                    w.wait()
+                torch.cuda.synchronize()
+                for k, (n, dt) in enumerate(zip(sizes, dtypes)):
+                    padded = (n + P - 1) // P * P
+                    c = padded // P
+                    pin = [torch.cat([ins[j][k], torch.zeros(padded - n, dtype=dt)]) for j in range(P)]
+                    want = np.concatenate([oracle.reduce([bits(t[q * c:(q + 1) * c]) for t in pin], q, TORCH_TO_CODE[dt],
+                                                         ops[name][1], scale) for q in range(P)])[:n]
+                    for r in range(P):
+                        assert same_bits(bits(ts[r][k]), want), what + (k, r)
