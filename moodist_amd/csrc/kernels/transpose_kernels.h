@@ -125,19 +125,26 @@ struct ElemType<16> {
   using type = u32x4;
 };
 
-// One tile of TA x TB elements per workgroup.  LDS holds the tile TRANSPOSED, TA rows along A, each
-// row TB elements along B plus 16 bytes of padding (rows stay 16-byte aligned and start in
-// different banks).
+// One tile of TA x TB elements per workgroup.  LDS holds the tile TRANSPOSED: TA rows along A, each
+// row TB elements along B.
 //
 // WIDE: every row of the box starts on the 16-byte grid on both sides and holds a whole number
 // of 16-byte vectors -- the host checks addresses, strides and extents: global memory moves as
 // 16-byte vectors (V = 16 / E elements); going in, a vector's elements are scattered over V
-// rows of LDS, going out, a row of LDS is read 16 bytes at a time.  Otherwise every access is
-// one element: still consecutive lanes on consecutive addresses on both sides, E bytes each.
+// rows of LDS, going out, a row of LDS is read 16 bytes at a time.  The rows carry no padding;
+// instead the 16-byte vectors of a row are permuted: vector j of row a sits at position
+// j ^ (a / V mod vectors per row).  A wave's scatter -- one element each to V-th rows, a few
+// neighbouring columns -- then lands in as many banks as it has lanes (with rows padded by 16
+// bytes, whatever keeps them aligned, it took 4 to 8 turns per instruction), and the 16-byte
+// reads of whole rows touch every bank once either way.
+//
+// Otherwise every access is one element: still consecutive lanes on consecutive addresses on
+// both sides, E bytes each; rows are padded by one bank (4 bytes; 8 and 16 for elements of that
+// size, which must stay aligned), so that a column of the tile walks through all banks.
 template<int E, bool WIDE, int TA, int TB>
 __global__ __launch_bounds__(kBlock) void transpose_kernel(TransArgs a) {
   using elem_t = typename ElemType<E>::type;
-  constexpr uint32_t kPitch = TB * E + 16;
+  constexpr uint32_t kPitch = WIDE ? TB * E : TB * E + (E <= 4 ? 4 : E);
   __shared__ __attribute__((aligned(16))) char tile[TA * kPitch];
   const TransLoc t = trans_locate(a, blockIdx.x, E);
   const TransBox& B = a.box[t.box];
@@ -169,9 +176,11 @@ __global__ __launch_bounds__(kBlock) void transpose_kernel(TransArgs a) {
       const uint32_t row_b = idx / kVecsA, col = idx % kVecsA;
       elem_t e[V];
       __builtin_memcpy(e, &v[i], 16);
+      // rows col * V ... + V - 1 share one permutation: a / V = col
+      const uint32_t at = ((row_b / V) ^ (col % kVecsB)) * 16 + (row_b % V) * E;
 #pragma unroll
       for (uint32_t k = 0; k < V; ++k) {
-        *(elem_t*)(tile + (col * V + k) * kPitch + row_b * E) = e[k];
+        *(elem_t*)(tile + (col * V + k) * kPitch + at) = e[k];
       }
     }
     __syncthreads();
@@ -180,7 +189,7 @@ __global__ __launch_bounds__(kBlock) void transpose_kernel(TransArgs a) {
       const uint32_t idx = i * kBlock + threadIdx.x;
       const uint32_t row_a = idx / kVecsB, col = idx % kVecsB;
       if (row_a < na && col * V < nb) {
-        const u32x4 out = *(const u32x4*)(tile + row_a * kPitch + col * 16);
+        const u32x4 out = *(const u32x4*)(tile + row_a * kPitch + (col ^ (row_a / V % kVecsB)) * 16);
         stream_store((u32x4*)(dst + (int64_t)row_a * dst_a + (int64_t)col * 16), out);
       }
     }
