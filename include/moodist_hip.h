@@ -261,7 +261,9 @@ int mdh_static_workspace(void** address, size_t* bytes);
  * strided-box kernel: 1 = plain, which pays when the sources are still in the Infinity Cache;
  * 0 or 2 = nt, the default), "box_preload" (1 = never start equal boxes of full tiles from
  * preloaded kernel arguments), "box_transpose" (1 = boxes that transpose take the plain strided
- * kernel instead of LDS-staged tiles; 2 = tiles, dealt row by row instead of along the diagonals), "box_transpose_tile" (0..3: the tile
+ * kernel instead of LDS-staged tiles; 2 = tiles, always dealt row by row; 3 = always along the
+ * diagonals; by default the destination's pitch decides), "box_transpose_wgs" (workgroups that walk the tiles of a transposing
+ * launch, each taking every grid-th tile; 0 = one workgroup per tile), "box_transpose_tile" (0..3: the tile
  * of the transposing copy, T x T, T x 2T, 2T x T or 2T x 2T elements, for measurement), "box_tile_cols" (a power of two: the columns, in 16-byte vectors, of
  * a strided-box tile; its rows follow from the tile's 256 x box_unroll slots), four variants of the dense copy of up to eight equal segments that
  * exist for measurement and that the library never chooses by itself -- "copy_xcd_run" (2, 4, 8, ...:

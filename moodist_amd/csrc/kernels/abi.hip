@@ -122,6 +122,9 @@ int* knob(const char* name) {
   if (!std::strcmp(name, "box_transpose")) {
     return &t.box_transpose;
   }
+  if (!std::strcmp(name, "box_transpose_wgs")) {
+    return &t.box_transpose_wgs;
+  }
   if (!std::strcmp(name, "box_tile_cols")) {
     return &t.box_tile_cols;
   }
@@ -166,7 +169,7 @@ extern "C" int mdh_set_tuning(const char* name, int value) {
       return MDH_EINVAL;
     }
   } else if (value < 0 || (std::strstr(name, "wg_per_cu") && value > 9) || (!std::strcmp(name, "box_policy") && value > 2) ||
-             (!std::strcmp(name, "box_preload") && value > 1) || (!std::strcmp(name, "box_transpose") && value > 2) || (!std::strcmp(name, "box_transpose_tile") && value > 3) || (!std::strcmp(name, "allow_capture") && value > 1)) {
+             (!std::strcmp(name, "box_preload") && value > 1) || (!std::strcmp(name, "box_transpose") && value > 3) || (!std::strcmp(name, "box_transpose_tile") && value > 3) || (!std::strcmp(name, "allow_capture") && value > 1)) {
     mdh::set_error("mdh_set_tuning: %s does not take %d", name, value);
     return MDH_EINVAL;
   }

@@ -1110,11 +1110,16 @@ struct Launcher {
             ++i;
           }
           a.total_tiles = (uint32_t)tiles;
-          a.diagonal = tuning().box_transpose == 2 ? 0u : 1u;
           const TransShape shape = trans_shape(1u << lg, wide ? tuning().box_transpose_tile : 0);
           a.tile_a = shape.a, a.tile_b = shape.b;
           Step st;
-          st.kind = Step::kTrans, st.vec = 1 << lg, st.unroll = 1, st.grid = a.total_tiles, st.grid_y = 0, st.lds = 0;
+          st.kind = Step::kTrans, st.vec = 1 << lg, st.unroll = 1, st.grid_y = 0, st.lds = 0;
+          // One workgroup per tile.  (The kernel can walk: with fewer workgroups each takes every
+          // grid-th tile and has the next one's loads under way while it stores the current one.
+          // Measured, eight resident workgroups per CU walking lose 3-14 % against a fresh
+          // workgroup per tile; the knob remains for measurement.)
+          const uint32_t walkers = tuning().box_transpose_wgs > 0 ? (uint32_t)tuning().box_transpose_wgs : a.total_tiles;
+          st.grid = a.total_tiles < walkers ? a.total_tiles : walkers;
           st.plain_loads = false, st.wide = wide != 0;
           submit(st, nullptr, nullptr, &a);
         }
@@ -1137,6 +1142,8 @@ struct Launcher {
   // long (below that a tile would be mostly empty, and the plain kernel, which then still
   // coalesces on one side, is no worse), and at most two other extents may remain.
   static constexpr int64_t kMinTransExtent = 16;
+  // a destination pitch that is a multiple of this puts a column of tiles into few DRAM channels
+  static constexpr int64_t kCrowdingPitch = 4096;
 
   bool try_transposing(const HostBox& h) {
     if (tuning().box_transpose == 1 || h.nd < 2 || h.nd > 2 + kTransBatchDims || h.run > 16 || (h.run & (h.run - 1)) != 0) {
@@ -1181,6 +1188,8 @@ struct Launcher {
     const bool wide = (align & 15) == 0 && E < 16;
     const TransShape shape = trans_shape(E, wide ? tuning().box_transpose_tile : 0);
     b.ta = (b.na + shape.a - 1) / shape.a, b.tb = (b.nb + shape.b - 1) / shape.b;
+    // the order of the tiles: see trans_locate
+    b.diagonal = tuning().box_transpose == 2 ? 0u : tuning().box_transpose == 3 ? 1u : b.dst_a % kCrowdingPitch == 0 ? 1u : 0u;
     if (!count_piece()) {
       return true;
     }
@@ -1883,7 +1892,7 @@ extern "C" int mdh_copy_plan_verify(const mdh_copy_plan* plan, const uint64_t* b
       // one tile per workgroup, every element of every tile through the kernel's own index function
       const TransArgs& a = st.trans;
       const uint32_t E = (uint32_t)st.vec;
-      if (st.grid != a.total_tiles || a.nboxes == 0 || a.nboxes > (uint32_t)kMaxTransBoxes || a.tile_a == 0 ||
+      if (st.grid == 0 || st.grid > a.total_tiles || a.nboxes == 0 || a.nboxes > (uint32_t)kMaxTransBoxes || a.tile_a == 0 ||
           a.tile_b == 0) {
         set_error("mdh_copy_plan_verify: step %zu has a grid of %u workgroups for %u tiles", s, st.grid, a.total_tiles);
         return MDH_EINVAL;

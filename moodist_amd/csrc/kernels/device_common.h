@@ -98,7 +98,8 @@ struct Tuning {
   int copy_wg_per_cu = 0; // as reduce_wg_per_cu, for the copy kernels
   int box_policy = 0;     // loads of the strided-box kernel: 1 plain, 0 or 2 nt
   int box_tile_cols = 0;  // columns (16-byte vectors) of a strided-box tile, a power of two; the tile's rows follow
-  int box_transpose = 0;  // 1: transposing boxes take the plain strided kernel instead of LDS-staged tiles; 2: tiles dealt row by row
+  int box_transpose = 0;  // 1: transposing boxes take the plain strided kernel instead of LDS-staged tiles; 2: tiles always dealt row by row; 3: always along the diagonals
+  int box_transpose_wgs = 0; // workgroups that walk the tiles of a transposing launch (0 = one per tile)
   int box_transpose_tile = 0; // tile of the transposing copy with 16-byte accesses: 0 T x T, 1 T x 2T, 2 2T x T, 3 2T x 2T (A x B)
   int box_preload = 0;    // 1: never launch equal boxes of full tiles from preloaded arguments
   // measurement variants of the dense copy of up to eight equal segments (see copy_flat8_kernel)

@@ -11,6 +11,8 @@
 // never transposes, and its Copy is an {offset, shape} box of a contiguous tensor
 // (core/cputhread.h:306-310).  mdh_copy_boxes takes any strides, transposing ones included.
 #pragma once
+#include <type_traits>
+
 #include "device_common.h"
 
 namespace mdh {
@@ -32,6 +34,8 @@ struct TransBox {
   uint32_t na, nb; // elements along A and B
   uint32_t no[kTransBatchDims];
   uint32_t ta, tb; // tiles along A and B
+  uint32_t diagonal; // 0: the tiles run along A first, then B; 1: along the diagonals (see trans_locate)
+  uint32_t reserved;
 };
 
 struct TransArgs {
@@ -39,7 +43,6 @@ struct TransArgs {
   uint32_t tile_end[kMaxTransBoxes]; // cumulative tiles; unused entries are ~0
   uint32_t nboxes;
   uint32_t total_tiles;
-  uint32_t diagonal; // 0: a box's tiles run along A first, then B; 1: along its diagonals (see trans_locate)
   uint32_t tile_a, tile_b; // elements along a tile's edges (the kernel's template arguments)
 };
 static_assert(sizeof(TransArgs) + 256 <= 4096, "kernel arguments are limited to 4 KiB");
@@ -75,13 +78,14 @@ MDH_HD TransLoc trans_locate(const TransArgs& a, uint32_t tile, uint32_t elem) {
   }
   const TransBox& B = a.box[b];
   uint32_t local = tile - start;
-  // Consecutive workgroups run at the same time.  Along A first, the tiles of a moment share
-  // their destination columns: they write a strip 256 bytes wide down every row of the
-  // destination, and with a power-of-two pitch that strip lives in a few DRAM channels (along
-  // B first it is the reads).  Along the diagonals -- B advances with every tile and A with it --
-  // both sides spread over rows and columns alike.
+  // Consecutive tiles run at the same time.  Along A first, the tiles of a moment read whole
+  // strips of source rows (every piece of a row is fetched while its neighbours are) and write
+  // one column of the destination's tiles: a strip TB elements wide down every destination row.
+  // When the destination's pitch is a multiple of a large power of two that strip lives in a
+  // few DRAM channels; such boxes go along the diagonals instead -- B advances with every tile
+  // and A with it --, which spreads both sides over rows and columns alike.
   uint32_t ta_i, tb_i;
-  if (a.diagonal) {
+  if (B.diagonal) {
     tb_i = local % B.tb;
     local /= B.tb;
     ta_i = (local % B.ta + tb_i) % B.ta;
@@ -144,87 +148,120 @@ struct ElemType<16> {
 template<int E, bool WIDE, int TA, int TB>
 __global__ __launch_bounds__(kBlock) void transpose_kernel(TransArgs a) {
   using elem_t = typename ElemType<E>::type;
+  constexpr uint32_t V = 16 / E;      // elements per 16-byte vector
+  constexpr uint32_t kVecsA = TA / V; // vectors along A: a source row of the tile
+  constexpr uint32_t kVecsB = TB / V; // vectors along B: a destination row of the tile
   constexpr uint32_t kPitch = WIDE ? TB * E : TB * E + (E <= 4 ? 4 : E);
+  constexpr uint32_t kPerLane = WIDE ? TB * kVecsA / kBlock : TA * TB / kBlock;
+  static_assert(!WIDE || (TB * kVecsA % kBlock == 0 && TA * kVecsB == TB * kVecsA), "whole vectors per lane");
+  static_assert(WIDE || TA * TB % kBlock == 0, "whole elements per lane");
+  using reg_t = typename std::conditional<WIDE, u32x4, elem_t>::type;
   __shared__ __attribute__((aligned(16))) char tile[TA * kPitch];
-  const TransLoc t = trans_locate(a, blockIdx.x, E);
-  const TransBox& B = a.box[t.box];
-  const char* src = B.src + t.src_off;
-  char* dst = B.dst + t.dst_off;
-  // what of the tile lies inside the box
-  const uint32_t na = B.na - t.ia < (uint32_t)TA ? B.na - t.ia : (uint32_t)TA;
-  const uint32_t nb = B.nb - t.ib < (uint32_t)TB ? B.nb - t.ib : (uint32_t)TB;
-  const int64_t src_b = B.src_b, dst_a = B.dst_a;
-  if (WIDE) {
-    constexpr uint32_t V = 16 / E;      // elements per vector
-    constexpr uint32_t kVecsA = TA / V; // vectors along A: a source row of the tile
-    constexpr uint32_t kVecsB = TB / V; // vectors along B: a destination row of the tile
-    constexpr uint32_t kPerLane = TB * kVecsA / kBlock;
-    static_assert(TB * kVecsA % kBlock == 0 && TA * kVecsB == TB * kVecsA, "whole vectors per lane");
-    u32x4 v[kPerLane];
+
+  struct Where {
+    const char* src;
+    char* dst;
+    int64_t src_b, dst_a;
+    uint32_t na, nb; // what of the tile lies inside the box
+  };
+  auto locate = [&](uint32_t index) {
+    const TransLoc t = trans_locate(a, index, E);
+    const TransBox& B = a.box[t.box];
+    Where w;
+    w.src = B.src + t.src_off;
+    w.dst = B.dst + t.dst_off;
+    w.src_b = B.src_b;
+    w.dst_a = B.dst_a;
+    w.na = B.na - t.ia < (uint32_t)TA ? B.na - t.ia : (uint32_t)TA;
+    w.nb = B.nb - t.ib < (uint32_t)TB ? B.nb - t.ib : (uint32_t)TB;
+    return w;
+  };
+
+  // A workgroup takes the tiles blockIdx.x, blockIdx.x + gridDim.x, ... -- as launched by the
+  // library, exactly one.  When there are more, the loads of the next tile are issued as soon as
+  // the registers are free (the current tile sits in LDS by then) and are under way while the
+  // current tile is read out of LDS and stored.
+  reg_t v[kPerLane];
+  auto load = [&](const Where& w) {
 #pragma unroll
     for (uint32_t i = 0; i < kPerLane; ++i) {
       const uint32_t idx = i * kBlock + threadIdx.x;
-      const uint32_t row_b = idx / kVecsA, col = idx % kVecsA;
-      v[i] = u32x4{0, 0, 0, 0};
-      if (row_b < nb && col * V < na) {
-        v[i] = stream_load((const u32x4*)(src + (int64_t)row_b * src_b + (int64_t)col * 16));
-      }
-    }
-#pragma unroll
-    for (uint32_t i = 0; i < kPerLane; ++i) {
-      const uint32_t idx = i * kBlock + threadIdx.x;
-      const uint32_t row_b = idx / kVecsA, col = idx % kVecsA;
-      elem_t e[V];
-      __builtin_memcpy(e, &v[i], 16);
-      // rows col * V ... + V - 1 share one permutation: a / V = col
-      const uint32_t at = ((row_b / V) ^ (col % kVecsB)) * 16 + (row_b % V) * E;
-#pragma unroll
-      for (uint32_t k = 0; k < V; ++k) {
-        *(elem_t*)(tile + (col * V + k) * kPitch + at) = e[k];
-      }
-    }
-    __syncthreads();
-#pragma unroll
-    for (uint32_t i = 0; i < kPerLane; ++i) {
-      const uint32_t idx = i * kBlock + threadIdx.x;
-      const uint32_t row_a = idx / kVecsB, col = idx % kVecsB;
-      if (row_a < na && col * V < nb) {
-        const u32x4 out = *(const u32x4*)(tile + row_a * kPitch + (col ^ (row_a / V % kVecsB)) * 16);
-        stream_store((u32x4*)(dst + (int64_t)row_a * dst_a + (int64_t)col * 16), out);
-      }
-    }
-  } else {
-    constexpr uint32_t kPerLane = TA * TB / kBlock;
-    // (loads in batches of eight: sixteen or more in flight per lane buy nothing here)
-    constexpr uint32_t kBatch = kPerLane < 8 ? kPerLane : 8;
-    for (uint32_t i0 = 0; i0 < kPerLane; i0 += kBatch) {
-      elem_t e[kBatch];
-#pragma unroll
-      for (uint32_t i = 0; i < kBatch; ++i) {
-        const uint32_t idx = (i0 + i) * kBlock + threadIdx.x;
+      v[i] = reg_t{};
+      if constexpr (WIDE) {
+        const uint32_t row_b = idx / kVecsA, col = idx % kVecsA;
+        if (row_b < w.nb && col * V < w.na) {
+          v[i] = stream_load((const reg_t*)(w.src + (int64_t)row_b * w.src_b + (int64_t)col * 16));
+        }
+      } else {
         const uint32_t row_b = idx / TA, col_a = idx % TA;
-        e[i] = elem_t{};
-        if (row_b < nb && col_a < na) {
-          e[i] = stream_load((const elem_t*)(src + (int64_t)row_b * src_b + (int64_t)col_a * E));
+        if (row_b < w.nb && col_a < w.na) {
+          v[i] = stream_load((const reg_t*)(w.src + (int64_t)row_b * w.src_b + (int64_t)col_a * E));
         }
       }
-#pragma unroll
-      for (uint32_t i = 0; i < kBatch; ++i) {
-        const uint32_t idx = (i0 + i) * kBlock + threadIdx.x;
-        const uint32_t row_b = idx / TA, col_a = idx % TA;
-        *(elem_t*)(tile + col_a * kPitch + row_b * E) = e[i];
-      }
     }
-    __syncthreads();
+  };
+  auto scatter = [&]() {
 #pragma unroll
     for (uint32_t i = 0; i < kPerLane; ++i) {
       const uint32_t idx = i * kBlock + threadIdx.x;
-      const uint32_t row_a = idx / TB, col_b = idx % TB;
-      if (row_a < na && col_b < nb) {
-        const elem_t out = *(const elem_t*)(tile + row_a * kPitch + col_b * E);
-        stream_store((elem_t*)(dst + (int64_t)row_a * dst_a + (int64_t)col_b * E), out);
+      if constexpr (WIDE) {
+        const uint32_t row_b = idx / kVecsA, col = idx % kVecsA;
+        elem_t e[V];
+        __builtin_memcpy(e, &v[i], 16);
+        // rows col * V ... + V - 1 share one permutation: a / V = col
+        const uint32_t at = ((row_b / V) ^ (col % kVecsB)) * 16 + (row_b % V) * E;
+#pragma unroll
+        for (uint32_t k = 0; k < V; ++k) {
+          *(elem_t*)(tile + (col * V + k) * kPitch + at) = e[k];
+        }
+      } else {
+        const uint32_t row_b = idx / TA, col_a = idx % TA;
+        elem_t e;
+        __builtin_memcpy(&e, &v[i], E);
+        *(elem_t*)(tile + col_a * kPitch + row_b * E) = e;
       }
     }
+  };
+  auto store = [&](const Where& w) {
+#pragma unroll
+    for (uint32_t i = 0; i < kPerLane; ++i) {
+      const uint32_t idx = i * kBlock + threadIdx.x;
+      if constexpr (WIDE) {
+        const uint32_t row_a = idx / kVecsB, col = idx % kVecsB;
+        if (row_a < w.na && col * V < w.nb) {
+          const u32x4 out = *(const u32x4*)(tile + row_a * kPitch + (col ^ (row_a / V % kVecsB)) * 16);
+          stream_store((u32x4*)(w.dst + (int64_t)row_a * w.dst_a + (int64_t)col * 16), out);
+        }
+      } else {
+        const uint32_t row_a = idx / TB, col_b = idx % TB;
+        if (row_a < w.na && col_b < w.nb) {
+          const elem_t out = *(const elem_t*)(tile + row_a * kPitch + col_b * E);
+          stream_store((elem_t*)(w.dst + (int64_t)row_a * w.dst_a + (int64_t)col_b * E), out);
+        }
+      }
+    }
+  };
+
+  uint32_t index = blockIdx.x;
+  Where cur = locate(index);
+  load(cur);
+  for (;;) {
+    scatter();
+    __syncthreads();
+    const uint32_t next = index + gridDim.x;
+    const bool more = next < a.total_tiles;
+    Where nxt = cur;
+    if (more) {
+      nxt = locate(next);
+      load(nxt);
+    }
+    store(cur);
+    if (!more) {
+      break;
+    }
+    __syncthreads(); // every wave has read the tile out of LDS before the next one goes in
+    cur = nxt;
+    index = next;
   }
 }
 

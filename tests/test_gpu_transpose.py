@@ -19,6 +19,20 @@ def st():
     return torch.cuda.current_stream().cuda_stream
 
 
+@pytest.fixture(params=[(0, 0), (3, 2), (7, 3)], ids=["default", "three_walkers_rows", "seven_walkers_diagonals"], autouse=True)
+def walkers_and_order(request):
+    """Every test of this file runs three times: as the library launches by itself (a workgroup per
+    tile on matrices of this size), and with three and seven workgroups walking all the tiles of a
+    launch -- many tiles per workgroup, ragged ones among them -- in either order of the tiles."""
+    wgs, order = request.param
+    old_wgs, old_order = abi.get_tuning("box_transpose_wgs"), abi.get_tuning("box_transpose")
+    abi.set_tuning("box_transpose_wgs", wgs)
+    abi.set_tuning("box_transpose", order)
+    yield
+    abi.set_tuning("box_transpose_wgs", old_wgs)
+    abi.set_tuning("box_transpose", old_order)
+
+
 def host_array(shape, itemsize, seed):
     rng = np.random.RandomState(seed)
     return rng.randint(0, 256, size=tuple(shape) + (itemsize,)).astype(np.uint8)
@@ -29,11 +43,12 @@ def as_tensor(a, dev):
 
 
 @pytest.mark.parametrize("itemsize", [1, 2, 4, 8, 16])
-@pytest.mark.parametrize("knob", [0, 1])
+@pytest.mark.parametrize("knob", [None, 1])
 def test_two_dimensional_transposes(dev, itemsize, knob):
     old = abi.get_tuning("box_transpose")
     try:
-        abi.set_tuning("box_transpose", knob)
+        if knob is not None:
+            abi.set_tuning("box_transpose", knob)
         # whole tiles, ragged edges, extents just over the threshold, one long and one short side
         for R, C in ((64, 64), (128, 256), (100, 36), (16, 16), (17, 333), (1000, 24), (65, 129), (512, 1024)):
             src = host_array((R, C), itemsize, R * 7 + C)
