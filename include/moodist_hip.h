@@ -139,6 +139,26 @@ typedef struct mdh_reduce_job {
 int mdh_reduce_many(const mdh_reduce_job* jobs, int njobs, int dtype, int op, float scale, void* stream);
 
 /*
+ * The same list of reductions with every job's result stored over ALL of the job's sources:
+ * afterwards each of jobs[j].srcs[0 .. nsrc-1] holds, in its first numel elements, what
+ * mdh_reduce(jobs[j].srcs, nsrc, jobs[j].first, ...) yields, bit for bit.  jobs[j].dst is ignored.
+ *
+ * Replaces: the allreduce of ranks whose tensors one GPU can address (all local ranks of a
+ * process here; with mapped peer memory, the ranks of a node), which the reference composes of
+ * a reduce_scatter into the rank's own chunk and an all_gather of the chunks
+ * (core/processgroup.cc:1674-1722): one job per chunk c, srcs[r] = rank r's tensor + c * chunk,
+ * first = c (the fold order of the rank that owns the chunk, core/group.cc:567-570).  One launch
+ * reads every tensor once and writes every tensor once -- 2 * P * bytes where the composition
+ * moves (3 * P - 1) * bytes in two launches per rank.
+ *
+ * A tile is read from every source before its first store and belongs to one wave, so the
+ * sources are read and overwritten in place.  The sources of a job must not overlap one
+ * another, and the jobs must be independent.  Jobs of any length stay in shared launches
+ * (pieces of 32 MiB per source).  Every job is checked before anything is enqueued.
+ */
+int mdh_allreduce_many(const mdh_reduce_job* jobs, int njobs, int dtype, int op, float scale, void* stream);
+
+/*
  * All-gather chunk assembly: for every shard s < nsrc and row r < rows,
  * copy `width` bytes from srcs[s] + r*src_pitch to
  * dst + s*dst_shard_stride + r*dst_pitch.

@@ -19,7 +19,7 @@ MAX_DIMS = 10
 ABI_VERSION = 2
 
 SYMBOLS = (
-    "mdh_abi_version", "mdh_error_string", "mdh_last_error", "mdh_reduce", "mdh_reduce_many", "mdh_gather", "mdh_copy_boxes",
+    "mdh_abi_version", "mdh_error_string", "mdh_last_error", "mdh_reduce", "mdh_reduce_many", "mdh_allreduce_many", "mdh_gather", "mdh_copy_boxes",
     "mdh_set_tuning", "mdh_get_tuning", "mdh_copy_plan_create", "mdh_copy_plan_launch", "mdh_copy_plan_launches",
     "mdh_copy_plan_verify", "mdh_copy_plan_destroy", "mdh_copy_plan_step_arguments", "mdh_static_workspace",
 )
@@ -75,6 +75,9 @@ def lib():
     L.mdh_reduce_many.argtypes = [ctypes.POINTER(ReduceJob), ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_float,
                                   ctypes.c_void_p]
     L.mdh_reduce_many.restype = ctypes.c_int
+    L.mdh_allreduce_many.argtypes = [ctypes.POINTER(ReduceJob), ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_float,
+                                  ctypes.c_void_p]
+    L.mdh_allreduce_many.restype = ctypes.c_int
     L.mdh_gather.argtypes = [vpp, ctypes.c_int, ctypes.c_void_p] + [ctypes.c_size_t] * 5 + [ctypes.c_void_p]
     L.mdh_gather.restype = ctypes.c_int
     L.mdh_copy_boxes.argtypes = [ctypes.POINTER(Box), ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
@@ -139,6 +142,14 @@ def reduce_many(jobs, dtype, op, scale=1.0, stream=0):
     """jobs: (src_ptrs, first, dst_ptr, numel) tuples, all of one element type and operation."""
     arr, tables = reduce_jobs(jobs)
     check(lib().mdh_reduce_many(arr, len(jobs), dtype, op, scale, stream))
+    del tables
+
+
+def allreduce_many(jobs, dtype, op, scale=1.0, stream=0):
+    """The same list with every job's result stored over all of the job's sources (dst_ptr is
+    ignored)."""
+    arr, tables = reduce_jobs(jobs)
+    check(lib().mdh_allreduce_many(arr, len(jobs), dtype, op, scale, stream))
     del tables
 
 

@@ -81,6 +81,7 @@ HipRuntime load() {
   resolve(kl, kn, "mdh_error_string", r.error_string);
   resolve(kl, kn, "mdh_reduce", r.reduce);
   resolve(kl, kn, "mdh_reduce_many", r.reduce_many);
+  resolve(kl, kn, "mdh_allreduce_many", r.allreduce_many);
   resolve(kl, kn, "mdh_gather", r.gather);
   resolve(kl, kn, "mdh_copy_boxes", r.copy_boxes);
   resolve(kl, kn, "mdh_copy_plan_create", r.copy_plan_create);

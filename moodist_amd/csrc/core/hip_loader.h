@@ -40,6 +40,7 @@ struct HipRuntime {
   decltype(&mdh_error_string) error_string;
   decltype(&mdh_reduce) reduce;
   decltype(&mdh_reduce_many) reduce_many;
+  decltype(&mdh_allreduce_many) allreduce_many;
   decltype(&mdh_gather) gather;
   decltype(&mdh_copy_boxes) copy_boxes;
   decltype(&mdh_copy_plan_create) copy_plan_create;
@@ -50,6 +51,7 @@ struct HipRuntime {
 
 constexpr int kHipMemcpyDeviceToDevice = 3;
 constexpr unsigned kHipEventDisableTiming = 2;
+constexpr int kHipErrorInvalidValue = 1;
 constexpr int kHipErrorStreamCaptureImplicit = 906;
 
 // Loads on first call; throws std::runtime_error naming the missing library or

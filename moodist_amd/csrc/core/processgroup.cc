@@ -431,74 +431,72 @@ std::shared_ptr<Collective> ProcessGroup::reduce_scatter_many(const moodist_tens
              inputs[0].dtype, (uint32_t)n, nullptr);
 }
 
+// allreduce (core/processgroup.cc:1674-1722): a reduce_scatter into this rank's own chunk of the
+// tensor and an all_gather of every rank's chunk; a tensor whose element count the group size
+// does not divide goes through a padded temporary (:1694-1720).  One collective here: when the
+// last rank arrives, the world either runs those two halves rank by rank or, when the ranks share
+// a stream, one launch that reduces every chunk and stores it into every rank's tensor
+// (World::run_allreduce).
 std::shared_ptr<Collective> ProcessGroup::allreduce(const moodist_tensor& tensor, const moodist_tensor* scratch,
     int reduce_op, void* stream, float premul, Keep keep) {
+  Busy guard(*this);
+  refuse_capture_early(stream, "allreduce");
   check_device_tensor(tensor, world->device, "allreduce tensor");
   MD_CHECK(tensor.numel > 0); // core/processgroup.cc:1678
   check_reduce_request(tensor.dtype, reduce_op); // before anything is enqueued or posted
   const int64_t n = tensor.numel;
+  Posting p;
+  p.stream = stream;
+  p.wants_output = true;
+  p.kernel_less = options.forceKernelLess || options.preferKernelLess;
+  size_t bytes = 0; // one chunk
   if (n % size == 0) {
-    // in place: reduce into this rank's own chunk, then gather every rank's chunk (:1686-1693)
-    moodist_tensor chunk = tensor;
-    chunk.numel = n / size;
-    chunk.data = (char*)tensor.data + (size_t)rank * (size_t)chunk.numel * (size_t)tensor.itemsize;
-    chunk.ndim = 1;
-    chunk.shape[0] = chunk.numel;
-    reduce_scatter(&chunk, tensor, reduce_op, stream, premul, keep); // both halves hold the tensor
-    // the gather's input is what the reduction will have written by then: never a snapshot
-    internal_input = true;
-    struct Reset {
-      bool& flag;
-      ~Reset() {
-        flag = false;
-      }
-    } reset{internal_input};
-    return all_gather(&tensor, chunk, stream, std::move(keep));
-  }
-  // padded temporary (:1694-1720)
-  const int64_t padded = (n + size - 1) / size * size;
-  if (!scratch) {
-    throw std::runtime_error("moodist: allreduce of " + std::to_string(n) + " elements over " + std::to_string(size) +
-                             " ranks needs a scratch tensor of " + std::to_string(padded) + " elements");
-  }
-  check_device_tensor(*scratch, world->device, "allreduce scratch");
-  MD_CHECK(scratch->dtype == tensor.dtype && scratch->numel >= padded);
-  const size_t bytes = bytes_of(tensor);
-  refuse_capture(stream, "allreduce");
-  check_hip(hip().MemcpyAsync(scratch->data, tensor.data, bytes, kHipMemcpyDeviceToDevice, stream), "hipMemcpyAsync");
-  moodist_tensor whole = *scratch;
-  whole.numel = padded;
-  whole.ndim = 1;
-  whole.shape[0] = padded;
-  moodist_tensor chunk = whole;
-  chunk.numel = padded / size;
-  chunk.data = (char*)whole.data + (size_t)rank * (size_t)chunk.numel * (size_t)tensor.itemsize;
-  chunk.shape[0] = chunk.numel;
-  // `whole` already is a copy made at the call's position in the stream: no second snapshot
-  internal_input = true;
-  struct Reset {
-    bool& flag;
-    ~Reset() {
-      flag = false;
+    // in place (:1686-1693)
+    bytes = bytes_of(tensor) / (size_t)size;
+    p.input = tensor;
+    snapshot(p.input, stream, keep); // the reduction then reads the copy; the result still lands in the tensor
+    p.output = tensor;
+  } else {
+    const int64_t padded = (n + size - 1) / size * size;
+    if (!scratch) {
+      throw std::runtime_error("moodist: allreduce of " + std::to_string(n) + " elements over " + std::to_string(size) +
+                               " ranks needs a scratch tensor of " + std::to_string(padded) + " elements");
     }
-  } reset{internal_input};
-  reduce_scatter(&chunk, whole, reduce_op, stream, premul, keep);
-  // the copy back into `tensor` follows this rank's gather, wherever that gets launched
-  return all_gather_impl(&whole, chunk, stream, &tensor, std::move(keep));
+    check_device_tensor(*scratch, world->device, "allreduce scratch");
+    MD_CHECK(scratch->dtype == tensor.dtype && scratch->numel >= padded);
+    refuse_capture(stream, "allreduce");
+    check_hip(hip().MemcpyAsync(scratch->data, tensor.data, bytes_of(tensor), kHipMemcpyDeviceToDevice, stream),
+        "hipMemcpyAsync");
+    // the temporary already is a copy made at the call's position in the stream: no snapshot
+    moodist_tensor whole = *scratch;
+    whole.numel = padded;
+    whole.ndim = 1;
+    whole.shape[0] = padded;
+    bytes = bytes_of(whole) / (size_t)size;
+    p.input = whole;
+    p.output = whole;
+    p.copy_back = tensor; // follows this rank's gather, wherever that gets launched
+    p.has_copy_back = true;
+  }
+  p.chunk_bytes = chunk_bytes_for(bytes);
+  p.keep = std::move(keep);
+  return last = world->post(Kind::allreduce, next_seq++, rank, std::move(p), reduce_op, premul, bytes, tensor.dtype, 0,
+             nullptr);
 }
 
 // allreduce_coalesced (wrapper/processgroup_wrapper.cc:182-191), for the tensors of the list that
 // need no padding: the reference runs one allreduce -- a reduce_scatter and an all_gather -- per
-// tensor; here one reduce_scatter of the whole list (its reductions share launches) is followed
-// by one gather of every tensor's chunks.
+// tensor; here the list is one collective (World::run_allreduce).
 std::shared_ptr<Collective> ProcessGroup::allreduce_many(const moodist_tensor* tensors, size_t n, int reduce_op,
     void* stream, float premul, Keep keep) {
+  Busy guard(*this);
+  refuse_capture_early(stream, "allreduce");
   if (n == 0 || n > 0xffffu) {
     throw std::runtime_error("moodist: a coalesced allreduce takes 1..65535 tensors, not " + std::to_string(n));
   }
-  std::vector<moodist_tensor> chunks(n);
   // the whole list is checked before anything is posted: a list that is refused leaves nothing
   // pending and the rank's sequence where it was
+  size_t total = 0;
   for (size_t t = 0; t < n; ++t) {
     check_device_tensor(tensors[t], world->device, "allreduce tensor");
     MD_CHECK(tensors[t].numel > 0 && tensors[t].numel % size == 0);
@@ -506,25 +504,21 @@ std::shared_ptr<Collective> ProcessGroup::allreduce_many(const moodist_tensor* t
     if (tensors[t].dtype != tensors[0].dtype) {
       throw std::runtime_error("moodist: the tensors of a coalesced allreduce must have one element type");
     }
+    total += bytes_of(tensors[t]) / (size_t)size;
   }
+  Posting p;
   for (size_t t = 0; t < n; ++t) {
-    moodist_tensor& chunk = chunks[t];
-    chunk = tensors[t];
-    chunk.numel = tensors[t].numel / size;
-    chunk.data = (char*)tensors[t].data + (size_t)rank * (size_t)chunk.numel * (size_t)tensors[t].itemsize;
-    chunk.ndim = 1;
-    chunk.shape[0] = chunk.numel;
+    moodist_tensor in = tensors[t];
+    snapshot(in, stream, keep);
+    p.inputs.push_back(in);
+    p.outputs.push_back(tensors[t]);
   }
-  reduce_scatter_many(chunks.data(), tensors, n, reduce_op, stream, premul, keep); // both halves hold the tensors
-  // the gather's inputs are what the reductions will have written by then: never snapshots
-  internal_input = true;
-  struct Reset {
-    bool& flag;
-    ~Reset() {
-      flag = false;
-    }
-  } reset{internal_input};
-  return all_gather_many(tensors, chunks.data(), n, stream, std::move(keep));
+  p.wants_output = true;
+  p.kernel_less = options.forceKernelLess || options.preferKernelLess;
+  p.keep = std::move(keep);
+  p.stream = stream;
+  return last = world->post(Kind::allreduce_many, next_seq++, rank, std::move(p), reduce_op, premul, total,
+             tensors[0].dtype, (uint32_t)n, nullptr);
 }
 
 std::shared_ptr<Collective> ProcessGroup::allreduce_static(const moodist_tensor& tensor, int reduce_op, void* stream,
@@ -916,7 +910,7 @@ std::vector<std::vector<int>> ranks_by_stream(const Collective& c) {
 } // namespace
 
 void World::launch(Collective& c, const std::shared_ptr<CompiledOp>& op) {
-  if (c.kind == Kind::all_gather_many || c.kind == Kind::reduce_scatter_many) {
+  if (c.kind == Kind::all_gather_many || c.kind == Kind::reduce_scatter_many || c.kind == Kind::allreduce_many) {
     // the ranks agreed on the number of tensors and their total size (post); now tensor by tensor
     const size_t n = c.post[0].inputs.size();
     for (int j = 0; j < size; ++j) {
@@ -949,15 +943,138 @@ void World::launch(Collective& c, const std::shared_ptr<CompiledOp>& op) {
     }
   }
   order_streams_before(c);
-  std::vector<const void*> srcs((size_t)size);
   log_debug("collective #%llu: launching %s for %d ranks, %zu bytes per rank, dtype %d", (unsigned long long)c.seq,
-      c.kind == Kind::reduce_scatter    ? "reduce_scatter"
-      : c.kind == Kind::all_gather      ? "all_gather"
-      : c.kind == Kind::all_gather_many ? "all_gather of a list"
+      c.kind == Kind::reduce_scatter        ? "reduce_scatter"
+      : c.kind == Kind::all_gather          ? "all_gather"
+      : c.kind == Kind::all_gather_many     ? "all_gather of a list"
       : c.kind == Kind::reduce_scatter_many ? "reduce_scatter of a list"
-                                        : "custom op",
+      : c.kind == Kind::allreduce           ? "allreduce"
+      : c.kind == Kind::allreduce_many      ? "allreduce of a list"
+                                            : "custom op",
       size, c.bytes, c.dtype);
+  if (c.kind == Kind::allreduce || c.kind == Kind::allreduce_many) {
+    run_allreduce(c);
+  } else {
+    run(c, op);
+  }
+  order_streams_after(c);
+  if (current != device && current >= 0) {
+    check_hip(h.SetDevice(current), "hipSetDevice");
+  }
+}
 
+namespace {
+
+// The q-th of `size` equal chunks of a contiguous tensor, as a 1-D tensor.
+moodist_tensor chunk_of(const moodist_tensor& t, int q, int size) {
+  moodist_tensor chunk = t;
+  chunk.numel = t.numel / size;
+  chunk.data = (char*)t.data + (size_t)q * (size_t)chunk.numel * (size_t)t.itemsize;
+  chunk.ndim = 1;
+  chunk.shape[0] = chunk.numel;
+  return chunk;
+}
+
+} // namespace
+
+// allreduce and allreduce of a list.  Every rank's tensors are addressable here, so when the
+// ranks share a stream ONE launch does it all: a job per chunk c (and tensor), sources = every
+// rank's chunk c, folded in the order of the rank that owns the chunk (first = c), the result
+// stored over every source (mdh_allreduce_many) -- every tensor is read once and written once,
+// where reduce_scatter + all_gather read them once, write a chunk, and read and write all other
+// chunks again.  Ranks on different streams, pieces (num_chunks / chunk_size / method), the
+// copy-engine gather or snapshots of the inputs take the composition: the reduce_scatter of every
+// rank, the streams ordered, the all_gather of every rank (core/processgroup.cc:1686-1693).
+void World::run_allreduce(Collective& c) {
+  const HipRuntime& h = hip();
+  const bool list = c.kind == Kind::allreduce_many;
+  const size_t n = list ? c.post[0].inputs.size() : 1;
+  bool one_launch = true;
+  for (const Posting& p : c.post) {
+    one_launch = one_launch && p.stream == c.post[0].stream && p.chunk_bytes == 0 && !p.kernel_less;
+    for (size_t t = 0; t < n; ++t) {
+      one_launch = one_launch && (list ? p.inputs[t].data == p.outputs[t].data : p.input.data == p.output.data);
+    }
+  }
+  if (one_launch) {
+    const size_t itemsize = dtype_size(c.dtype);
+    const float scale = c.reduce_op == MDH_OP_AVG ? 1.0f / (float)size : c.premul;
+    std::vector<const void*> tables(n * (size_t)size * (size_t)size);
+    std::vector<mdh_reduce_job> jobs(n * (size_t)size);
+    size_t k = 0;
+    for (size_t t = 0; t < n; ++t) {
+      const size_t bytes = list ? bytes_of(c.post[0].inputs[t]) / (size_t)size : c.bytes;
+      for (int q = 0; q < size; ++q, ++k) {
+        for (int j = 0; j < size; ++j) {
+          const moodist_tensor& in = list ? c.post[(size_t)j].inputs[t] : c.post[(size_t)j].input;
+          tables[k * (size_t)size + (size_t)j] = (const char*)in.data + bytes * (size_t)q;
+        }
+        jobs[k].srcs = tables.data() + k * (size_t)size;
+        jobs[k].nsrc = size;
+        jobs[k].first = q;
+        jobs[k].dst = nullptr;
+        jobs[k].numel = bytes / itemsize;
+      }
+    }
+    void* stream = c.post[0].stream;
+    check_mdh(h.allreduce_many(jobs.data(), (int)jobs.size(), c.dtype, c.reduce_op, scale, stream));
+    for (const Posting& p : c.post) {
+      if (p.has_copy_back) { // through a padded temporary (core/processgroup.cc:1716-1720)
+        check_hip(h.MemcpyAsync(p.copy_back.data, p.output.data, (size_t)p.copy_back.numel * (size_t)p.copy_back.itemsize,
+                      kHipMemcpyDeviceToDevice, stream),
+            "hipMemcpyAsync");
+      }
+    }
+    return;
+  }
+  // the two halves, as two collectives of their own kinds
+  Collective rs, ag;
+  rs.kind = list ? Kind::reduce_scatter_many : Kind::reduce_scatter;
+  ag.kind = list ? Kind::all_gather_many : Kind::all_gather;
+  rs.seq = ag.seq = c.seq;
+  rs.reduce_op = c.reduce_op;
+  rs.premul = c.premul;
+  rs.bytes = ag.bytes = c.bytes;
+  rs.dtype = ag.dtype = c.dtype;
+  rs.post.resize((size_t)size);
+  ag.post.resize((size_t)size);
+  for (int q = 0; q < size; ++q) {
+    const Posting& p = c.post[(size_t)q];
+    Posting& r = rs.post[(size_t)q];
+    Posting& g = ag.post[(size_t)q];
+    r.arrived = g.arrived = true;
+    r.wants_output = g.wants_output = true;
+    r.stream = g.stream = p.stream;
+    r.chunk_bytes = p.chunk_bytes;
+    g.kernel_less = p.kernel_less;
+    if (list) {
+      for (size_t t = 0; t < n; ++t) {
+        const moodist_tensor mine = chunk_of(p.outputs[t], q, size);
+        r.inputs.push_back(p.inputs[t]);
+        r.outputs.push_back(mine);
+        g.inputs.push_back(mine);
+        g.outputs.push_back(p.outputs[t]);
+      }
+    } else {
+      const moodist_tensor mine = chunk_of(p.output, q, size);
+      r.input = p.input;
+      r.output = mine;
+      g.input = mine;
+      g.output = p.output;
+      g.has_copy_back = p.has_copy_back;
+      g.copy_back = p.copy_back;
+    }
+  }
+  run(rs, nullptr);
+  // every rank's gather reads what the other ranks' reductions write
+  order_streams_after(rs);
+  order_streams_before(ag);
+  run(ag, nullptr);
+}
+
+void World::run(Collective& c, const std::shared_ptr<CompiledOp>& op) {
+  const HipRuntime& h = hip();
+  std::vector<const void*> srcs((size_t)size);
   if (c.kind == Kind::reduce_scatter) {
     // out_q = in_q[q] (+) in_{q+1}[q] (+) ... in rank order starting at q (core/group.cc:567-570;
     // core/reduce_scatter.cc:180-191), pitch = bytes (core/processgroup.cc:1322)
@@ -1146,10 +1263,24 @@ void World::launch(Collective& c, const std::shared_ptr<CompiledOp>& op) {
                 "hipMemcpyAsync");
             ++kernel_less_copies_1d;
           } else {
-            check_hip(h.Memcpy2DAsync(dst, c.bytes, srcs[run.first], run.src_pitch, c.bytes, run.count,
-                          kHipMemcpyDeviceToDevice, pq.stream),
-                "hipMemcpy2DAsync");
-            ++kernel_less_copies_2d;
+            const int rc = h.Memcpy2DAsync(dst, c.bytes, srcs[run.first], run.src_pitch, c.bytes, run.count,
+                kHipMemcpyDeviceToDevice, pq.stream);
+            if (rc == kHipErrorInvalidValue) {
+              // The runtime refuses some shapes when it checks its arguments, before anything is
+              // enqueued (seen with rows of a few bytes at an odd pitch): rank by rank then.
+              (void)h.GetLastError();
+              log_debug("hipMemcpy2DAsync refused width %zu, %zu rows, pitches %zu -> %zu: one copy per rank", c.bytes,
+                  run.count, run.src_pitch, c.bytes);
+              for (size_t k = 0; k < run.count; ++k) {
+                check_hip(h.MemcpyAsync((char*)dst + c.bytes * k, (const char*)srcs[run.first] + run.src_pitch * k, c.bytes,
+                              kHipMemcpyDeviceToDevice, pq.stream),
+                    "hipMemcpyAsync");
+                ++kernel_less_copies_1d;
+              }
+            } else {
+              check_hip(rc, "hipMemcpy2DAsync");
+              ++kernel_less_copies_2d;
+            }
           }
         }
       } else {
@@ -1230,10 +1361,6 @@ void World::launch(Collective& c, const std::shared_ptr<CompiledOp>& op) {
       }
       check_mdh(h.copy_plan_launch(pt.plan, pt.bases.data(), (int)pt.bases.size(), pq.stream));
     }
-  }
-  order_streams_after(c);
-  if (current != device && current >= 0) {
-    check_hip(h.SetDevice(current), "hipSetDevice");
   }
 }
 

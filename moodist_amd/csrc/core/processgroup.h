@@ -22,7 +22,15 @@ namespace moodist {
 
 class World;
 
-enum class Kind : int { all_gather = 0, reduce_scatter = 1, custom = 2, all_gather_many = 3, reduce_scatter_many = 4 };
+enum class Kind : int {
+  all_gather = 0,
+  reduce_scatter = 1,
+  custom = 2,
+  all_gather_many = 3,
+  reduce_scatter_many = 4,
+  allreduce = 5,      // input = output = the tensor (or its padded temporary); bytes = one chunk
+  allreduce_many = 6, // inputs = outputs = the tensors
+};
 
 // What one rank brought to a collective.
 struct Posting {
@@ -123,8 +131,8 @@ public:
       int reduce_op, void* stream, float premul, Keep keep = {});
   std::shared_ptr<Collective> allreduce(const moodist_tensor& tensor, const moodist_tensor* scratch, int reduce_op,
       void* stream, float premul, Keep keep = {});
-  // n in-place allreduces of one element type whose element counts the group size divides: ONE
-  // reduce_scatter of the list into the rank's own chunks, then ONE gather of all the chunks
+  // n in-place allreduces of one element type whose element counts the group size divides, as
+  // one collective
   std::shared_ptr<Collective> allreduce_many(const moodist_tensor* tensors, size_t n, int reduce_op, void* stream,
       float premul, Keep keep = {});
   // allreduce whose padded temporary is this rank's slice of the kernel library's fixed
@@ -194,6 +202,10 @@ public:
 
 private:
   void launch(Collective& c, const std::shared_ptr<CompiledOp>& op);
+  // the launches of one collective of any kind but the allreduces, streams already ordered
+  void run(Collective& c, const std::shared_ptr<CompiledOp>& op);
+  // an allreduce: one launch for all ranks when they share a stream, else its two halves
+  void run_allreduce(Collective& c);
   void order_streams_before(Collective& c);
   void order_streams_after(Collective& c);
 

@@ -175,15 +175,15 @@ int dispatch_single(int dtype, int fold_op, const ReduceArgs& a, hipStream_t s) 
 #undef MDH_DISPATCH
 }
 
-int dispatch_many(int dtype, int fold_op, const ManyJob* jobs, int njobs, int mode, float scale, hipStream_t s) {
+int dispatch_many(int dtype, int fold_op, const ManyJob* jobs, int njobs, int mode, float scale, bool spread, hipStream_t s) {
 #define MDH_DISPATCH(tname)                                             \
   switch (fold_op) {                                                    \
   case kSum:                                                            \
-    return reduce_many_launch_##tname##_sum(jobs, njobs, mode, scale, s); \
+    return reduce_many_launch_##tname##_sum(jobs, njobs, mode, scale, spread, s); \
   case kMin:                                                            \
-    return reduce_many_launch_##tname##_min(jobs, njobs, mode, scale, s); \
+    return reduce_many_launch_##tname##_min(jobs, njobs, mode, scale, spread, s); \
   default:                                                              \
-    return reduce_many_launch_##tname##_max(jobs, njobs, mode, scale, s); \
+    return reduce_many_launch_##tname##_max(jobs, njobs, mode, scale, spread, s); \
   }
   switch (dtype) {
   case MDH_DTYPE_FLOAT32:
@@ -207,6 +207,7 @@ int dispatch_many(int dtype, int fold_op, const ManyJob* jobs, int njobs, int mo
 // long).  Below, sharing still pays: eight jobs of 8 x 4 MiB take 49 us in one launch and 60 us
 // in eight, of 8 x 8 MiB 97.8 against 100.1 us; of 8 x 16 MiB 196.5 against 183.3 us.
 constexpr size_t kOwnLaunchBytes = (size_t)16 << 20;
+constexpr size_t kSpreadPieceBytes = (size_t)32 << 20;
 
 } // namespace
 } // namespace mdh
@@ -241,14 +242,19 @@ extern "C" int mdh_reduce(const void* const* srcs, int nsrc, int first, void* ds
   return dispatch_single(dtype, info.fold_op, a, (hipStream_t)stream);
 }
 
-extern "C" int mdh_reduce_many(const mdh_reduce_job* jobs, int njobs, int dtype, int op, float scale, void* stream) {
-  using namespace mdh;
+namespace mdh {
+namespace {
+
+// mdh_reduce_many and mdh_allreduce_many: the second stores every job's result over all of the
+// job's sources (`spread`) and ignores jobs[j].dst.
+int reduce_list(const char* who, const mdh_reduce_job* jobs, int njobs, int dtype, int op, float scale, bool spread,
+    void* stream) {
   if (njobs < 0 || njobs > 65535 || (njobs > 0 && !jobs)) {
-    set_error("mdh_reduce_many: bad job table (%d jobs)", njobs);
+    set_error("%s: bad job table (%d jobs)", who, njobs);
     return MDH_EINVAL;
   }
   OpInfo info;
-  if (const int rc = parse_dtype_and_op("mdh_reduce_many", dtype, op, &info)) {
+  if (const int rc = parse_dtype_and_op(who, dtype, op, &info)) {
     return rc;
   }
   // every job is checked before anything is enqueued
@@ -265,38 +271,94 @@ extern "C" int mdh_reduce_many(const mdh_reduce_job* jobs, int njobs, int dtype,
     char label[32];
     std::snprintf(label, sizeof(label), " (job %d)", j);
     pool_at[(size_t)j] = at;
-    if (const int rc = check_operands("mdh_reduce_many", label, jobs[j].srcs, jobs[j].nsrc, jobs[j].first, jobs[j].dst,
-            jobs[j].numel, info.itemsize, pool.data() + at)) {
+    const mdh_reduce_job& job = jobs[j];
+    // (spread: the first source of the fold stands in for the destination, which it is)
+    const void* dst = job.dst;
+    if (spread && job.srcs && job.nsrc >= 1 && job.nsrc <= MDH_MAX_SOURCES && job.first >= 0 && job.first < job.nsrc) {
+      dst = job.srcs[job.first];
+    }
+    if (const int rc = check_operands(who, label, job.srcs, job.nsrc, job.first, dst, job.numel, info.itemsize, pool.data() + at)) {
       return rc;
     }
-    at += (size_t)jobs[j].nsrc;
-    any = any || jobs[j].numel != 0;
+    if (spread && job.numel != 0) {
+      // every source is written: no two of them may share a byte
+      const uintptr_t bytes = (uintptr_t)job.numel * info.itemsize;
+      for (int x = 0; x < job.nsrc; ++x) {
+        for (int y = x + 1; y < job.nsrc; ++y) {
+          const uintptr_t a = (uintptr_t)job.srcs[x], b = (uintptr_t)job.srcs[y];
+          if (a < b + bytes && b < a + bytes) {
+            set_error("%s: sources %d and %d overlap%s", who, x, y, label);
+            return MDH_EINVAL;
+          }
+        }
+      }
+    }
+    at += (size_t)job.nsrc;
+    any = any || job.numel != 0;
   }
   if (!any) {
     return MDH_OK;
   }
-  if (const int rc = refuse_capture((hipStream_t)stream, "mdh_reduce_many")) {
+  if (const int rc = refuse_capture((hipStream_t)stream, who)) {
     return rc;
   }
+  // A spread job stays in the list whatever its size (the single reduction's kernel has one
+  // destination); a very long one is cut into pieces of kSpreadPieceBytes per source so that
+  // launches keep their usual length.
+  size_t piece_pointers = 0, piece_jobs = 0;
+  for (int j = 0; spread && j < njobs; ++j) {
+    const size_t bytes = jobs[j].numel * info.itemsize;
+    if (bytes > kSpreadPieceBytes) {
+      const size_t pieces = (bytes + kSpreadPieceBytes - 1) / kSpreadPieceBytes;
+      piece_jobs += pieces;
+      piece_pointers += pieces * (size_t)jobs[j].nsrc;
+    }
+  }
+  std::vector<const void*> piece_pool(piece_pointers);
+  size_t piece_at = 0;
   std::vector<ManyJob> shared;
-  shared.reserve((size_t)njobs);
+  shared.reserve((size_t)njobs + piece_jobs);
   for (int j = 0; j < njobs; ++j) {
     const mdh_reduce_job& job = jobs[j];
     if (job.numel == 0) {
       continue;
     }
     const void* const* ordered = pool.data() + pool_at[(size_t)j];
-    if (job.numel * info.itemsize >= kOwnLaunchBytes) {
+    if (spread && job.numel * info.itemsize > kSpreadPieceBytes) {
+      const size_t piece_elems = kSpreadPieceBytes / info.itemsize;
+      for (size_t from = 0; from < job.numel; from += piece_elems) {
+        const void** mine = piece_pool.data() + piece_at;
+        for (int q = 0; q < job.nsrc; ++q) {
+          mine[q] = (const char*)ordered[q] + from * info.itemsize;
+        }
+        piece_at += (size_t)job.nsrc;
+        const size_t n = job.numel - from < piece_elems ? job.numel - from : piece_elems;
+        shared.push_back(ManyJob{mine, job.nsrc, const_cast<void*>(mine[0]), (uint64_t)n});
+      }
+      continue;
+    }
+    if (!spread && job.numel * info.itemsize >= kOwnLaunchBytes) {
       const ReduceArgs a = single_launch_args(ordered, job.nsrc, job.dst, job.numel, info.itemsize, info.mode, scale);
       if (const int rc = dispatch_single(dtype, info.fold_op, a, (hipStream_t)stream)) {
         return rc;
       }
       continue;
     }
-    shared.push_back(ManyJob{ordered, job.nsrc, job.dst, (uint64_t)job.numel});
+    shared.push_back(ManyJob{ordered, job.nsrc, spread ? const_cast<void*>(ordered[0]) : job.dst, (uint64_t)job.numel});
   }
   if (shared.empty()) {
     return MDH_OK;
   }
-  return dispatch_many(dtype, info.fold_op, shared.data(), (int)shared.size(), info.mode, scale, (hipStream_t)stream);
+  return dispatch_many(dtype, info.fold_op, shared.data(), (int)shared.size(), info.mode, scale, spread, (hipStream_t)stream);
+}
+
+} // namespace
+} // namespace mdh
+
+extern "C" int mdh_reduce_many(const mdh_reduce_job* jobs, int njobs, int dtype, int op, float scale, void* stream) {
+  return mdh::reduce_list("mdh_reduce_many", jobs, njobs, dtype, op, scale, false, stream);
+}
+
+extern "C" int mdh_allreduce_many(const mdh_reduce_job* jobs, int njobs, int dtype, int op, float scale, void* stream) {
+  return mdh::reduce_list("mdh_allreduce_many", jobs, njobs, dtype, op, scale, true, stream);
 }

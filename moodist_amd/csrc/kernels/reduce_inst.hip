@@ -24,7 +24,7 @@ int MDH_CAT(reduce_launch_, MDH_TNAME, _, MDH_FNAME)(const ReduceArgs& a, hipStr
 }
 
 int MDH_CAT(reduce_many_launch_, MDH_TNAME, _, MDH_FNAME)(const ManyJob* jobs, int njobs, int mode, float scale,
-    hipStream_t stream) {
-  return launch_many<MDH_TNAME, MDH_FNAME>(jobs, njobs, mode, scale, stream);
+    bool spread, hipStream_t stream) {
+  return launch_many<MDH_TNAME, MDH_FNAME>(jobs, njobs, mode, scale, spread, stream);
 }
 } // namespace mdh

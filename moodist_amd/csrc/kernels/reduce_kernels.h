@@ -226,8 +226,8 @@ __device__ __forceinline__ void fold_chunk(float scale, const char* const (&src)
 // One element, folded in source order.  The loads of eight sources are issued together: one
 // after the other, every source would cost this lane a whole memory round trip.
 template<typename T, int F>
-__device__ __forceinline__ void reduce_one_elem_from(const void* const* src, int nsrc, void* dst, int mode, float scale,
-    int64_t i) {
+__device__ __forceinline__ typename Traits<T>::elem_t reduce_one_elem_value(const void* const* src, int nsrc, int mode,
+    float scale, int64_t i) {
   using Tr = Traits<T>;
   using elem_t = typename Tr::elem_t;
   using acc_t = typename Tr::acc_t;
@@ -251,7 +251,13 @@ __device__ __forceinline__ void reduce_one_elem_from(const void* const* src, int
       }
     }
   }
-  ((elem_t*)dst)[i] = Tr::template finish<F>(acc, mode, scale);
+  return Tr::template finish<F>(acc, mode, scale);
+}
+
+template<typename T, int F>
+__device__ __forceinline__ void reduce_one_elem_from(const void* const* src, int nsrc, void* dst, int mode, float scale,
+    int64_t i) {
+  ((typename Traits<T>::elem_t*)dst)[i] = reduce_one_elem_value<T, F>(src, nsrc, mode, scale, i);
 }
 
 template<typename T, int F>
@@ -291,10 +297,11 @@ __device__ __forceinline__ void fold_rest(float scale, int rest, const char* con
 // Where the source pointers come from is the caller's business: early(integral_constant<int, K>,
 // p) fills p with the pointers of sources K .. K+CH-1 for a K known at compile time (the first
 // two groups), later(first, p) does the same for any group.  Slots past the last source may hold
-// anything; they are never used.
-template<typename T, int F, int U, int CH, int MODE, typename Early, typename Later>
+// anything; they are never used.  more_stores(out, lane_byte) is called after the tile's stores with
+// the tile's result still in registers (for results that go to more than one place).
+template<typename T, int F, int U, int CH, int MODE, typename Early, typename Later, typename More>
 __device__ __forceinline__ void reduce_tile_from(Early early_pointers, Later pointers, const char* dst, int nsrc, int mode_arg,
-    float scale, uint64_t tile_byte, uint32_t tile_bytes) {
+    float scale, uint64_t tile_byte, uint32_t tile_bytes, More more_stores) {
   using Tr = Traits<T>;
   using elem_t = typename Tr::elem_t;
   using acc_t = typename Tr::acc_t;
@@ -356,6 +363,7 @@ __device__ __forceinline__ void reduce_tile_from(Early early_pointers, Later poi
   for (int u = 0; u < U; ++u) {
     tile_store(rd, lane_byte + (uint32_t)u * (kWave * 16), out[u]); // dropped by the hardware past the end
   }
+  more_stores(out, lane_byte);
 }
 
 // The tile of a single reduction: pointers from the launch's argument struct, the first
@@ -382,7 +390,8 @@ __device__ __forceinline__ void reduce_tile(const ReduceArgs& a, const char* con
       p[k] = j < kEarlySources ? early[j < kEarlySources ? j : 0] : (const char*)a.src[j < MDH_MAX_SOURCES ? j : MDH_MAX_SOURCES - 1];
     }
   };
-  reduce_tile_from<T, F, U, CH, MODE>(early_pointers, pointers, (const char*)a.dst, nsrc, mode_arg, scale, tile_byte, tile_bytes);
+  reduce_tile_from<T, F, U, CH, MODE>(early_pointers, pointers, (const char*)a.dst, nsrc, mode_arg, scale, tile_byte, tile_bytes,
+      [](const u32x4 (&)[U], uint32_t) {});
 }
 
 // A tile is kWave*U consecutive 16-byte vectors (U KiB); tiles are dealt to
@@ -628,6 +637,7 @@ struct ManyArgs {
   uint32_t edge_wgs;
   float scale;
   int mode;
+  uint32_t spread; // 1: a job's result is stored over every one of its sources (dst is its first)
 };
 static_assert(sizeof(ManyArgs) + 256 <= 4096, "kernel arguments are limited to 4 KiB");
 
@@ -638,8 +648,16 @@ __device__ __attribute__((noinline)) void reduce_many_edges(const ManyArgs* args
   const uint32_t idx = wg * kWave + lane_id;
   const uint32_t job = idx / kManyTailSlots, k = idx % kManyTailSlots;
   if (job < a.njobs && k < a.tail[job]) {
+    using elem_t = typename Traits<T>::elem_t;
     const int64_t i = (int64_t)a.nvec[job] * per_vec<T>() + k;
-    reduce_one_elem_from<T, F>(a.ptr + a.first_ptr[job], a.nsrc[job], a.dst[job], a.mode, a.scale, i);
+    const void* const* src = a.ptr + a.first_ptr[job];
+    const elem_t r = reduce_one_elem_value<T, F>(src, a.nsrc[job], a.mode, a.scale, i);
+    ((elem_t*)a.dst[job])[i] = r;
+    if (a.spread) {
+      for (uint32_t q = 1; q < a.nsrc[job]; ++q) {
+        ((elem_t*)const_cast<void*>(src[q]))[i] = r;
+      }
+    }
   }
 }
 
@@ -673,8 +691,24 @@ __global__ __launch_bounds__(kWave) void reduce_many_kernel(ManyArgs a) {
       }
     };
     auto early_pointers = [&](auto first, const char* (&p)[CH]) { pointers(decltype(first)::value, p); };
-    reduce_tile_from<T, F, U, CH, PREMUL ? kPremul : kPlain>(early_pointers, pointers, (const char*)a.dst[job], (int)a.nsrc[job],
-        a.mode, a.scale, tile_byte, n);
+    // spread: the result goes over every source.  A tile is read from all of them before its
+    // first store (the result depends on every load), and no other wave touches its bytes.
+    const uint32_t nsrc = a.nsrc[job];
+    const bool spread = a.spread != 0;
+    auto more_stores = [&](const u32x4 (&out)[U], uint32_t lane_byte) {
+      if (spread) {
+        for (uint32_t q = 1; q < nsrc; ++q) {
+          const uint32_t j = base + q;
+          const __amdgpu_buffer_rsrc_t rd = tile_rsrc((const char*)a.ptr[j < (uint32_t)kManyPointers ? j : (uint32_t)kManyPointers - 1] + tile_byte, n);
+#pragma unroll
+          for (int u = 0; u < U; ++u) {
+            tile_store(rd, lane_byte + (uint32_t)u * (kWave * 16), out[u]);
+          }
+        }
+      }
+    };
+    reduce_tile_from<T, F, U, CH, PREMUL ? kPremul : kPlain>(early_pointers, pointers, (const char*)a.dst[job], (int)nsrc,
+        a.mode, a.scale, tile_byte, n, more_stores);
     tile += a.tile_waves;
   } while (tile < a.total_tiles);
 }
@@ -710,7 +744,7 @@ int launch_many_one(const ManyArgs& a, int unroll, hipStream_t stream) {
 // pointers each) and enqueues them.  The tile is the longest of 16, 8, 4, 2, 1 KiB that leaves
 // the launch about a thousand tiles (a wave per SIMD), as for a single reduction.
 template<typename T, int F, bool PREMUL>
-int launch_many_typed(const ManyJob* jobs, int njobs, int mode, float scale, hipStream_t stream) {
+int launch_many_typed(const ManyJob* jobs, int njobs, int mode, float scale, bool spread, hipStream_t stream) {
   using elem_t = typename Traits<T>::elem_t;
   constexpr uint64_t kPerVec = 16 / sizeof(elem_t);
   int at = 0;
@@ -768,6 +802,7 @@ int launch_many_typed(const ManyJob* jobs, int njobs, int mode, float scale, hip
     a.edge_wgs = (a.njobs * kManyTailSlots + kWave - 1) / kWave;
     a.scale = scale;
     a.mode = mode;
+    a.spread = spread ? 1u : 0u;
     const int rc = launch_many_one<T, F, PREMUL>(a, u, stream);
     if (rc != MDH_OK) {
       return rc;
@@ -778,20 +813,20 @@ int launch_many_typed(const ManyJob* jobs, int njobs, int mode, float scale, hip
 }
 
 template<typename T, int F>
-int launch_many(const ManyJob* jobs, int njobs, int mode, float scale, hipStream_t stream) {
+int launch_many(const ManyJob* jobs, int njobs, int mode, float scale, bool spread, hipStream_t stream) {
   if constexpr (F == kSum && (std::is_floating_point_v<T> || sizeof(typename Traits<T>::elem_t) == 2)) {
     if (mode == kPremul) {
-      return launch_many_typed<T, F, true>(jobs, njobs, mode, scale, stream);
+      return launch_many_typed<T, F, true>(jobs, njobs, mode, scale, spread, stream);
     }
   }
-  return launch_many_typed<T, F, false>(jobs, njobs, mode, scale, stream);
+  return launch_many_typed<T, F, false>(jobs, njobs, mode, scale, spread, stream);
 }
 
 // One entry per (element type, fold), each instantiated in its own object
 // file (reduce_inst.hip compiled once per pair) so they build in parallel.
 #define MDH_REDUCE_ENTRY(tname, fname)                                                  \
   int reduce_launch_##tname##_##fname(const ReduceArgs& a, hipStream_t stream);         \
-  int reduce_many_launch_##tname##_##fname(const ManyJob* jobs, int njobs, int mode, float scale, hipStream_t stream)
+  int reduce_many_launch_##tname##_##fname(const ManyJob* jobs, int njobs, int mode, float scale, bool spread, hipStream_t stream)
 #define MDH_REDUCE_ENTRIES(tname) \
   MDH_REDUCE_ENTRY(tname, sum);   \
   MDH_REDUCE_ENTRY(tname, min);   \

@@ -71,6 +71,10 @@ def test_box_struct_layout_matches_header():
     (lambda: abi.reduce_many([([16], 0, 32, 4)], abi.DTYPE_INT32, abi.OP_AVG), "Unsupported reduce operation"),
     (lambda: abi.reduce_many([([16] * 65, 0, 32, 4)], abi.DTYPE_FLOAT32, abi.OP_SUM), "nsrc 65 outside"),
     (lambda: abi.reduce_many([([64], 0, 68, 4)], abi.DTYPE_FLOAT32, abi.OP_SUM), "partially overlaps"),
+    (lambda: abi.allreduce_many([([16, 48], 2, 0, 4)], abi.DTYPE_FLOAT32, abi.OP_SUM), r"first 2 outside 0..1 \(job 0\)"),
+    (lambda: abi.allreduce_many([([64, 72], 0, 0, 4)], abi.DTYPE_FLOAT32, abi.OP_SUM), r"overlaps source 1 \(job 0\)"),
+    (lambda: abi.allreduce_many([([64, 128, 64], 0, 0, 4)], abi.DTYPE_FLOAT32, abi.OP_SUM), r"sources 0 and 2 overlap"),
+    (lambda: abi.allreduce_many([([64, 128], 0, 0, 4)], abi.DTYPE_INT64, abi.OP_PREMUL_SUM), "Unsupported reduce operation"),
     (lambda: abi.set_tuning("reduce_wg_per_cu", 10), "does not take 10"),
     (lambda: abi.set_tuning("no_such_knob", 1), "unknown knob"),
     (lambda: abi.set_tuning("reduce_unroll", 3), "does not take 3"),

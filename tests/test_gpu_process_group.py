@@ -732,3 +732,106 @@ print("ok")
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300, cwd=root)
     assert r.returncode == 0 and "ok" in r.stdout, (r.stdout[-1000:], r.stderr[-3000:])
+
+
+# ---------------------------------------------------------------- allreduce: one launch, or its two halves
+
+
+def allreduce_want(srcs, n, dtype, op, scale):
+    """What allreduce leaves in every rank's tensor: chunk c is the fold that starts at rank c
+    (core/processgroup.cc:1674-1722 with core/group.cc:567-570), over zero padding if needed."""
+    padded = (n + P - 1) // P * P
+    chunk = padded // P
+    full = [torch.cat([s, torch.zeros(padded - n, dtype=dtype)]) for s in srcs]
+    return np.concatenate([oracle.reduce([bits(f[c * chunk:(c + 1) * chunk]) for f in full], c, TORCH_TO_CODE[dtype], op,
+                                         scale) for c in range(P)])[:n]
+
+
+ALLREDUCE_ROUTES = ["one_launch", "own_streams", "two_streams", "num_chunks", "kernel_less", "snapshot"]
+
+
+@pytest.mark.parametrize("route", ALLREDUCE_ROUTES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.int64], ids=str)
+def test_allreduce_routes_agree_with_the_oracle_bit_for_bit(world, dev, dtype, route):
+    """Ranks that share a stream get ONE launch that reduces every chunk and stores it into every
+    rank's tensor; ranks on different streams, pieces, the copy-engine gather and input snapshots
+    get reduce_scatter + all_gather.  Every route must leave the same bits: the oracle's."""
+    streams = {"own_streams": [torch.cuda.Stream(device=dev) for _ in range(P)],
+               "two_streams": [torch.cuda.Stream(device=dev) for _ in range(2)] * (P // 2)}.get(route)
+    for pg in world:
+        if route == "num_chunks":
+            pg.options().num_chunks = 3
+        elif route == "kernel_less":
+            pg.options().force_kernel_less = True
+        elif route == "snapshot":
+            pg.options().snapshot_inputs = True
+    try:
+        for n in (8, 8 * 1000, 8 * 1000 + 3, 5, 8 * 40001, 300007):
+            for name, code in (("SUM", oracle.OP_SUM), ("MAX", oracle.OP_MAX), ("AVG", oracle.OP_AVG)):
+                if code == oracle.OP_AVG and not dtype.is_floating_point:
+                    continue
+                srcs = random_sources(P, n, dtype, seed=n + code)
+                want = allreduce_want(srcs, n, dtype, code, 1.0 / P if code == oracle.OP_AVG else 1.0)
+                o = dist.AllreduceOptions()
+                o.reduceOp = getattr(dist.ReduceOp, name)
+                ts = [None] * P
+                works = []
+                torch.cuda.synchronize()
+                for r, pg in enumerate(world):
+                    if streams:
+                        with torch.cuda.stream(streams[r]):
+                            ts[r] = srcs[r].to(dev)  # produced on the rank's own stream
+                            works.append(pg.allreduce([ts[r]], o))
+                    else:
+                        ts[r] = srcs[r].to(dev)
+                        works.append(pg.allreduce([ts[r]], o))
+                for w in works:
+                    w.wait()
+                torch.cuda.synchronize()
+                for r in range(P):
+                    assert same_bits(bits(ts[r]), want), (route, dtype, n, name, r)
+    finally:
+        for pg in world:
+            pg.options().num_chunks = -1
+            pg.options().force_kernel_less = False
+            pg.options().snapshot_inputs = False
+
+
+@pytest.mark.parametrize("own_streams", [False, True])
+def test_allreduce_coalesced_routes_agree_with_the_oracle(world, dev, own_streams):
+    # a list of divisible tensors (one collective) with two that need padding (an allreduce each)
+    sizes = [8, 8 * 7, 8 * 1000, 8 * 12345, 13, 8 * 3, 1001]
+    streams = [torch.cuda.Stream(device=dev) for _ in range(P)] if own_streams else None
+    srcs = [random_sources(P, n, torch.float32, seed=3 * n) for n in sizes]  # [tensor][rank]
+    wants = [allreduce_want(srcs[k], n, torch.float32, oracle.OP_SUM, 1.0) for k, n in enumerate(sizes)]
+    ts = [None] * P
+    works = []
+    torch.cuda.synchronize()
+    for r, pg in enumerate(world):
+        if streams:
+            with torch.cuda.stream(streams[r]):
+                ts[r] = [srcs[k][r].to(dev) for k in range(len(sizes))]
+                works.append(pg.allreduce_coalesced(ts[r]))
+        else:
+            ts[r] = [srcs[k][r].to(dev) for k in range(len(sizes))]
+            works.append(pg.allreduce_coalesced(ts[r]))
+    for w in works:
+        w.wait()
+    torch.cuda.synchronize()
+    for r in range(P):
+        for k in range(len(sizes)):
+            assert same_bits(bits(ts[r][k]), wants[k]), (own_streams, r, k)
+
+
+def test_allreduce_of_a_large_tensor_in_one_launch(world, dev):
+    # 8 ranks x 72 MiB: chunks of 9 MiB, jobs that fill more than one launch of the list kernel
+    n = 8 * (9 << 18) + 8
+    g = torch.Generator().manual_seed(77)
+    host = [torch.randint(-1000, 1000, (n,), dtype=torch.int32, generator=g) for _ in range(P)]
+    ts = [h.to(dev) for h in host]
+    each_rank(world, lambda r, pg: pg.allreduce([ts[r]]))
+    want = host[0].clone()
+    for h in host[1:]:
+        want += h
+    for t in ts:
+        assert torch.equal(t.cpu(), want)

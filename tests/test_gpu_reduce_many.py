@@ -115,3 +115,79 @@ def test_in_place_jobs_and_equality_with_single_launches(dev):
         torch.cuda.synchronize()
         for k, srcs in enumerate(sets):
             assert same_bits(bits(srcs[k % P]), bits(singles[k])), (dtype, k)
+
+
+# ---------------------------------------------------------------- results stored over every source
+
+
+def run_spread_jobs(dev, dtype, op, specs, scale, offsets=None):
+    """mdh_allreduce_many: specs as for run_jobs.  Afterwards EVERY source of a job must hold the
+    oracle's result of that job in its first n elements, and nothing else may have changed."""
+    st = torch.cuda.current_stream().cuda_stream
+    jobs, results = [], []
+    for k, (P, n, first) in enumerate(specs):
+        off = 0 if offsets is None else offsets[k]
+        srcs = random_sources(P, n, dtype, seed=2000 * k + 17 * P + n)
+        dev_full = [torch.full((n + off + 64,), 55, dtype=dtype, device=dev) for _ in range(P)]
+        for f, s in zip(dev_full, srcs):
+            f[off:off + n].copy_(s)
+        isz = dev_full[0].element_size()
+        jobs.append(([f.data_ptr() + off * isz for f in dev_full], first, 0, n))
+        want = oracle.reduce([bits(s) for s in srcs], first, TORCH_TO_CODE[dtype], op, scale) if n else None
+        results.append((dev_full, off, n, want, (P, n, first)))
+    abi.allreduce_many(jobs, TORCH_TO_CODE[dtype], op, scale, st)
+    torch.cuda.synchronize()
+    guard = torch.full((1,), 55, dtype=dtype)
+    for dev_full, off, n, want, spec in results:
+        for r, f in enumerate(dev_full):
+            if n:
+                assert same_bits(bits(f[off:off + n]), want), (dtype, op, spec, r)
+            assert torch.equal(f[:off].cpu(), guard.expand(off)), (spec, r)
+            assert torch.equal(f[off + n:].cpu(), guard.expand(64)), (spec, r)
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES, ids=str)
+def test_spread_ragged_sizes_mixed_source_counts_all_ops(dev, dtype):
+    specs = [(8, 1, 3), (3, 7, 0), (8, 64, 7), (1, 255, 0), (16, 1031, 5), (8, 4096 + 5, 2), (64, 70001, 63), (2, 0, 1),
+             (7, 65536, 6), (33, 12345, 17), (8, 300000 + 3, 1), (9, 2, 8), (64, 513, 0), (64, 31, 40), (64, 8, 1),
+             (17, 100000, 16)]
+    for op in (oracle.OP_SUM, oracle.OP_MIN, oracle.OP_MAX, oracle.OP_AVG, oracle.OP_PREMUL_SUM):
+        if op in (oracle.OP_AVG, oracle.OP_PREMUL_SUM) and not dtype.is_floating_point:
+            continue
+        run_spread_jobs(dev, dtype, op, specs, scale_for(op, 8))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.int64], ids=str)
+def test_spread_operands_off_the_vector_grid(dev, dtype):
+    # every operand of a job starts `off` elements into its allocation: vectors off the 16-byte grid
+    specs = [(8, 5000 + k, k % 8) for k in range(9)]
+    run_spread_jobs(dev, dtype, oracle.OP_SUM, specs, 1.0, offsets=[0, 1, 2, 3, 5, 7, 9, 11, 13])
+
+
+def test_spread_is_the_allreduce_of_local_ranks(dev):
+    # eight ranks' tensors of 8 x 3001 fp32, one job per chunk c with first = c: every tensor ends up
+    # holding what reduce_scatter (chunk c folded in rank c's order) and all_gather would leave
+    P, n = 8, 3001
+    tensors = random_sources(P, P * n, torch.float32, seed=5)
+    d = [t.to(dev) for t in tensors]
+    jobs = [([x.data_ptr() + c * n * 4 for x in d], c, 0, n) for c in range(P)]
+    abi.allreduce_many(jobs, abi.DTYPE_FLOAT32, abi.OP_SUM, 1.0, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    want = np.concatenate([oracle.reduce([bits(t[c * n:(c + 1) * n]) for t in tensors], c, abi.DTYPE_FLOAT32, oracle.OP_SUM, 1.0)
+                           for c in range(P)])
+    for x in d:
+        assert same_bits(bits(x), want)
+
+
+def test_spread_long_jobs_are_cut_into_pieces(dev):
+    # 40 MiB per source (more than one 32 MiB piece), three sources, element-wise known answer
+    n = (40 << 20) // 4 + 3
+    g = torch.Generator().manual_seed(9)
+    srcs = [torch.randint(-1000, 1000, (n,), dtype=torch.int32, generator=g) for _ in range(3)]
+    d = [s.to(dev) for s in srcs]
+    abi.allreduce_many([([x.data_ptr() for x in d], 1, 0, n)], abi.DTYPE_INT32, abi.OP_SUM, 1.0,
+                       torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    want = srcs[0] + srcs[1] + srcs[2]
+    for x in d:
+        assert torch.equal(x.cpu(), want)
