@@ -18,7 +18,7 @@ not in the 256 MB Infinity Cache either.  Prints one JSON line.
     gather:<sources>:<bytes per shard>
     rows:<boxes>:<rows per box>:<run bytes>:<source pitch bytes>    strided rows into a dense destination
     transpose:<rows>:<cols>:<itemsize>                              2-D element transpose
-    coalesced:<tensors>:<elements>[:loop]                           allreduce_coalesced of eight local ranks
+    coalesced:<tensors>:<elements>[:loop|:halves]                   allreduce_coalesced of eight local ranks
     reduce_many:<jobs>:<sources>:<elements>[:single]                a list of reductions in shared launches
 """
 
@@ -323,7 +323,7 @@ def build_workload(name, torch, abi, dev, rotation_bytes):
         return desc, set_bytes, launch, check, "reduce_vec_kernel" if single else "reduce_many_kernel"
 
     if name.startswith("coalesced:"):
-        # coalesced:<tensors>:<elements>[:loop] -- allreduce_coalesced (MAX, fp32, in place) of a list of
+        # coalesced:<tensors>:<elements>[:loop|:halves] -- allreduce_coalesced (MAX, fp32, in place) of a list of
         # tensors of about that many elements each, called by all eight ranks of a local group: what
         # a DDP or ZeRO bucket of many small tensors costs, host and GPU together.  With ":loop", one
         # allreduce per tensor instead, as the reference serves the call
@@ -335,6 +335,7 @@ def build_workload(name, torch, abi, dev, rotation_bytes):
         parts = name.split(":")
         T, n = int(parts[1]), int(parts[2])
         loop = len(parts) > 3 and parts[3] == "loop"
+        halves = len(parts) > 3 and parts[3] == "halves"
         P = 8
         world = moodist_amd.LocalWorld(P, dev)
         sizes = [n + 8 * k for k in range(T)]  # multiples of the group size when n is
@@ -345,10 +346,22 @@ def build_workload(name, torch, abi, dev, rotation_bytes):
         opts.reduceOp = dist.ReduceOp.MAX  # idempotent: the launches can repeat on the same tensors
         one = dist.AllreduceOptions()
         one.reduceOp = dist.ReduceOp.MAX
-        set_bytes = sum(P * ((P + 1) * m // P + 2 * m * (P - 1) // P) * 4 for m in sizes)
+        # every rank's tensor read once and written once (what reduce_scatter + all_gather move is
+        # (3P - 1) / 2P of that again)
+        set_bytes = sum(2 * P * m * 4 for m in sizes)
+        # ":halves": the two coalesced collectives an allreduce_coalesced is composed of, called
+        # one after the other on chunk views
+        chunks = [[t[r * (t.numel() // P):(r + 1) * (t.numel() // P)] for t in tensors[r]] for r in range(P)]
+        rs_opts = dist.ReduceScatterOptions()
+        rs_opts.reduceOp = dist.ReduceOp.MAX
 
         def launch(i):
-            if loop:
+            if halves:
+                for r in range(P):
+                    world.groups[r].reduce_scatter_tensor_coalesced(chunks[r], tensors[r], rs_opts)
+                for r in range(P):
+                    world.groups[r].allgather_into_tensor_coalesced(tensors[r], chunks[r])
+            elif loop:
                 for k in range(T):
                     for r in range(P):
                         world.groups[r].allreduce([tensors[r][k]], one)
@@ -365,10 +378,10 @@ def build_workload(name, torch, abi, dev, rotation_bytes):
                     if not torch.equal(tensors[r][k].cpu(), want):
                         raise SystemExit("bench: result differs from the expected allreduce")
 
-        desc = {"workload": name, "op": "allreduce_coalesced MAX, eight local ranks" + (", one allreduce per tensor" if loop else ""),
+        desc = {"workload": name, "op": "allreduce_coalesced MAX, eight local ranks" + (", one allreduce per tensor" if loop else ", as reduce_scatter_tensor_coalesced + allgather_into_tensor_coalesced" if halves else ""),
                 "tensors": T, "numel": n, "dtype": "float32", "buffer_sets": 1,
                 "note": "a step is all eight ranks' calls; ms_per_step is host and GPU together"}
-        return desc, set_bytes, launch, check, "reduce_many_kernel + copy_flat_kernel"
+        return desc, set_bytes, launch, check, "reduce_many_kernel + copy_flat_kernel" if halves else "reduce_many_kernel"
 
     if name.startswith("rows:"):
         # rows:<boxes>:<rows per box>:<run bytes>:<source pitch bytes> -- every box is `rows` runs of

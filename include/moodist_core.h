@@ -30,6 +30,12 @@
  *
  * Nothing here synchronises the host with the device.
  *
+ * Every rank numbers its collectives; call k of one rank meets call k of the others, and calls
+ * that differ (operation, size, element type, reduction) are an error for the rank that arrives
+ * with the difference -- the reference aborts there (core/cputhread.h:100-112).  A call that
+ * is refused, for this or for its arguments, has posted nothing and leaves the rank's numbering
+ * where it was.
+ *
  * A stream that is being captured into a graph (hipStreamBeginCapture) is refused by every
  * collective, with an error and nothing recorded: replaying a graph that holds this library's
  * launches is not supported.
@@ -126,16 +132,22 @@ int moodist_pg_reduce_scatter_many(moodist_pg* pg, const moodist_tensor* outputs
  * reduce-scatter into the rank's own chunk followed by an all-gather, in place.  When numel
  * is not a multiple of the group size the reference allocates a padded temporary through
  * torch (:1694-1697); here the caller passes it as `scratch` (>= roundup(numel, size)
- * elements, same dtype), or NULL when numel divides evenly. */
+ * elements, same dtype), or NULL when numel divides evenly.
+ * The call is ONE collective (one sequence number; every rank must call allreduce).  Ranks that
+ * passed the same stream get one kernel launch for all of them, which reduces every chunk in
+ * its owner's fold order and stores it into every rank's tensor (mdh_allreduce_many); ranks on
+ * different streams, the chunk options, the copy-engine gather and snapshot_inputs get the
+ * reduce_scatter and the all_gather, rank by rank.  The results are the same bit for bit. */
 int moodist_pg_allreduce(moodist_pg* pg, const moodist_tensor* tensor, const moodist_tensor* scratch, int reduce_op,
     void* stream, float premul_value, moodist_work** work);
 /* c10d's allreduce_coalesced (wrapper/processgroup_wrapper.cc:182-191), which the reference serves
  * with one allreduce per tensor, for tensors of one element type whose element counts the group
- * size divides (the others go through moodist_pg_allreduce one by one): ONE reduce_scatter of
- * the list into the rank's own chunks, in place (moodist_pg_reduce_scatter_many), then ONE
- * all_gather of every tensor's chunks (moodist_pg_all_gather_many).  `*work` is the gather; the
- * reduce_scatter has been launched when it has.  A list that is refused (mixed element types,
- * an operation the type does not support) leaves nothing posted. */
+ * size divides (the others go through moodist_pg_allreduce one by one): ONE collective, served
+ * like moodist_pg_allreduce -- by shared launches that reduce every chunk of every tensor and
+ * store it into every rank's tensor when the ranks passed the same stream, else by the
+ * reduce_scatter of the list into the rank's own chunks and the all_gather of every tensor's
+ * chunks.  A list that is refused (mixed element types, an operation the type does not support)
+ * leaves nothing posted. */
 int moodist_pg_allreduce_many(moodist_pg* pg, const moodist_tensor* tensors, size_t n, int reduce_op, void* stream,
     float premul_value, moodist_work** work);
 /* No counterpart in the reference.  moodist_pg_allreduce for callers that cannot allocate

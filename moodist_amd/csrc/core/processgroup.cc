@@ -236,6 +236,25 @@ void ProcessGroup::snapshot(moodist_tensor& input, void* stream, Keep& keep) {
   input.data = copy;
 }
 
+// Posts `p` as this rank's next collective.  The rank's sequence advances when the world has
+// taken the posting -- also when the launches this arrival triggered then failed, since every
+// rank has spent that number --, and stays where it was when the posting is refused (the ranks
+// disagree about the collective).
+std::shared_ptr<Collective> ProcessGroup::post_next(Kind kind, Posting p, int reduce_op, float premul, size_t bytes,
+    int dtype, uint32_t op_id, const std::shared_ptr<CompiledOp>& op) {
+  bool taken = false;
+  struct Advance {
+    uint64_t& seq;
+    const bool& taken;
+    ~Advance() {
+      if (taken) {
+        ++seq;
+      }
+    }
+  } advance{next_seq, taken};
+  return last = world->post(kind, next_seq, rank, std::move(p), reduce_op, premul, bytes, dtype, op_id, op, &taken);
+}
+
 std::shared_ptr<Collective> ProcessGroup::all_gather(const moodist_tensor* output, const moodist_tensor& input,
     void* stream, Keep keep) {
   return all_gather_impl(output, input, stream, nullptr, std::move(keep));
@@ -264,7 +283,7 @@ std::shared_ptr<Collective> ProcessGroup::all_gather_impl(const moodist_tensor* 
     }
   }
   p.kernel_less = options.forceKernelLess || options.preferKernelLess;
-  return last = world->post(Kind::all_gather, next_seq++, rank, std::move(p), 0, 1.0f, bytes, input.dtype, 0, nullptr);
+  return post_next(Kind::all_gather, std::move(p), 0, 1.0f, bytes, input.dtype, 0, nullptr);
 }
 
 // The list form of all_gather (wrapper/processgroup_wrapper.cc:112-129).  The reference gathers
@@ -294,7 +313,7 @@ std::shared_ptr<Collective> ProcessGroup::all_gather_list(const moodist_tensor* 
     p.outputs.push_back(outputs[i]);
   }
   p.kernel_less = options.forceKernelLess || options.preferKernelLess;
-  return last = world->post(Kind::all_gather, next_seq++, rank, std::move(p), 0, 1.0f, bytes, input.dtype, 0, nullptr);
+  return post_next(Kind::all_gather, std::move(p), 0, 1.0f, bytes, input.dtype, 0, nullptr);
 }
 
 // allgather_into_tensor_coalesced (wrapper/processgroup_wrapper.cc:139-148).  The reference loops
@@ -328,7 +347,7 @@ std::shared_ptr<Collective> ProcessGroup::all_gather_many(const moodist_tensor* 
   p.keep = std::move(keep);
   p.stream = stream;
   p.kernel_less = options.forceKernelLess || options.preferKernelLess;
-  return last = world->post(Kind::all_gather_many, next_seq++, rank, std::move(p), 0, 1.0f, total, inputs[0].dtype,
+  return post_next(Kind::all_gather_many, std::move(p), 0, 1.0f, total, inputs[0].dtype,
              (uint32_t)n, nullptr);
 }
 
@@ -355,7 +374,7 @@ std::shared_ptr<Collective> ProcessGroup::reduce_scatter(const moodist_tensor* o
   p.keep = std::move(keep);
   p.stream = stream;
   p.chunk_bytes = chunk_bytes_for(bytes);
-  return last = world->post(Kind::reduce_scatter, next_seq++, rank, std::move(p), reduce_op, premul, bytes,
+  return post_next(Kind::reduce_scatter, std::move(p), reduce_op, premul, bytes,
              input.dtype, 0, nullptr);
 }
 
@@ -427,7 +446,7 @@ std::shared_ptr<Collective> ProcessGroup::reduce_scatter_many(const moodist_tens
   p.wants_output = outputs != nullptr;
   p.keep = std::move(keep);
   p.stream = stream;
-  return last = world->post(Kind::reduce_scatter_many, next_seq++, rank, std::move(p), reduce_op, premul, total,
+  return post_next(Kind::reduce_scatter_many, std::move(p), reduce_op, premul, total,
              inputs[0].dtype, (uint32_t)n, nullptr);
 }
 
@@ -480,7 +499,7 @@ std::shared_ptr<Collective> ProcessGroup::allreduce(const moodist_tensor& tensor
   }
   p.chunk_bytes = chunk_bytes_for(bytes);
   p.keep = std::move(keep);
-  return last = world->post(Kind::allreduce, next_seq++, rank, std::move(p), reduce_op, premul, bytes, tensor.dtype, 0,
+  return post_next(Kind::allreduce, std::move(p), reduce_op, premul, bytes, tensor.dtype, 0,
              nullptr);
 }
 
@@ -517,7 +536,7 @@ std::shared_ptr<Collective> ProcessGroup::allreduce_many(const moodist_tensor* t
   p.kernel_less = options.forceKernelLess || options.preferKernelLess;
   p.keep = std::move(keep);
   p.stream = stream;
-  return last = world->post(Kind::allreduce_many, next_seq++, rank, std::move(p), reduce_op, premul, total,
+  return post_next(Kind::allreduce_many, std::move(p), reduce_op, premul, total,
              tensors[0].dtype, (uint32_t)n, nullptr);
 }
 
@@ -651,7 +670,7 @@ std::shared_ptr<Collective> ProcessGroup::custom_op(const std::shared_ptr<Compil
     check_device_tensor(outputs[i], world->device, "custom op output");
     p.outputs.push_back(outputs[i]);
   }
-  return last = world->post(Kind::custom, next_seq++, rank, std::move(p), 0, 1.0f, 0, op->dtype, op->id, op);
+  return post_next(Kind::custom, std::move(p), 0, 1.0f, 0, op->dtype, op->id, op);
 }
 
 // ---------------------------------------------------------------- kernel-less runs
@@ -766,7 +785,7 @@ World::~World() {
 }
 
 std::shared_ptr<Collective> World::post(Kind kind, uint64_t seq, int rank, Posting p, int reduce_op, float premul,
-    size_t bytes, int dtype, uint32_t op_id, const std::shared_ptr<CompiledOp>& op) {
+    size_t bytes, int dtype, uint32_t op_id, const std::shared_ptr<CompiledOp>& op, bool* taken) {
   std::lock_guard<std::mutex> l(mutex);
   std::shared_ptr<Collective>& slot = pending[seq];
   if (!slot) {
@@ -792,6 +811,9 @@ std::shared_ptr<Collective> World::post(Kind kind, uint64_t seq, int rank, Posti
   p.arrived = true;
   mine = std::move(p);
   ++c->arrived;
+  if (taken) {
+    *taken = true;
+  }
   if (c->arrived == size) {
     pending.erase(seq);
     // what the ranks asked to keep alive is let go once the launches are enqueued (or have

@@ -154,6 +154,8 @@ public:
   std::shared_ptr<Collective> last; // the collective this rank posted most recently
 
 private:
+  std::shared_ptr<Collective> post_next(Kind kind, Posting p, int reduce_op, float premul, size_t bytes, int dtype,
+      uint32_t op_id, const std::shared_ptr<CompiledOp>& op);
   std::shared_ptr<Collective> all_gather_impl(const moodist_tensor* output, const moodist_tensor& input, void* stream,
       const moodist_tensor* copy_back, Keep keep);
   // snapshot_inputs: replaces input.data by a copy made now on `stream`; the copy joins `keep`
@@ -187,8 +189,9 @@ public:
   // Posts `p` for (kind, seq); launches when the last rank arrives.  Throws if the ranks
   // disagree about what collective number `seq` is (the reference aborts on this,
   // core/cputhread.h:100-112).
+  // `taken`, if given, is set once the posting has been accepted (before any launch).
   std::shared_ptr<Collective> post(Kind kind, uint64_t seq, int rank, Posting p, int reduce_op, float premul,
-      size_t bytes, int dtype, uint32_t op_id, const std::shared_ptr<CompiledOp>& op);
+      size_t bytes, int dtype, uint32_t op_id, const std::shared_ptr<CompiledOp>& op, bool* taken = nullptr);
 
   // Adds `held` to what rank `rank` keeps alive for collective `c`; if the collective has
   // launched already, `held` is simply dropped.

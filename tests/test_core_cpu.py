@@ -306,6 +306,33 @@ def test_mismatched_collectives_are_detected(core):
     core.moodist_world_destroy(w)
 
 
+def test_allreduce_is_one_collective(core):
+    # an allreduce takes ONE collective number: after it, the rank's next call is its number 1,
+    # and a rank that spells the two halves out does not pair with ranks that call allreduce
+    w = make_world(core, 2)
+    a, b = core.moodist_world_group(w, 0), core.moodist_world_group(w, 1)
+    work = ctypes.c_void_p()
+    t = fake(8)
+    assert core.moodist_pg_allreduce(a, ctypes.byref(t), None, 0, None, 0.0, ctypes.byref(work)) == 0, core.moodist_last_error()
+    assert core.moodist_work_is_completed(work) == 0  # rank 1 has not called
+    core.moodist_work_destroy(work)
+    # rank 0's number 1 is an all_gather; rank 1's number 0 must be the allreduce, not a reduce_scatter
+    assert core.moodist_pg_all_gather(a, ctypes.byref(fake(8)), ctypes.byref(fake(4)), None, ctypes.byref(work)) == 0
+    core.moodist_work_destroy(work)
+    assert core.moodist_pg_reduce_scatter(b, ctypes.byref(fake(4)), ctypes.byref(fake(8)), 0, None, 0.0,
+                                          ctypes.byref(work)) != 0
+    assert b"different operation" in core.moodist_last_error()
+    # an allreduce of another size or with another reduction is a mismatch as well
+    assert core.moodist_pg_allreduce(b, ctypes.byref(fake(16)), None, 0, None, 0.0, ctypes.byref(work)) != 0
+    assert core.moodist_pg_allreduce(b, ctypes.byref(fake(8)), None, 4, None, 0.0, ctypes.byref(work)) != 0
+    # refused before anything is posted: an operation the type does not take, a missing temporary
+    assert core.moodist_pg_allreduce(b, ctypes.byref(fake(8, dtype=3)), None, 1, None, 0.0, ctypes.byref(work)) != 0
+    assert b"Unsupported reduce operation" in core.moodist_last_error()
+    assert core.moodist_pg_allreduce(b, ctypes.byref(fake(7)), None, 0, None, 0.0, ctypes.byref(work)) != 0
+    assert b"needs a scratch tensor of 8 elements" in core.moodist_last_error()
+    core.moodist_world_destroy(w)
+
+
 # ---------------- planner: C++ against the oracle's restatement ----------------
 
 @pytest.mark.parametrize("case", list(_cases()), ids=lambda c: c[0])
