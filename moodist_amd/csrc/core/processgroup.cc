@@ -1021,12 +1021,17 @@ void World::run_allreduce(Collective& c) {
   if (one_launch) {
     const size_t itemsize = dtype_size(c.dtype);
     const float scale = c.reduce_op == MDH_OP_AVG ? 1.0f / (float)size : c.premul;
-    std::vector<const void*> tables(n * (size_t)size * (size_t)size);
-    std::vector<mdh_reduce_job> jobs(n * (size_t)size);
+    // a job per tensor and chunk, handed over in batches of a few thousand (a long list over
+    // many ranks would otherwise need size x size pointers per tensor all at once)
+    constexpr size_t kBatchJobs = 4096;
+    const size_t per_call = n * (size_t)size < kBatchJobs ? n * (size_t)size : kBatchJobs;
+    std::vector<const void*> tables(per_call * (size_t)size);
+    std::vector<mdh_reduce_job> jobs(per_call);
+    void* stream = c.post[0].stream;
     size_t k = 0;
     for (size_t t = 0; t < n; ++t) {
       const size_t bytes = list ? bytes_of(c.post[0].inputs[t]) / (size_t)size : c.bytes;
-      for (int q = 0; q < size; ++q, ++k) {
+      for (int q = 0; q < size; ++q) {
         for (int j = 0; j < size; ++j) {
           const moodist_tensor& in = list ? c.post[(size_t)j].inputs[t] : c.post[(size_t)j].input;
           tables[k * (size_t)size + (size_t)j] = (const char*)in.data + bytes * (size_t)q;
@@ -1036,10 +1041,15 @@ void World::run_allreduce(Collective& c) {
         jobs[k].first = q;
         jobs[k].dst = nullptr;
         jobs[k].numel = bytes / itemsize;
+        if (++k == per_call) {
+          check_mdh(h.allreduce_many(jobs.data(), (int)k, c.dtype, c.reduce_op, scale, stream));
+          k = 0;
+        }
       }
     }
-    void* stream = c.post[0].stream;
-    check_mdh(h.allreduce_many(jobs.data(), (int)jobs.size(), c.dtype, c.reduce_op, scale, stream));
+    if (k > 0) {
+      check_mdh(h.allreduce_many(jobs.data(), (int)k, c.dtype, c.reduce_op, scale, stream));
+    }
     for (const Posting& p : c.post) {
       if (p.has_copy_back) { // through a padded temporary (core/processgroup.cc:1716-1720)
         check_hip(h.MemcpyAsync(p.copy_back.data, p.output.data, (size_t)p.copy_back.numel * (size_t)p.copy_back.itemsize,

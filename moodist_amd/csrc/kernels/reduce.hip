@@ -2,6 +2,8 @@
 // of the pointer table, dispatch on element type.
 #include "reduce_kernels.h"
 
+#include <algorithm>
+#include <utility>
 #include <vector>
 
 namespace mdh {
@@ -283,13 +285,17 @@ int reduce_list(const char* who, const mdh_reduce_job* jobs, int njobs, int dtyp
     if (spread && job.numel != 0) {
       // every source is written: no two of them may share a byte
       const uintptr_t bytes = (uintptr_t)job.numel * info.itemsize;
+      std::pair<uintptr_t, int> by_address[MDH_MAX_SOURCES];
       for (int x = 0; x < job.nsrc; ++x) {
-        for (int y = x + 1; y < job.nsrc; ++y) {
-          const uintptr_t a = (uintptr_t)job.srcs[x], b = (uintptr_t)job.srcs[y];
-          if (a < b + bytes && b < a + bytes) {
-            set_error("%s: sources %d and %d overlap%s", who, x, y, label);
-            return MDH_EINVAL;
-          }
+        by_address[x] = {(uintptr_t)job.srcs[x], x};
+      }
+      std::sort(by_address, by_address + job.nsrc);
+      for (int x = 0; x + 1 < job.nsrc; ++x) {
+        if (by_address[x + 1].first - by_address[x].first < bytes) {
+          const int lo = std::min(by_address[x].second, by_address[x + 1].second);
+          const int hi = std::max(by_address[x].second, by_address[x + 1].second);
+          set_error("%s: sources %d and %d overlap%s", who, lo, hi, label);
+          return MDH_EINVAL;
         }
       }
     }
