@@ -576,7 +576,7 @@ def measure(name, args, torch, abi, dev):
             if prefilled and enqueued > 0.9 * spin_cycles / cycles_per_ms and lengthened < 6:
                 # the host was still enqueuing when the spin ended (a profiler slows the launch
                 # call several times over): this window measured the host; again behind a longer spin
-                spin_cycles = int(spin_cycles * 1.6)
+                spin_cycles = max(int(spin_cycles * 1.6), int(enqueued * 1.3 * cycles_per_ms))
                 lengthened += 1
                 continue
             enqueue_ms.append(enqueued)
