@@ -638,6 +638,32 @@ def test_kernel_less_gather_from_padded_staging_equals_the_kernel_path(world, de
         pg.options().force_kernel_less = False
 
 
+def test_kernel_less_gather_of_rows_far_apart(world, dev):
+    # Rows of 75,002 bytes at a pitch of 3,669,242 bytes: a shape the runtime's 2-D copy has been
+    # seen to refuse when it checks its arguments.  Whether it takes it (one 2-D copy per rank's
+    # output) or not (the run then goes rank by rank), the bytes must be the gather's.
+    width, pitch = 75002, 3669242
+    g = torch.Generator().manual_seed(8)
+    staging = torch.randint(0, 256, (P * pitch,), dtype=torch.uint8, generator=g).to(dev)
+    ins = [staging[r * pitch:r * pitch + width] for r in range(P)]
+    for pg in world:
+        pg.options().force_kernel_less = True
+    try:
+        c = lambda: (world.groups[0]._get_option("kernel_less_copies_1d"), world.groups[0]._get_option("kernel_less_copies_2d"))
+        before = c()
+        outs = [torch.zeros(P * width, dtype=torch.uint8, device=dev) for _ in range(P)]
+        each_rank(world, lambda r, pg: pg._allgather_base(outs[r], ins[r]))
+        after = c()
+        want = torch.cat(ins)
+        for r in range(P):
+            assert torch.equal(outs[r], want), r
+        # per rank's output: one 2-D copy, or eight copies of one row each
+        assert (after[0] - before[0], after[1] - before[1]) in ((0, P), (P * P, 0))
+    finally:
+        for pg in world:
+            pg.options().force_kernel_less = False
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.int64], ids=str)
 def test_reduce_scatter_coalesced_is_one_collective_and_matches_the_oracle(world, dev, dtype):
     # reference wrapper/processgroup_wrapper.cc:159-170 runs one reduce_scatter per tensor; here a
