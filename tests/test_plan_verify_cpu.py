@@ -176,13 +176,13 @@ def test_random_permuted_boxes():
     # sources that are permuted views of padded parents, extents up to 90: transposing pairs with
     # batch dimensions around them, partial tiles, every element size, several boxes per plan
     rng = np.random.RandomState(23)
-    for trial in range(10):
+    for trial in range(150):
         itemsize = int(rng.choice([1, 2, 4, 8, 16]))
         nboxes = int(rng.randint(1, 4))
         boxes, sizes, dst_elems = [], [], 0
         for _ in range(nboxes):
             nd = int(rng.randint(2, 5))
-            shape = [int(rng.choice([1, 2, 3, 17, 33, 64, 90])) for _ in range(nd)]
+            shape = [int(rng.choice([1, 2, 3, 7, 17, 33])) for _ in range(nd)]  # (every element is replayed on the host)
             for d in rng.choice(nd, 2, replace=False):
                 shape[d] = int(rng.choice([16, 31, 64, 70, 90]))
             pshape = [s + int(rng.randint(0, 3)) for s in shape]
