@@ -59,6 +59,8 @@ DTYPE_NAMES = {"float32": "f32", "bfloat16": "bf16", "float16": "f16", "float64"
 ALL_WORKLOADS = ("reduce_fp32_p8", "reduce_bf16_p16", "reduce_fp32_p64_sum", "reduce_fp32_p64_avg", "reduce_fp32_p64_max",
                  "allgather_bf16_p8", "allgather_bf16_p8_strided", "redistribute_fp32_8192", "redistribute_bf16_8192",
                  "redistribute_bf16_3d")
+# measured after them by a default run, reported under "others"
+OTHER_WORKLOADS = ["transpose:4096:4096:4", "transpose:8192:8192:2", "coalesced:1:4194304", "coalesced:48:65536"]
 
 
 def box_kernel(abi):
@@ -447,7 +449,7 @@ def build_workload(name, torch, abi, dev, rotation_bytes):
 
         desc = {"workload": name, "op": "2-D element transpose (mdh_copy_boxes)", "rows": R, "cols": C, "itemsize": isz,
                 "dtype": "uint8", "buffer_sets": nsets}
-        return desc, set_bytes, launch, check, "strided-box kernels"
+        return desc, set_bytes, launch, check, "transpose_kernel (copy_boxes_kernel with the knob box_transpose=1)"
 
     raise SystemExit("bench: unknown workload %r" % name)
 
@@ -707,6 +709,27 @@ def main():
                 "buffer_sets": r["config"]["buffer_sets"], "result_checked": r["result_checked"],
             }
         out["configs"] = configs
+        # what the library serves beyond those configurations: boxes that transpose, and the
+        # allreduce of eight local ranks (one collective, a step is all eight ranks' calls)
+        others = {}
+        for name in OTHER_WORKLOADS:
+            sys.stderr.write("bench: %s (%.0f s so far)\n" % (name, time.perf_counter() - t_start))
+            sys.stderr.flush()
+            a = argparse.Namespace(**vars(args))
+            if name.startswith("coalesced:"):
+                a.steps, a.warmup = min(args.steps, 30), min(args.warmup, 5)
+            try:
+                r = measure(name, a, torch, abi, dev)
+            except (Exception, SystemExit) as e:  # the line above all reports the configurations: it still goes out
+                others[name] = {"error": str(e)}
+                continue
+            rf = r["roofline"]
+            others[name] = {
+                "kernel": rf["kernel"], "kernel_us": rf["kernel_us"], "frac": rf["frac"], "achieved": rf["achieved"],
+                "algorithmic_bytes": rf["algorithmic_bytes_per_launch"], "ms_per_step": r["ms_per_step"],
+                "steps": a.steps, "buffer_sets": r["config"]["buffer_sets"], "result_checked": r["result_checked"],
+            }
+        out["others"] = others
         out["bench_wall_s"] = round(time.perf_counter() - t_start, 1)
     print(json.dumps(out))
 
